@@ -1,0 +1,212 @@
+/*
+ * tilefusion_hip.h -- C ABI of libtilefusion_hip, the MI355X (gfx950) engine behind
+ * the tile-fusion API (include/tile-fusion.h).
+ *
+ * Plain pointers, sizes and opaque handles only.  fp32 values, int32 indices, CSR
+ * sparse matrices, row-major dense matrices -- the reference's conventions.
+ *
+ * Each entry point cites the reference interface it stands in for (paths relative
+ * to the reference checkout).  Names in the comments follow the README API:
+ *     D = A * (B * C)        A sparse;  B sparse (SpMM-SpMM) or dense (GeMM-SpMM);
+ *                            C dense;   the product B*C is "the intermediate" T.
+ *
+ * All functions return 0 on success or a negative tf_status; the text of the last
+ * error on the calling thread is available from tf_last_error_string().
+ */
+#ifndef TILEFUSION_HIP_H
+#define TILEFUSION_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int tf_status;
+enum {
+  TF_OK = 0,
+  TF_EINVAL = -1,       /* bad argument (null pointer, negative size, shape mismatch)      */
+  TF_EHIP = -2,         /* a HIP runtime call failed (no device, launch failure, ...)       */
+  TF_ENOMEM = -3,       /* host or device allocation failed                                 */
+  TF_ESCHEDULE = -4,    /* schedule is invalid or does not belong to these operands         */
+  TF_EUNSUPPORTED = -5  /* shape outside what the kernels take (e.g. N not a multiple of 4) */
+};
+
+/* The reference has no error channel (void executors, exit(1) in its drivers,
+ * fusion/src/Fusion_Utils.cpp:208-211); this is the replacement. */
+const char *tf_last_error_string(void);
+
+/* Library version "major.minor". */
+const char *tf_version(void);
+
+/* ---- device ----------------------------------------------------------------- */
+
+typedef struct {
+  int device;              /* HIP device ordinal in use                           */
+  int compute_units;       /* 256 on MI355X                                       */
+  int xcds;                /* accelerator complex dies sharing an L2 each (8)     */
+  int lds_bytes_per_block; /* max LDS one workgroup may take (163840 on gfx950)   */
+  int wavefront;           /* 64                                                  */
+  int clock_khz;
+  size_t hbm_bytes;
+  char arch[64];           /* "gfx950..."                                         */
+} tf_device_info;
+
+/* Selects the device for the calling thread and reports its properties.  Optional:
+ * every other entry point works on the current HIP device. */
+tf_status tf_device_init(int device, tf_device_info *info);
+tf_status tf_device_synchronize(void);
+
+/* Streams and events are passed as void* so that callers need no HIP headers; a
+ * stream argument of NULL is the default stream.  A hipStream_t obtained elsewhere
+ * (e.g. torch.cuda.current_stream().cuda_stream) can be passed as is. */
+tf_status tf_stream_create(void **stream);
+tf_status tf_stream_destroy(void *stream);
+tf_status tf_stream_synchronize(void *stream);
+tf_status tf_event_create(void **event);
+tf_status tf_event_destroy(void *event);
+tf_status tf_event_record(void *event, void *stream);
+tf_status tf_event_synchronize(void *event);
+tf_status tf_event_elapsed_ms(void *start, void *stop, float *ms);
+
+/* ---- operands ---------------------------------------------------------------- */
+
+/* Device-resident CSR matrix.  Stands in for sym_lib::CSR {m,n,nnz,p,i,x} as the
+ * executors receive it (fusion/src/SpMM_SpMM_vectorized.cpp:876-880: Ap, Ai, Ax). */
+typedef struct tf_csr tf_csr;
+/* Device-resident dense row-major matrix (the reference's bare float* operands). */
+typedef struct tf_dense tf_dense;
+
+/* Copies a host CSR to the device.  Column indices need not be sorted. */
+tf_status tf_csr_upload(int M, int N, const int *Ap, const int *Ai, const float *Ax,
+                        tf_csr **out);
+/* Wraps CSR arrays that already live in device memory; nothing is copied or owned. */
+tf_status tf_csr_wrap_device(int M, int N, int nnz, const int *dAp, const int *dAi,
+                             const float *dAx, tf_csr **out);
+void tf_csr_free(tf_csr *a);
+
+tf_status tf_dense_upload(int M, int N, const float *host, tf_dense **out);
+tf_status tf_dense_alloc(int M, int N, tf_dense **out); /* contents undefined */
+tf_status tf_dense_wrap_device(int M, int N, float *dptr, tf_dense **out);
+tf_status tf_dense_download(const tf_dense *d, float *host);
+tf_status tf_dense_fill(tf_dense *d, float value, void *stream);
+float *tf_dense_device_ptr(const tf_dense *d);
+void tf_dense_free(tf_dense *d);
+
+/* ---- inspector ---------------------------------------------------------------- */
+
+enum { TF_OP_SPMM_SPMM = 0, TF_OP_GEMM_SPMM = 1 };
+
+/* Parameters of the gfx950 schedule.  Zero in any field means "default". */
+typedef struct {
+  int op;                /* TF_OP_SPMM_SPMM or TF_OP_GEMM_SPMM                               */
+  int N;                 /* columns of C and D (reference: bCols / EmbedDim)                 */
+  int K;                 /* GeMM-SpMM: columns of dense B = rows of C (FeatureDim); else 0   */
+  int lds_budget_bytes;  /* LDS one fused tile may take; plays the role of the cache budget
+                            ScheduleParameters::TileM of the reference's variable-tile
+                            inspector.  Default 65536, max 163840.                            */
+  int tile_rows;         /* cap on the rows a tile owns; default: sized so that the launch
+                            has about four tiles per compute unit                             */
+  float max_redundancy;  /* a tile may compute up to this many intermediate rows per owned
+                            row (halo rows recomputed so that boundary rows still fuse);
+                            1.0 disables recomputation = the reference's tiling.
+                            Default 3.0 for SpMM-SpMM, 1.5 for GeMM-SpMM.                    */
+  int long_row_nnz;      /* remainder rows with more stored entries than this are split into
+                            chunks reduced by a wavefront-level tree; default 2048           */
+  int compute_units;     /* sizing hint; default: the current device, or 256 with no device  */
+} tf_inspect_opts;
+
+typedef struct tf_schedule tf_schedule;
+
+/* Builds the fused-tile schedule for D = A*(B*C) from the sparsity pattern of A
+ * (host arrays; A is L x M, the intermediate has M rows).  Pure host work: no GPU is
+ * needed.  Replaces InspectorForTileFusedCSRVariableTileSize::
+ * generateVariableTileSizeScheduleGeMMSpMM (fusion/include/sparse-fusion/
+ * Fusion_Inspector.h:850-1017) and ...ForBothWavefronts (:676-846): same roles
+ * (tiles own contiguous first-op rows; a second-op row is fused into a tile iff all
+ * its column indices lie in the rows the tile computes; everything else goes to an
+ * unfused remainder), re-derived for one workgroup's LDS instead of a CPU cache. */
+tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai, const tf_inspect_opts *opts,
+                     tf_schedule **out);
+void tf_schedule_free(tf_schedule *s);
+
+typedef struct {
+  int op, N, K;
+  int rows;              /* L: rows of A / D                                        */
+  int inter_rows;        /* M: rows of the intermediate                             */
+  int n_tiles;
+  int n_fused_rows;      /* second-op rows served from LDS                          */
+  int n_remainder_rows;  /* second-op rows served from the intermediate in HBM      */
+  int n_long_rows;       /* of those, rows split into chunks                        */
+  int n_long_chunks;
+  int n_producer_rows;   /* sum over tiles of rows computed (>= M with recomputation) */
+  int n_writeback_rows;  /* intermediate rows that are written to HBM               */
+  int max_tile_producer_rows;
+  int lds_bytes;         /* dynamic LDS of the fused-tile kernel                    */
+  long long fused_nnz;   /* stored entries of A in fused rows (getFusedNnzNum)      */
+  long long workspace_bytes; /* device memory the executor keeps (intermediate + partials) */
+} tf_schedule_info;
+
+tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info *info);
+
+/* The schedule in the layout of sym_lib::MultiDimensionalSet
+ * (fusion/include/sparse-fusion/MultiDimensionalSet.h:15-21, as filled at
+ * Fusion_Inspector.h:959-1010): n1 = 2 levels; level 0 = fused tiles, level 1 =
+ * remainder partitions of up to 64 rows (one wavefront's row group);
+ * ptr1[3], ptr2[P+1], ker_begin[2P], id[n_id], type[n_id].  First-op ids of a tile are
+ * the rows it OWNS (each intermediate row is owned by exactly one tile); recomputed
+ * halo rows are not listed there but are given by tile_range.
+ * tile_range[4*t + {0,1,2,3}] = producer_begin, producer_end, own_begin, own_end.
+ * Pointers are views into the schedule, valid until tf_schedule_free. */
+typedef struct {
+  int n1, n_part, n_id, n_tiles;
+  const int *ptr1, *ptr2, *ker_begin, *id, *type;
+  const int *tile_range;
+  const int *writeback; /* [2*n_tiles] begin,end of intermediate rows a tile stores to HBM */
+} tf_schedule_view;
+
+tf_status tf_schedule_get_view(const tf_schedule *s, tf_schedule_view *view);
+
+/* Exact check of a schedule against the pattern it was built from: every first-op
+ * row owned once, every second-op row scheduled once, every fused row's columns
+ * inside its tile's producer range, every remainder row's columns covered by a
+ * write-back range, LDS budget respected.  Returns TF_ESCHEDULE with a message
+ * naming the first violation.  (The reference never checks its schedules.) */
+tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, const int *Ap,
+                               const int *Ai);
+
+/* ---- executors ---------------------------------------------------------------- */
+
+enum {
+  TF_ACCUMULATE = 1u /* D += A*(B*C), the reference's convention (its callers zero D
+                        first); without it D is overwritten and need not be initialised */
+};
+
+/* D = A * (B * C), A and B sparse.  Stands in for
+ * swiftware::sparse::spmmCsrSpmmCsrFusedVectorized2_32SP
+ * (fusion/src/SpMM_SpMM_vectorized.cpp:876-989; the reference names the inner
+ * matrix "A" and the outer one "B", the README and this ABI name them the other way
+ * round).  A is L x M, B is M x Kc, C is Kc x N, D is L x N.  The schedule must come
+ * from tf_inspect on A's pattern with op = TF_OP_SPMM_SPMM and the same N.
+ * Asynchronous on `stream`.  One call at a time per schedule (it owns the workspace). */
+tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_dense *C, tf_dense *D,
+                       tf_schedule *schedule, unsigned flags, void *stream);
+
+/* D = A * (B * C), A sparse, B and C dense.  Stands in for
+ * forwardForOneLayerFusedParallelSeparatedVectorizedSP
+ * (fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:218-291): B is M x K (Features), C is
+ * K x N (Weight, not transposed), D is L x N.  The tile GEMM runs on fp32 MFMA. */
+tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf_dense *D,
+                       tf_schedule *schedule, unsigned flags, void *stream);
+
+/* Unfused building blocks, the reference's in-process baselines:
+ * Y = A * X   (swiftware::sparse::spmmCsrParallel<float>, fusion/src/SpMM_SpMM.cpp:37-55) */
+tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, unsigned flags, void *stream);
+/* Y = X * W   (the cblas_sgemm call at fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:1144) */
+tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TILEFUSION_HIP_H */

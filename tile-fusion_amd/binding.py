@@ -1,0 +1,322 @@
+"""ctypes binding of libtilefusion_hip (declared in include/tilefusion_hip.h).
+
+Mirrors the README API of the reference (README.md:21-38): ``inspector`` builds a
+``FusedSchedule`` from a CSR matrix, ``spmm_spmm`` / ``gemm_spmm`` are the executors.
+There is no fallback: if the shared library is missing, loading raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+OP_SPMM_SPMM = 0
+OP_GEMM_SPMM = 1
+ACCUMULATE = 1
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def lib_path():
+    return os.path.join(_HERE, "lib", "libtilefusion_hip.so")
+
+
+class TileFusionError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"tilefusion status {status}: {message}")
+        self.status = status
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [("device", C.c_int), ("compute_units", C.c_int), ("xcds", C.c_int),
+                ("lds_bytes_per_block", C.c_int), ("wavefront", C.c_int), ("clock_khz", C.c_int),
+                ("hbm_bytes", C.c_size_t), ("arch", C.c_char * 64)]
+
+
+class InspectOpts(C.Structure):
+    _fields_ = [("op", C.c_int), ("N", C.c_int), ("K", C.c_int), ("lds_budget_bytes", C.c_int),
+                ("tile_rows", C.c_int), ("max_redundancy", C.c_float), ("long_row_nnz", C.c_int),
+                ("compute_units", C.c_int)]
+
+
+class ScheduleInfo(C.Structure):
+    _fields_ = [("op", C.c_int), ("N", C.c_int), ("K", C.c_int), ("rows", C.c_int),
+                ("inter_rows", C.c_int), ("n_tiles", C.c_int), ("n_fused_rows", C.c_int),
+                ("n_remainder_rows", C.c_int), ("n_long_rows", C.c_int), ("n_long_chunks", C.c_int),
+                ("n_producer_rows", C.c_int), ("n_writeback_rows", C.c_int),
+                ("max_tile_producer_rows", C.c_int), ("lds_bytes", C.c_int),
+                ("fused_nnz", C.c_longlong), ("workspace_bytes", C.c_longlong)]
+
+
+class ScheduleView(C.Structure):
+    _fields_ = [("n1", C.c_int), ("n_part", C.c_int), ("n_id", C.c_int), ("n_tiles", C.c_int),
+                ("ptr1", C.POINTER(C.c_int)), ("ptr2", C.POINTER(C.c_int)),
+                ("ker_begin", C.POINTER(C.c_int)), ("id", C.POINTER(C.c_int)),
+                ("type", C.POINTER(C.c_int)), ("tile_range", C.POINTER(C.c_int)),
+                ("writeback", C.POINTER(C.c_int))]
+
+
+_PI = C.POINTER(C.c_int)
+_PF = C.POINTER(C.c_float)
+_VP = C.c_void_p
+
+# name -> (restype, argtypes); every symbol include/tilefusion_hip.h declares
+SIGNATURES = {
+    "tf_last_error_string": (C.c_char_p, []),
+    "tf_version": (C.c_char_p, []),
+    "tf_device_init": (C.c_int, [C.c_int, C.POINTER(DeviceInfo)]),
+    "tf_device_synchronize": (C.c_int, []),
+    "tf_stream_create": (C.c_int, [C.POINTER(_VP)]),
+    "tf_stream_destroy": (C.c_int, [_VP]),
+    "tf_stream_synchronize": (C.c_int, [_VP]),
+    "tf_event_create": (C.c_int, [C.POINTER(_VP)]),
+    "tf_event_destroy": (C.c_int, [_VP]),
+    "tf_event_record": (C.c_int, [_VP, _VP]),
+    "tf_event_synchronize": (C.c_int, [_VP]),
+    "tf_event_elapsed_ms": (C.c_int, [_VP, _VP, _PF]),
+    "tf_csr_upload": (C.c_int, [C.c_int, C.c_int, _PI, _PI, _PF, C.POINTER(_VP)]),
+    "tf_csr_wrap_device": (C.c_int, [C.c_int, C.c_int, C.c_int, _VP, _VP, _VP, C.POINTER(_VP)]),
+    "tf_csr_free": (None, [_VP]),
+    "tf_dense_upload": (C.c_int, [C.c_int, C.c_int, _PF, C.POINTER(_VP)]),
+    "tf_dense_alloc": (C.c_int, [C.c_int, C.c_int, C.POINTER(_VP)]),
+    "tf_dense_wrap_device": (C.c_int, [C.c_int, C.c_int, _VP, C.POINTER(_VP)]),
+    "tf_dense_download": (C.c_int, [_VP, _PF]),
+    "tf_dense_fill": (C.c_int, [_VP, C.c_float, _VP]),
+    "tf_dense_device_ptr": (_VP, [_VP]),
+    "tf_dense_free": (None, [_VP]),
+    "tf_inspect": (C.c_int, [C.c_int, C.c_int, _PI, _PI, C.POINTER(InspectOpts), C.POINTER(_VP)]),
+    "tf_schedule_free": (None, [_VP]),
+    "tf_schedule_get_info": (C.c_int, [_VP, C.POINTER(ScheduleInfo)]),
+    "tf_schedule_get_view": (C.c_int, [_VP, C.POINTER(ScheduleView)]),
+    "tf_schedule_validate": (C.c_int, [_VP, C.c_int, C.c_int, _PI, _PI]),
+    "tf_spmm_spmm": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
+    "tf_gemm_spmm": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
+    "tf_spmm": (C.c_int, [_VP, _VP, _VP, C.c_uint, _VP]),
+    "tf_gemm": (C.c_int, [_VP, _VP, _VP, _VP]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built (no CPU fallback exists)."""
+    global _lib
+    if _lib is None:
+        path = lib_path()
+        if not os.path.exists(path):
+            raise ImportError(f"{path} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'`")
+        handle = C.CDLL(path)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def _check(status):
+    if status != 0:
+        raise TileFusionError(status, lib().tf_last_error_string().decode())
+
+
+def _i32(a):
+    a = np.ascontiguousarray(a, dtype=np.int32)
+    return a, a.ctypes.data_as(_PI)
+
+
+def _f32(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a, a.ctypes.data_as(_PF)
+
+
+def device_init(device=0):
+    info = DeviceInfo()
+    _check(lib().tf_device_init(device, C.byref(info)))
+    return {f: (getattr(info, f).decode() if f == "arch" else getattr(info, f)) for f, _ in DeviceInfo._fields_}
+
+
+def device_synchronize():
+    _check(lib().tf_device_synchronize())
+
+
+class Stream:
+    def __init__(self):
+        self.h = _VP()
+        _check(lib().tf_stream_create(C.byref(self.h)))
+
+    def synchronize(self):
+        _check(lib().tf_stream_synchronize(self.h))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().tf_stream_destroy(self.h)
+            self.h = None
+
+
+class Event:
+    def __init__(self):
+        self.h = _VP()
+        _check(lib().tf_event_create(C.byref(self.h)))
+
+    def record(self, stream=None):
+        _check(lib().tf_event_record(self.h, stream.h if stream else None))
+
+    def synchronize(self):
+        _check(lib().tf_event_synchronize(self.h))
+
+    def elapsed_ms(self, stop):
+        ms = C.c_float()
+        _check(lib().tf_event_elapsed_ms(self.h, stop.h, C.byref(ms)))
+        return ms.value
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().tf_event_destroy(self.h)
+            self.h = None
+
+
+class CsrMatrix:
+    """swiftware::def::CSRMatrix(M, N, Ap, Ai, Ax) (README.md:35): host views, plus a
+    device-resident copy made by ``to_device``."""
+
+    def __init__(self, M, N, Ap, Ai, Ax):
+        self.M, self.N = int(M), int(N)
+        self.Ap, self._pp = _i32(Ap)
+        self.Ai, self._pi = _i32(Ai)
+        self.Ax, self._px = _f32(Ax)
+        self.h = None
+
+    @classmethod
+    def from_scipy(cls, m):
+        m = m.tocsr()
+        return cls(m.shape[0], m.shape[1], m.indptr, m.indices, m.data)
+
+    @property
+    def nnz(self):
+        return int(self.Ap[-1])
+
+    def to_device(self):
+        if self.h is None:
+            h = _VP()
+            _check(lib().tf_csr_upload(self.M, self.N, self._pp, self._pi, self._px, C.byref(h)))
+            self.h = h
+        return self
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().tf_csr_free(self.h)
+            self.h = None
+
+
+class DenseMatrix:
+    """swiftware::def::Matrix(M, N, Data) (README.md:36) with a device-resident buffer."""
+
+    def __init__(self, M, N, data=None):
+        self.M, self.N = int(M), int(N)
+        self.h = _VP()
+        if data is None:
+            _check(lib().tf_dense_alloc(self.M, self.N, C.byref(self.h)))
+        else:
+            a, p = _f32(data)
+            if a.size != self.M * self.N:
+                raise ValueError("data size does not match M x N")
+            _check(lib().tf_dense_upload(self.M, self.N, p, C.byref(self.h)))
+
+    @classmethod
+    def from_numpy(cls, a):
+        a = np.asarray(a)
+        return cls(a.shape[0], a.shape[1], a)
+
+    @classmethod
+    def wrap_device(cls, M, N, device_ptr):
+        self = cls.__new__(cls)
+        self.M, self.N = int(M), int(N)
+        self.h = _VP()
+        _check(lib().tf_dense_wrap_device(self.M, self.N, _VP(device_ptr), C.byref(self.h)))
+        return self
+
+    def fill(self, value, stream=None):
+        _check(lib().tf_dense_fill(self.h, float(value), stream.h if stream else None))
+
+    def device_ptr(self):
+        return lib().tf_dense_device_ptr(self.h)
+
+    def to_numpy(self):
+        out = np.empty((self.M, self.N), dtype=np.float32)
+        _check(lib().tf_dense_download(self.h, out.ctypes.data_as(_PF)))
+        return out
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().tf_dense_free(self.h)
+            self.h = None
+
+
+class FusedSchedule:
+    """swiftware::def::FusedSchedule: owns the schedule; exposes the reference's flat
+    arrays (n1_, ptr1_, ptr2_, ker_begin_, id_, type_) plus the tile ranges."""
+
+    def __init__(self, handle, A):
+        self.h = handle
+        self._A = A
+
+    def info(self):
+        s = ScheduleInfo()
+        _check(lib().tf_schedule_get_info(self.h, C.byref(s)))
+        return {f: getattr(s, f) for f, _ in ScheduleInfo._fields_}
+
+    def view(self):
+        v = ScheduleView()
+        _check(lib().tf_schedule_get_view(self.h, C.byref(v)))
+        P, nid, nt = v.n_part, v.n_id, v.n_tiles
+
+        def arr(p, n):
+            return np.ctypeslib.as_array(p, shape=(n,)).copy() if n > 0 else np.zeros(0, np.int32)
+        return {"n1_": v.n1, "ptr1_": arr(v.ptr1, 3), "ptr2_": arr(v.ptr2, P + 1),
+                "ker_begin_": arr(v.ker_begin, 2 * P), "id_": arr(v.id, nid), "type_": arr(v.type, nid),
+                "tile_range": arr(v.tile_range, 4 * nt).reshape(nt, 4),
+                "writeback": arr(v.writeback, 2 * nt).reshape(nt, 2)}
+
+    def validate(self, A=None):
+        A = A or self._A
+        _check(lib().tf_schedule_validate(self.h, A.M, A.N, A._pp, A._pi))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().tf_schedule_free(self.h)
+            self.h = None
+
+
+def inspector(A, NumThreads=1, *, op, N, K=0, lds_budget_bytes=0, tile_rows=0, max_redundancy=0.0,
+              long_row_nnz=0, compute_units=0):
+    """swiftware::fusion::inspector(A, NumThreads) (README.md:25).  NumThreads is accepted
+    for signature parity and unused: the schedule is sized by the GPU, not by a CPU
+    thread count.  The extra keywords are the parameters the reference passes to its
+    inspector classes out of band (bCols, embed dim, cache budget)."""
+    del NumThreads
+    o = InspectOpts(op, N, K, lds_budget_bytes, tile_rows, max_redundancy, long_row_nnz, compute_units)
+    h = _VP()
+    _check(lib().tf_inspect(A.M, A.N, A._pp, A._pi, C.byref(o), C.byref(h)))
+    return FusedSchedule(h, A)
+
+
+def spmm_spmm(A, B, Cm, D, schedule, NumThreads=1, *, accumulate=False, stream=None):
+    """spMMSpMMExecutor(A, B, C, D, schedule, NumThreads) (README.md:30): D = A*(B*C)."""
+    del NumThreads
+    _check(lib().tf_spmm_spmm(A.to_device().h, B.to_device().h, Cm.h, D.h, schedule.h,
+                              ACCUMULATE if accumulate else 0, stream.h if stream else None))
+
+
+def gemm_spmm(A, B, Cm, D, schedule, NumThreads=1, *, accumulate=False, stream=None):
+    """geMMSpMMExecutor(A, B, C, D, schedule, NumThreads) (README.md:31): D = A*(B*C)."""
+    del NumThreads
+    _check(lib().tf_gemm_spmm(A.to_device().h, B.h, Cm.h, D.h, schedule.h,
+                              ACCUMULATE if accumulate else 0, stream.h if stream else None))
+
+
+def spmm(A, X, Y, *, accumulate=False, stream=None):
+    _check(lib().tf_spmm(A.to_device().h, X.h, Y.h, ACCUMULATE if accumulate else 0,
+                         stream.h if stream else None))
+
+
+def gemm(X, W, Y, *, stream=None):
+    _check(lib().tf_gemm(X.h, W.h, Y.h, stream.h if stream else None))

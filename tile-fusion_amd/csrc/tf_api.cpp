@@ -1,0 +1,406 @@
+// C ABI of libtilefusion_hip: error channel, device objects, executors.
+// Compiled by hipcc together with tf_inspector.cpp and tf_kernels.hip.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+
+#include "tf_internal.h"
+
+// ---- handles ---------------------------------------------------------------------
+
+struct tf_csr {
+  int M = 0, N = 0, nnz = 0;
+  int *p = nullptr, *i = nullptr;
+  float *x = nullptr;
+  bool owns = false;
+};
+
+struct tf_dense {
+  int M = 0, N = 0;
+  float *d = nullptr;
+  bool owns = false;
+};
+
+namespace tf {
+
+struct DeviceSchedule {
+  int device = -1;
+  TileDesc *tiles = nullptr;
+  int *fused_ids = nullptr;
+  int *rem_rows = nullptr;
+  LongChunk *long_chunks = nullptr;
+  LongRow *long_rows = nullptr;
+  float *inter = nullptr;    // M x N intermediate, only if some tile writes back
+  float *partial = nullptr;  // n_long_chunks x N
+};
+
+// launchers in tf_kernels.hip
+hipError_t launch_fused_spmm_spmm(const TileDesc *, int, const int *, const int *, const int *,
+                                  const float *, const float *, const int *, const int *,
+                                  const float *, float *, float *, int, int, int, hipStream_t);
+hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
+                            float *, int, int, hipStream_t);
+hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const int *, const float *,
+                            const float *, float *, float *, int, int, hipStream_t);
+hipError_t launch_fused_gemm_spmm(const TileDesc *, int, const int *, const float *, const float *,
+                                  int, int, const int *, const int *, const float *, float *,
+                                  float *, int, int, int, hipStream_t);
+hipError_t launch_gemm(const float *, const float *, float *, int, int, int, int, hipStream_t);
+hipError_t launch_fill(float *, size_t, float, hipStream_t);
+
+static thread_local char g_err[512] = "";
+
+tf_status fail(tf_status code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static tf_status hip_fail(hipError_t e, const char *what) {
+  return fail(e == hipErrorOutOfMemory ? TF_ENOMEM : TF_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define TF_HIP(call)                                         \
+  do {                                                       \
+    hipError_t e_ = (call);                                  \
+    if (e_ != hipSuccess) return tf::hip_fail(e_, #call);    \
+  } while (0)
+
+int default_compute_units() {
+  int dev = 0, cu = 0;
+  if (hipGetDevice(&dev) == hipSuccess &&
+      hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cu > 0)
+    return cu;
+  (void)hipGetLastError();
+  return 256;
+}
+
+void release_device_schedule(DeviceSchedule *d) {
+  if (!d) return;
+  (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->rem_rows);
+  (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows);
+  (void)hipFree(d->inter); (void)hipFree(d->partial);
+  delete d;
+}
+
+template <class T> static tf_status upload_vec(const std::vector<T> &v, T **out) {
+  *out = nullptr;
+  if (v.empty()) return TF_OK;
+  TF_HIP(hipMalloc(reinterpret_cast<void **>(out), v.size() * sizeof(T)));
+  TF_HIP(hipMemcpy(*out, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice));
+  return TF_OK;
+}
+
+// Device copies of the schedule arrays and the workspace, made on first use.
+static tf_status ensure_device(tf_schedule *s) {
+  static std::mutex mu;
+  std::lock_guard<std::mutex> lock(mu);
+  int dev = 0;
+  TF_HIP(hipGetDevice(&dev));
+  if (s->dev) {
+    if (s->dev->device != dev)
+      return fail(TF_ESCHEDULE, "schedule was uploaded to device %d, current device is %d", s->dev->device, dev);
+    return TF_OK;
+  }
+  auto *d = new (std::nothrow) DeviceSchedule();
+  if (!d) return fail(TF_ENOMEM, "out of host memory");
+  d->device = dev;
+  tf_status rc = upload_vec(s->tiles, &d->tiles);
+  if (!rc) rc = upload_vec(s->fused_ids, &d->fused_ids);
+  if (!rc) rc = upload_vec(s->rem_rows, &d->rem_rows);
+  if (!rc) rc = upload_vec(s->long_chunks, &d->long_chunks);
+  if (!rc) rc = upload_vec(s->long_rows, &d->long_rows);
+  if (!rc && s->n_writeback_rows > 0) {
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->inter), (size_t)s->M * s->opts.N * sizeof(float));
+    if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(intermediate)");
+  }
+  if (!rc && !s->long_chunks.empty()) {
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->partial), s->long_chunks.size() * (size_t)s->opts.N * sizeof(float));
+    if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(partials)");
+  }
+  if (rc) { release_device_schedule(d); return rc; }
+  s->dev = d;
+  return TF_OK;
+}
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Second-op rows that no tile fused: served from the intermediate in HBM.
+static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int accumulate, hipStream_t st) {
+  const DeviceSchedule *d = s->dev;
+  const int N = s->opts.N;
+  if (!s->rem_rows.empty()) {
+    const bool all = (int)s->rem_rows.size() == s->L;  // identity list: no indirection needed
+    TF_HIP(launch_spmm_rows(all ? nullptr : d->rem_rows, (int)s->rem_rows.size(), A->p, A->i, A->x,
+                            d->inter, D->d, N, accumulate, st));
+  }
+  if (!s->long_chunks.empty())
+    TF_HIP(launch_long_rows(d->long_chunks, (int)s->long_chunks.size(), d->long_rows,
+                            (int)s->long_rows.size(), A->i, A->x, d->inter, d->partial, D->d, N,
+                            accumulate, st));
+  return TF_OK;
+}
+
+}  // namespace tf
+
+using tf::fail;
+
+// ---- errors, device, streams -----------------------------------------------------
+
+extern "C" const char *tf_last_error_string(void) { return tf::g_err; }
+extern "C" const char *tf_version(void) { return "0.1"; }
+
+extern "C" tf_status tf_device_init(int device, tf_device_info *info) {
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= 0) {
+    (void)hipGetLastError();
+    return fail(TF_EHIP, "no HIP device available (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+  }
+  if (device < 0 || device >= count) return fail(TF_EINVAL, "device %d out of range (have %d)", device, count);
+  TF_HIP(hipSetDevice(device));
+  if (info) {
+    hipDeviceProp_t p;
+    TF_HIP(hipGetDeviceProperties(&p, device));
+    std::memset(info, 0, sizeof(*info));
+    info->device = device;
+    info->compute_units = p.multiProcessorCount;
+    info->xcds = 8;
+    info->lds_bytes_per_block = (int)p.sharedMemPerBlock;
+    int optin = 0;
+    if (hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, device) == hipSuccess && optin > info->lds_bytes_per_block)
+      info->lds_bytes_per_block = optin;
+    (void)hipGetLastError();
+    info->wavefront = p.warpSize;
+    info->clock_khz = p.clockRate;
+    info->hbm_bytes = p.totalGlobalMem;
+    std::snprintf(info->arch, sizeof(info->arch), "%s", p.gcnArchName);
+  }
+  return TF_OK;
+}
+
+extern "C" tf_status tf_device_synchronize(void) {
+  TF_HIP(hipDeviceSynchronize());
+  return TF_OK;
+}
+
+extern "C" tf_status tf_stream_create(void **stream) {
+  if (!stream) return fail(TF_EINVAL, "tf_stream_create: null");
+  hipStream_t s;
+  TF_HIP(hipStreamCreate(&s));
+  *stream = s;
+  return TF_OK;
+}
+extern "C" tf_status tf_stream_destroy(void *stream) {
+  if (stream) TF_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return TF_OK;
+}
+extern "C" tf_status tf_stream_synchronize(void *stream) {
+  TF_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return TF_OK;
+}
+extern "C" tf_status tf_event_create(void **event) {
+  if (!event) return fail(TF_EINVAL, "tf_event_create: null");
+  hipEvent_t e;
+  TF_HIP(hipEventCreate(&e));
+  *event = e;
+  return TF_OK;
+}
+extern "C" tf_status tf_event_destroy(void *event) {
+  if (event) TF_HIP(hipEventDestroy(static_cast<hipEvent_t>(event)));
+  return TF_OK;
+}
+extern "C" tf_status tf_event_record(void *event, void *stream) {
+  TF_HIP(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+  return TF_OK;
+}
+extern "C" tf_status tf_event_synchronize(void *event) {
+  TF_HIP(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+  return TF_OK;
+}
+extern "C" tf_status tf_event_elapsed_ms(void *start, void *stop, float *ms) {
+  if (!ms) return fail(TF_EINVAL, "tf_event_elapsed_ms: null");
+  TF_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return TF_OK;
+}
+
+// ---- operands ----------------------------------------------------------------------
+
+extern "C" tf_status tf_csr_upload(int M, int N, const int *Ap, const int *Ai, const float *Ax,
+                                   tf_csr **out) {
+  if (!out) return fail(TF_EINVAL, "tf_csr_upload: out is null");
+  *out = nullptr;
+  if (M <= 0 || N <= 0 || !Ap) return fail(TF_EINVAL, "tf_csr_upload: bad M/N/Ap");
+  if (Ap[0] != 0) return fail(TF_EINVAL, "tf_csr_upload: Ap[0] != 0");
+  for (int r = 0; r < M; ++r)
+    if (Ap[r + 1] < Ap[r]) return fail(TF_EINVAL, "tf_csr_upload: Ap not monotone at row %d", r);
+  const int nnz = Ap[M];
+  if (nnz > 0 && (!Ai || !Ax)) return fail(TF_EINVAL, "tf_csr_upload: Ai/Ax null");
+  for (int k = 0; k < nnz; ++k)
+    if (Ai[k] < 0 || Ai[k] >= N) return fail(TF_EINVAL, "tf_csr_upload: column %d out of range at entry %d", Ai[k], k);
+  auto *a = new (std::nothrow) tf_csr();
+  if (!a) return fail(TF_ENOMEM, "out of host memory");
+  a->M = M; a->N = N; a->nnz = nnz; a->owns = true;
+  hipError_t e = hipMalloc(reinterpret_cast<void **>(&a->p), (size_t)(M + 1) * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&a->i), (size_t)std::max(nnz, 1) * sizeof(int));
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&a->x), (size_t)std::max(nnz, 1) * sizeof(float));
+  if (e == hipSuccess) e = hipMemcpy(a->p, Ap, (size_t)(M + 1) * sizeof(int), hipMemcpyHostToDevice);
+  if (e == hipSuccess && nnz > 0) e = hipMemcpy(a->i, Ai, (size_t)nnz * sizeof(int), hipMemcpyHostToDevice);
+  if (e == hipSuccess && nnz > 0) e = hipMemcpy(a->x, Ax, (size_t)nnz * sizeof(float), hipMemcpyHostToDevice);
+  if (e != hipSuccess) { tf_csr_free(a); return tf::hip_fail(e, "tf_csr_upload"); }
+  *out = a;
+  return TF_OK;
+}
+
+extern "C" tf_status tf_csr_wrap_device(int M, int N, int nnz, const int *dAp, const int *dAi,
+                                        const float *dAx, tf_csr **out) {
+  if (!out) return fail(TF_EINVAL, "tf_csr_wrap_device: out is null");
+  *out = nullptr;
+  if (M <= 0 || N <= 0 || nnz < 0 || !dAp || (nnz > 0 && (!dAi || !dAx)))
+    return fail(TF_EINVAL, "tf_csr_wrap_device: bad argument");
+  auto *a = new (std::nothrow) tf_csr();
+  if (!a) return fail(TF_ENOMEM, "out of host memory");
+  a->M = M; a->N = N; a->nnz = nnz; a->owns = false;
+  a->p = const_cast<int *>(dAp); a->i = const_cast<int *>(dAi); a->x = const_cast<float *>(dAx);
+  *out = a;
+  return TF_OK;
+}
+
+extern "C" void tf_csr_free(tf_csr *a) {
+  if (!a) return;
+  if (a->owns) { (void)hipFree(a->p); (void)hipFree(a->i); (void)hipFree(a->x); }
+  delete a;
+}
+
+extern "C" tf_status tf_dense_alloc(int M, int N, tf_dense **out) {
+  if (!out) return fail(TF_EINVAL, "tf_dense_alloc: out is null");
+  *out = nullptr;
+  if (M <= 0 || N <= 0) return fail(TF_EINVAL, "tf_dense_alloc: bad shape %d x %d", M, N);
+  auto *d = new (std::nothrow) tf_dense();
+  if (!d) return fail(TF_ENOMEM, "out of host memory");
+  d->M = M; d->N = N; d->owns = true;
+  hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->d), (size_t)M * N * sizeof(float));
+  if (e != hipSuccess) { delete d; return tf::hip_fail(e, "tf_dense_alloc"); }
+  *out = d;
+  return TF_OK;
+}
+
+extern "C" tf_status tf_dense_upload(int M, int N, const float *host, tf_dense **out) {
+  if (!host) return fail(TF_EINVAL, "tf_dense_upload: host is null");
+  tf_status rc = tf_dense_alloc(M, N, out);
+  if (rc) return rc;
+  hipError_t e = hipMemcpy((*out)->d, host, (size_t)M * N * sizeof(float), hipMemcpyHostToDevice);
+  if (e != hipSuccess) { tf_dense_free(*out); *out = nullptr; return tf::hip_fail(e, "tf_dense_upload"); }
+  return TF_OK;
+}
+
+extern "C" tf_status tf_dense_wrap_device(int M, int N, float *dptr, tf_dense **out) {
+  if (!out) return fail(TF_EINVAL, "tf_dense_wrap_device: out is null");
+  *out = nullptr;
+  if (M <= 0 || N <= 0 || !dptr) return fail(TF_EINVAL, "tf_dense_wrap_device: bad argument");
+  if (!tf::aligned16(dptr)) return fail(TF_EINVAL, "tf_dense_wrap_device: pointer must be 16-byte aligned");
+  auto *d = new (std::nothrow) tf_dense();
+  if (!d) return fail(TF_ENOMEM, "out of host memory");
+  d->M = M; d->N = N; d->d = dptr; d->owns = false;
+  *out = d;
+  return TF_OK;
+}
+
+extern "C" tf_status tf_dense_download(const tf_dense *d, float *host) {
+  if (!d || !host) return fail(TF_EINVAL, "tf_dense_download: null argument");
+  TF_HIP(hipMemcpy(host, d->d, (size_t)d->M * d->N * sizeof(float), hipMemcpyDeviceToHost));
+  return TF_OK;
+}
+
+extern "C" tf_status tf_dense_fill(tf_dense *d, float value, void *stream) {
+  if (!d) return fail(TF_EINVAL, "tf_dense_fill: null argument");
+  TF_HIP(tf::launch_fill(d->d, (size_t)d->M * d->N, value, static_cast<hipStream_t>(stream)));
+  return TF_OK;
+}
+
+extern "C" float *tf_dense_device_ptr(const tf_dense *d) { return d ? d->d : nullptr; }
+
+extern "C" void tf_dense_free(tf_dense *d) {
+  if (!d) return;
+  if (d->owns) (void)hipFree(d->d);
+  delete d;
+}
+
+// ---- executors -----------------------------------------------------------------------
+
+static tf_status check_common(const char *who, const tf_csr *A, const tf_dense *C, const tf_dense *D,
+                              const tf_schedule *s, int op) {
+  if (!A || !C || !D || !s) return fail(TF_EINVAL, "%s: null argument", who);
+  if (s->opts.op != op) return fail(TF_ESCHEDULE, "%s: schedule was built for the other operation", who);
+  if (A->M != s->L || A->N != s->M || A->nnz != s->nnz)
+    return fail(TF_ESCHEDULE, "%s: schedule was built for a %d x %d pattern with %lld entries, A is %d x %d with %d",
+                who, s->L, s->M, s->nnz, A->M, A->N, A->nnz);
+  if (C->N != s->opts.N || D->N != s->opts.N)
+    return fail(TF_ESCHEDULE, "%s: schedule was built for N = %d, C has %d and D has %d columns", who, s->opts.N, C->N, D->N);
+  if (D->M != A->M) return fail(TF_EINVAL, "%s: D has %d rows, A has %d", who, D->M, A->M);
+  return TF_OK;
+}
+
+extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_dense *C, tf_dense *D,
+                                  tf_schedule *s, unsigned flags, void *stream) {
+  tf_status rc = check_common("tf_spmm_spmm", A, C, D, s, TF_OP_SPMM_SPMM);
+  if (rc) return rc;
+  if (!B) return fail(TF_EINVAL, "tf_spmm_spmm: B is null");
+  if (B->M != A->N) return fail(TF_EINVAL, "tf_spmm_spmm: B has %d rows, A has %d columns", B->M, A->N);
+  if (C->M != B->N) return fail(TF_EINVAL, "tf_spmm_spmm: C has %d rows, B has %d columns", C->M, B->N);
+  rc = tf::ensure_device(s);
+  if (rc) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
+  const tf::DeviceSchedule *d = s->dev;
+  TF_HIP(tf::launch_fused_spmm_spmm(d->tiles, (int)s->tiles.size(), d->fused_ids, B->p, B->i, B->x,
+                                    C->d, A->p, A->i, A->x, D->d, d->inter, s->opts.N,
+                                    s->lds_bytes, acc, st));
+  return tf::run_remainder(A, D, s, acc, st);
+}
+
+extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf_dense *D,
+                                  tf_schedule *s, unsigned flags, void *stream) {
+  tf_status rc = check_common("tf_gemm_spmm", A, C, D, s, TF_OP_GEMM_SPMM);
+  if (rc) return rc;
+  if (!B) return fail(TF_EINVAL, "tf_gemm_spmm: B is null");
+  if (B->M != A->N) return fail(TF_EINVAL, "tf_gemm_spmm: B has %d rows, A has %d columns", B->M, A->N);
+  if (B->N != s->opts.K || C->M != s->opts.K)
+    return fail(TF_ESCHEDULE, "tf_gemm_spmm: schedule was built for K = %d, B has %d columns and C has %d rows", s->opts.K, B->N, C->M);
+  rc = tf::ensure_device(s);
+  if (rc) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
+  const tf::DeviceSchedule *d = s->dev;
+  TF_HIP(tf::launch_fused_gemm_spmm(d->tiles, (int)s->tiles.size(), d->fused_ids, B->d, C->d,
+                                    s->opts.K, s->gemm_kc, A->p, A->i, A->x, D->d, d->inter,
+                                    s->opts.N, s->lds_bytes, acc, st));
+  return tf::run_remainder(A, D, s, acc, st);
+}
+
+extern "C" tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, unsigned flags, void *stream) {
+  if (!A || !X || !Y) return fail(TF_EINVAL, "tf_spmm: null argument");
+  if (X->M != A->N || Y->M != A->M || X->N != Y->N)
+    return fail(TF_EINVAL, "tf_spmm: shapes A %d x %d, X %d x %d, Y %d x %d", A->M, A->N, X->M, X->N, Y->M, Y->N);
+  TF_HIP(tf::launch_spmm_rows(nullptr, A->M, A->p, A->i, A->x, X->d, Y->d, X->N,
+                              (flags & TF_ACCUMULATE) ? 1 : 0, static_cast<hipStream_t>(stream)));
+  return TF_OK;
+}
+
+extern "C" tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, void *stream) {
+  if (!X || !W || !Y) return fail(TF_EINVAL, "tf_gemm: null argument");
+  if (X->N != W->M || Y->M != X->M || Y->N != W->N)
+    return fail(TF_EINVAL, "tf_gemm: shapes X %d x %d, W %d x %d, Y %d x %d", X->M, X->N, W->M, W->N, Y->M, Y->N);
+  const int K = X->N, N = W->N;
+  if (K % 8 != 0 || N % 32 != 0 || N > 256)
+    return fail(TF_EUNSUPPORTED, "tf_gemm: needs K %% 8 == 0, N %% 32 == 0, N <= 256 (K=%d N=%d)", K, N);
+  const int kc = std::min(K, std::max(8, (32768 / (4 * N)) / 8 * 8));
+  TF_HIP(tf::launch_gemm(X->d, W->d, Y->d, X->M, K, N, kc, static_cast<hipStream_t>(stream)));
+  return TF_OK;
+}

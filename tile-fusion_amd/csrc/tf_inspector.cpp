@@ -1,0 +1,323 @@
+// Host-side inspector of libtilefusion_hip: builds the gfx950 fused-tile schedule
+// from the sparsity pattern of A, and checks schedules exactly.
+//
+// Roles follow the reference's variable-tile inspector
+// (fusion/include/sparse-fusion/Fusion_Inspector.h:850-1017 and :676-846): tiles own
+// contiguous first-op rows, a second-op row is fused into its tile iff every column
+// it reads is produced inside the tile, the rest is an unfused remainder.  What is
+// different is the machine model: a tile is one workgroup whose intermediate slab
+// must fit an LDS budget, tiles may recompute a few halo rows of the intermediate
+// so that boundary rows still fuse, and the remainder is cut into wavefront-sized
+// row groups plus chunks of very long rows.
+#include <algorithm>
+#include <climits>
+#include <cstdio>
+#include <cstring>
+
+#include "tf_internal.h"
+
+namespace {
+
+constexpr int kMaxLds = 163840;  // LDS per workgroup on gfx950
+
+int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+}  // namespace
+
+extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
+                                const tf_inspect_opts *user, tf_schedule **out) {
+  if (!out) return tf::fail(TF_EINVAL, "tf_inspect: out is null");
+  *out = nullptr;
+  if (L <= 0 || M <= 0 || !Ap || !user) return tf::fail(TF_EINVAL, "tf_inspect: bad L/M/Ap/opts");
+  if (Ap[0] != 0) return tf::fail(TF_EINVAL, "tf_inspect: Ap[0] != 0");
+  for (int i = 0; i < L; ++i)
+    if (Ap[i + 1] < Ap[i]) return tf::fail(TF_EINVAL, "tf_inspect: Ap not monotone at row %d", i);
+  const long long nnz = Ap[L];
+  if (nnz > 0 && !Ai) return tf::fail(TF_EINVAL, "tf_inspect: Ai is null");
+
+  tf_inspect_opts o = *user;
+  if (o.op != TF_OP_SPMM_SPMM && o.op != TF_OP_GEMM_SPMM)
+    return tf::fail(TF_EINVAL, "tf_inspect: unknown op %d", o.op);
+  if (o.N <= 0) return tf::fail(TF_EINVAL, "tf_inspect: N must be positive");
+  if ((long long)std::max(L, M) * o.N > INT_MAX)
+    return tf::fail(TF_EUNSUPPORTED, "tf_inspect: rows*N exceeds int32 indexing");
+  if (o.op == TF_OP_GEMM_SPMM) {
+    if (o.K <= 0) return tf::fail(TF_EINVAL, "tf_inspect: GeMM-SpMM needs K > 0");
+    if (o.K % 8 != 0 || o.N % 32 != 0)
+      return tf::fail(TF_EUNSUPPORTED,
+                      "tf_inspect: the MFMA tile GEMM needs K %% 8 == 0 and N %% 32 == 0 (K=%d N=%d)",
+                      o.K, o.N);
+    if (o.N > 256) return tf::fail(TF_EUNSUPPORTED, "tf_inspect: GeMM-SpMM supports N <= 256");
+  } else {
+    o.K = 0;
+  }
+  if (o.lds_budget_bytes <= 0) o.lds_budget_bytes = 65536;
+  if (o.lds_budget_bytes > kMaxLds)
+    return tf::fail(TF_EINVAL, "tf_inspect: lds_budget_bytes %d exceeds %d", o.lds_budget_bytes, kMaxLds);
+  if (o.max_redundancy <= 0.f) o.max_redundancy = (o.op == TF_OP_GEMM_SPMM) ? 1.5f : 3.0f;
+  if (o.max_redundancy < 1.f) o.max_redundancy = 1.f;
+  if (o.long_row_nnz <= 0) o.long_row_nnz = 2048;
+  if (o.compute_units <= 0) o.compute_units = tf::default_compute_units();
+
+  // LDS the tile GEMM needs for staging C, before any slab row.
+  int gemm_kc = 0, staging = 0;
+  if (o.op == TF_OP_GEMM_SPMM) {
+    gemm_kc = std::min(o.K, std::max(8, (32768 / (4 * o.N)) / 8 * 8));
+    staging = gemm_kc * o.N * 4;
+  }
+  const int row_bytes = o.N * 4;
+  const int p_max = (o.lds_budget_bytes - staging) / row_bytes;
+  if (p_max < 8)
+    return tf::fail(TF_EINVAL, "tf_inspect: LDS budget %d holds only %d intermediate rows of N=%d",
+                    o.lds_budget_bytes, p_max, o.N);
+  int r_cap = o.tile_rows > 0 ? o.tile_rows : ceil_div(M, 2 * o.compute_units);
+  if (o.op == TF_OP_GEMM_SPMM) r_cap = ceil_div(r_cap, 32) * 32;
+  r_cap = std::max(r_cap, o.tile_rows > 0 ? 1 : 32);
+  r_cap = std::min(r_cap, p_max);
+  o.tile_rows = r_cap;
+
+  auto *S = new (std::nothrow) tf_schedule();
+  if (!S) return tf::fail(TF_ENOMEM, "tf_inspect: out of host memory");
+  try {
+    S->opts = o;
+    S->L = L;
+    S->M = M;
+    S->nnz = nnz;
+    S->gemm_kc = gemm_kc;
+
+    // Column extent of every second-op row (columns need not be sorted).
+    std::vector<int> lo(L), hi(L);
+    for (int i = 0; i < L; ++i) {
+      int a = INT_MAX, b = -1;
+      for (int k = Ap[i]; k < Ap[i + 1]; ++k) {
+        const int c = Ai[k];
+        if (c < 0 || c >= M) {
+          delete S;
+          return tf::fail(TF_EINVAL, "tf_inspect: column %d out of range at row %d", c, i);
+        }
+        a = std::min(a, c);
+        b = std::max(b, c);
+      }
+      if (b < 0) { a = std::min(i, M - 1); b = a - 1; }  // empty row: no dependence
+      lo[i] = a;
+      hi[i] = b + 1;
+    }
+    // A row whose own reach (itself plus its columns) exceeds the slab can never fuse.
+    auto reach_lo = [&](int i) { return std::min(lo[i], std::min(i, M - 1)); };
+    auto reach_hi = [&](int i) { return std::max(hi[i], std::min(i, M - 1) + 1); };
+    auto never = [&](int i) { return reach_hi(i) - reach_lo(i) > p_max; };
+
+    std::vector<char> fused(L, 0);
+    int slab_rows = 0;
+    int s = 0;
+    while (s < M) {
+      tf::TileDesc t{};
+      // 1. grow a tile whose producer window covers every fusable row it owns
+      int wlo = s, whi = s, e = s;
+      while (e < M && e - s < r_cap) {
+        int nlo = std::min(wlo, e), nhi = std::max(whi, e + 1);
+        if (e < L && !never(e)) { nlo = std::min(nlo, lo[e]); nhi = std::max(nhi, hi[e]); }
+        if (nhi - nlo > p_max) break;
+        wlo = nlo; whi = nhi; ++e;
+      }
+      const bool halo_ok = (e > s) && (e - s >= std::min(r_cap, 16) || e == M) &&
+                           (float)(whi - wlo) <= o.max_redundancy * (float)(e - s);
+      t.cons_begin = (int)S->fused_ids.size();
+      if (halo_ok) {
+        t.own_begin = s; t.own_end = e; t.prod_begin = wlo; t.prod_end = whi;
+        for (int i = s; i < e && i < L; ++i)
+          if (!never(i)) { S->fused_ids.push_back(i); fused[i] = 1; }
+      } else {
+        // 2. the reference's tiling: no recomputation, rows fuse iff their columns are in the tile
+        e = std::min(M, s + r_cap);
+        t.own_begin = s; t.own_end = e; t.prod_begin = s; t.prod_end = e;
+        for (int i = s; i < e && i < L; ++i)
+          if (lo[i] >= s && hi[i] <= e) { S->fused_ids.push_back(i); fused[i] = 1; }
+      }
+      t.cons_end = (int)S->fused_ids.size();
+      if (t.cons_end > t.cons_begin) slab_rows = std::max(slab_rows, t.prod_end - t.prod_begin);
+      else { t.prod_begin = t.own_begin; t.prod_end = t.own_end; }  // nothing to fuse: no halo
+      t.wb_begin = t.wb_end = t.own_begin;
+      S->n_producer_rows += t.prod_end - t.prod_begin;
+      S->tiles.push_back(t);
+      s = e;
+    }
+
+    // Remainder: rows not fused; long ones are cut into chunks.
+    std::vector<char> need(M, 0);
+    for (int i = 0; i < L; ++i) {
+      if (fused[i]) { S->fused_nnz += Ap[i + 1] - Ap[i]; continue; }
+      for (int k = Ap[i]; k < Ap[i + 1]; ++k) need[Ai[k]] = 1;
+      const int len = Ap[i + 1] - Ap[i];
+      if (len > o.long_row_nnz) {
+        tf::LongRow lr{i, (int)S->long_chunks.size(), 0, 0};
+        for (int k = Ap[i]; k < Ap[i + 1]; k += o.long_row_nnz) {
+          tf::LongChunk c{i, k, std::min(Ap[i + 1], k + o.long_row_nnz), (int)S->long_chunks.size()};
+          S->long_chunks.push_back(c);
+          ++lr.count;
+        }
+        S->long_rows.push_back(lr);
+      } else {
+        S->rem_rows.push_back(i);
+      }
+    }
+    for (auto &t : S->tiles) {
+      int a = -1, b = -1;
+      for (int r = t.own_begin; r < t.own_end; ++r)
+        if (need[r]) { if (a < 0) a = r; b = r + 1; }
+      if (a >= 0) { t.wb_begin = a; t.wb_end = b; S->n_writeback_rows += b - a; }
+    }
+    S->slab_rows = slab_rows;
+    S->lds_bytes = slab_rows * row_bytes + staging;
+
+    // MultiDimensionalSet-layout view (Fusion_Inspector.h:959-1010).
+    const int nt = (int)S->tiles.size();
+    std::vector<int> rem_all;
+    rem_all.reserve(S->rem_rows.size() + S->long_rows.size());
+    for (int i = 0; i < L; ++i)
+      if (!fused[i]) rem_all.push_back(i);
+    const int nrp = ceil_div((int)rem_all.size(), 64);
+    const int P = nt + nrp;
+    S->ptr1 = {0, nt, P};
+    S->ptr2.assign(P + 1, 0);
+    S->ker_begin.assign(2 * (size_t)P, 0);
+    S->id.reserve((size_t)M + L);
+    S->type.reserve((size_t)M + L);
+    S->tile_range.resize(4 * (size_t)nt);
+    S->writeback.resize(2 * (size_t)nt);
+    for (int p = 0; p < nt; ++p) {
+      const auto &t = S->tiles[p];
+      for (int r = t.own_begin; r < t.own_end; ++r) { S->id.push_back(r); S->type.push_back(0); }
+      S->ker_begin[2 * p] = (int)S->id.size();
+      for (int q = t.cons_begin; q < t.cons_end; ++q) { S->id.push_back(S->fused_ids[q]); S->type.push_back(1); }
+      S->ker_begin[2 * p + 1] = (int)S->id.size();
+      S->ptr2[p + 1] = (int)S->id.size();
+      S->tile_range[4 * p + 0] = t.prod_begin; S->tile_range[4 * p + 1] = t.prod_end;
+      S->tile_range[4 * p + 2] = t.own_begin;  S->tile_range[4 * p + 3] = t.own_end;
+      S->writeback[2 * p] = t.wb_begin; S->writeback[2 * p + 1] = t.wb_end;
+    }
+    for (int g = 0; g < nrp; ++g) {
+      const int p = nt + g;
+      S->ker_begin[2 * p] = (int)S->id.size();
+      for (int q = g * 64; q < std::min((int)rem_all.size(), (g + 1) * 64); ++q) {
+        S->id.push_back(rem_all[q]); S->type.push_back(1);
+      }
+      S->ker_begin[2 * p + 1] = (int)S->id.size();
+      S->ptr2[p + 1] = (int)S->id.size();
+    }
+  } catch (const std::bad_alloc &) {
+    delete S;
+    return tf::fail(TF_ENOMEM, "tf_inspect: out of host memory");
+  }
+  *out = S;
+  return TF_OK;
+}
+
+extern "C" void tf_schedule_free(tf_schedule *s) {
+  if (!s) return;
+  tf::release_device_schedule(s->dev);
+  delete s;
+}
+
+extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info *info) {
+  if (!s || !info) return tf::fail(TF_EINVAL, "tf_schedule_get_info: null argument");
+  std::memset(info, 0, sizeof(*info));
+  info->op = s->opts.op; info->N = s->opts.N; info->K = s->opts.K;
+  info->rows = s->L; info->inter_rows = s->M;
+  info->n_tiles = (int)s->tiles.size();
+  info->n_fused_rows = (int)s->fused_ids.size();
+  info->n_remainder_rows = (int)(s->rem_rows.size() + s->long_rows.size());
+  info->n_long_rows = (int)s->long_rows.size();
+  info->n_long_chunks = (int)s->long_chunks.size();
+  info->n_producer_rows = (int)std::min<long long>(s->n_producer_rows, INT_MAX);
+  info->n_writeback_rows = s->n_writeback_rows;
+  info->max_tile_producer_rows = s->slab_rows;
+  info->lds_bytes = s->lds_bytes;
+  info->fused_nnz = s->fused_nnz;
+  long long ws = 0;
+  if (s->n_writeback_rows > 0) ws += (long long)s->M * s->opts.N * 4;
+  ws += (long long)s->long_chunks.size() * s->opts.N * 4;
+  info->workspace_bytes = ws;
+  return TF_OK;
+}
+
+extern "C" tf_status tf_schedule_get_view(const tf_schedule *s, tf_schedule_view *v) {
+  if (!s || !v) return tf::fail(TF_EINVAL, "tf_schedule_get_view: null argument");
+  v->n1 = 2;
+  v->n_part = s->ptr1[2];
+  v->n_id = (int)s->id.size();
+  v->n_tiles = (int)s->tiles.size();
+  v->ptr1 = s->ptr1.data(); v->ptr2 = s->ptr2.data(); v->ker_begin = s->ker_begin.data();
+  v->id = s->id.data(); v->type = s->type.data();
+  v->tile_range = s->tile_range.data(); v->writeback = s->writeback.data();
+  return TF_OK;
+}
+
+extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, const int *Ap,
+                                          const int *Ai) {
+  if (!s || !Ap) return tf::fail(TF_EINVAL, "tf_schedule_validate: null argument");
+  if (L != s->L || M != s->M || Ap[L] != s->nnz)
+    return tf::fail(TF_ESCHEDULE, "schedule was built for %d x %d with %lld entries, got %d x %d with %d",
+                    s->L, s->M, s->nnz, L, M, Ap[L]);
+  const int row_bytes = s->opts.N * 4;
+  std::vector<int> owner(M, -1), done(L, 0);
+  std::vector<char> stored(M, 0);
+  int prev_end = 0;
+  for (size_t ti = 0; ti < s->tiles.size(); ++ti) {
+    const auto &t = s->tiles[ti];
+    if (t.own_begin != prev_end || t.own_end <= t.own_begin)
+      return tf::fail(TF_ESCHEDULE, "tile %zu: owned rows [%d,%d) do not continue at %d", ti, t.own_begin, t.own_end, prev_end);
+    prev_end = t.own_end;
+    if (t.prod_begin > t.own_begin || t.prod_end < t.own_end || t.prod_begin < 0 || t.prod_end > M)
+      return tf::fail(TF_ESCHEDULE, "tile %zu: producer range [%d,%d) does not cover owned rows [%d,%d)", ti, t.prod_begin, t.prod_end, t.own_begin, t.own_end);
+    if (t.cons_end > t.cons_begin &&
+        (long long)(t.prod_end - t.prod_begin) * row_bytes > s->opts.lds_budget_bytes)
+      return tf::fail(TF_ESCHEDULE, "tile %zu: slab of %d rows exceeds the LDS budget", ti, t.prod_end - t.prod_begin);
+    if (t.wb_begin < t.own_begin || t.wb_end > t.own_end || t.wb_end < t.wb_begin)
+      return tf::fail(TF_ESCHEDULE, "tile %zu: write-back range [%d,%d) outside owned rows", ti, t.wb_begin, t.wb_end);
+    for (int r = t.own_begin; r < t.own_end; ++r) owner[r] = (int)ti;
+    for (int r = t.wb_begin; r < t.wb_end; ++r) stored[r] = 1;
+    if (t.cons_begin < 0 || t.cons_end > (int)s->fused_ids.size() || t.cons_end < t.cons_begin)
+      return tf::fail(TF_ESCHEDULE, "tile %zu: bad fused id range", ti);
+    for (int q = t.cons_begin; q < t.cons_end; ++q) {
+      const int i = s->fused_ids[q];
+      if (i < 0 || i >= L) return tf::fail(TF_ESCHEDULE, "tile %zu: fused row %d out of range", ti, i);
+      if (done[i]++) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled twice", i);
+      for (int k = Ap[i]; k < Ap[i + 1]; ++k)
+        if (Ai[k] < t.prod_begin || Ai[k] >= t.prod_end)
+          return tf::fail(TF_ESCHEDULE, "fused row %d reads intermediate row %d outside tile %zu [%d,%d)", i, Ai[k], ti, t.prod_begin, t.prod_end);
+    }
+  }
+  if (prev_end != M) return tf::fail(TF_ESCHEDULE, "owned rows end at %d, expected %d", prev_end, M);
+  auto check_rem = [&](int i) -> tf_status {
+    if (i < 0 || i >= L) return tf::fail(TF_ESCHEDULE, "remainder row %d out of range", i);
+    for (int k = Ap[i]; k < Ap[i + 1]; ++k)
+      if (!stored[Ai[k]])
+        return tf::fail(TF_ESCHEDULE, "remainder row %d reads intermediate row %d that no tile stores", i, Ai[k]);
+    return TF_OK;
+  };
+  for (int i : s->rem_rows) {
+    if (done[i]++) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled twice", i);
+    if (Ap[i + 1] - Ap[i] > s->opts.long_row_nnz)
+      return tf::fail(TF_ESCHEDULE, "remainder row %d is long but not chunked", i);
+    if (tf_status rc = check_rem(i)) return rc;
+  }
+  for (const auto &lr : s->long_rows) {
+    if (tf_status rc = check_rem(lr.row)) return rc;
+    if (done[lr.row]++) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled twice", lr.row);
+    int k = Ap[lr.row];
+    if (lr.first < 0 || lr.count <= 0 || lr.first + lr.count > (int)s->long_chunks.size())
+      return tf::fail(TF_ESCHEDULE, "long row %d: bad chunk range", lr.row);
+    for (int c = lr.first; c < lr.first + lr.count; ++c) {
+      const auto &ch = s->long_chunks[c];
+      if (ch.row != lr.row || ch.k_begin != k || ch.k_end <= ch.k_begin || ch.slot != c ||
+          ch.k_end - ch.k_begin > s->opts.long_row_nnz)
+        return tf::fail(TF_ESCHEDULE, "long row %d: chunk %d does not continue at entry %d", lr.row, c, k);
+      k = ch.k_end;
+    }
+    if (k != Ap[lr.row + 1]) return tf::fail(TF_ESCHEDULE, "long row %d: chunks end at %d, row ends at %d", lr.row, k, Ap[lr.row + 1]);
+  }
+  for (int i = 0; i < L; ++i)
+    if (done[i] != 1) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled %d times", i, done[i]);
+  return TF_OK;
+}

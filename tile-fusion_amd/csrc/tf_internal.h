@@ -1,0 +1,67 @@
+// Internal declarations shared by the host-side inspector, the C ABI and the HIP
+// kernels of libtilefusion_hip.  Not installed; the public surface is
+// include/tilefusion_hip.h.
+#pragma once
+#include <cstdarg>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "tilefusion_hip.h"
+
+namespace tf {
+
+// One fused tile = one workgroup.  The workgroup computes intermediate rows
+// [prod_begin, prod_end) into LDS, stores rows [wb_begin, wb_end) of them to the
+// intermediate in HBM (the ones remainder rows will read), then computes the
+// second-op rows ids[cons_begin .. cons_end) out of LDS.
+struct TileDesc {
+  int prod_begin, prod_end;
+  int own_begin, own_end;
+  int wb_begin, wb_end;
+  int cons_begin, cons_end;
+};
+static_assert(sizeof(TileDesc) == 32, "TileDesc is read as two int4 by the kernels");
+
+// A chunk of one long remainder row: stored entries [k_begin, k_end) of `row`,
+// reduced by a whole workgroup into partial[slot].
+struct LongChunk {
+  int row, k_begin, k_end, slot;
+};
+// All partials of one long row: D[row] = sum partial[first .. first+count).
+struct LongRow {
+  int row, first, count, pad;
+};
+
+struct DeviceSchedule;  // device copies + workspace, defined in tf_api.cpp
+
+}  // namespace tf
+
+struct tf_schedule {
+  tf_inspect_opts opts{};  // resolved (no zero "default" fields left)
+  int L = 0, M = 0;
+  int lds_bytes = 0;          // dynamic LDS of the fused kernel: intermediate slab (+ GEMM staging)
+  int slab_rows = 0;          // max producer rows of any tile
+  int gemm_kc = 0;            // rows of C staged in LDS per step (GeMM-SpMM)
+  std::vector<tf::TileDesc> tiles;
+  std::vector<int> fused_ids;       // second-op rows per tile, tile after tile
+  std::vector<int> rem_rows;        // remainder rows handled one row per lane group
+  std::vector<tf::LongChunk> long_chunks;
+  std::vector<tf::LongRow> long_rows;
+  long long fused_nnz = 0;
+  int n_writeback_rows = 0;
+  long long n_producer_rows = 0;
+  // MultiDimensionalSet-layout view
+  std::vector<int> ptr1, ptr2, ker_begin, id, type, tile_range, writeback;
+  // pattern fingerprint, checked by the executors against their operands
+  long long nnz = 0;
+  tf::DeviceSchedule *dev = nullptr;
+};
+
+namespace tf {
+
+tf_status fail(tf_status code, const char *fmt, ...);
+void release_device_schedule(DeviceSchedule *d);
+int default_compute_units();
+
+}  // namespace tf

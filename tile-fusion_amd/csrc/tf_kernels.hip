@@ -1,0 +1,502 @@
+// HIP kernels of libtilefusion_hip, written for gfx950 (CDNA4): 64-wide wavefronts,
+// LDS slabs of the intermediate, fp32 MFMA for the tile GEMM.
+//
+// Work decomposition used by every sparse kernel here: a wavefront is cut into lane
+// groups of LPR lanes; one group owns one output row at a time and each lane owns VEC
+// adjacent columns of it (LPR*VEC columns per pass, a 16-byte load per lane when
+// VEC = 4).  A group first loads up to LPR (column, value) pairs of its CSR row with
+// one coalesced load, then walks them in CSR order, broadcasting each pair inside the
+// group, so the per-element sequence is acc = fma(value, x[column], acc) exactly as in
+// the reference's AVX2 kernels (fusion/src/SpMM_SpMM_vectorized.cpp:892-936).
+#include <hip/hip_runtime.h>
+
+#include "tf_internal.h"
+
+namespace tf {
+
+constexpr int kBlock = 256;  // threads per workgroup of every kernel in this file
+constexpr int kXcds = 8;     // workgroup ids are dealt round-robin over the 8 XCDs
+
+template <int V> struct alignas(4 * V) fvec { float v[V]; };
+
+template <int V> __device__ __forceinline__ fvec<V> vzero() {
+  fvec<V> r;
+#pragma unroll
+  for (int i = 0; i < V; ++i) r.v[i] = 0.f;
+  return r;
+}
+template <int V> __device__ __forceinline__ void vfma(float a, const fvec<V> &x, fvec<V> &acc) {
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc.v[i] = __builtin_fmaf(a, x.v[i], acc.v[i]);
+}
+template <int V> __device__ __forceinline__ void vadd(const fvec<V> &x, fvec<V> &acc) {
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc.v[i] += x.v[i];
+}
+
+// Consecutive workgroup ids land on different XCDs (each with its own L2).  Remap so
+// that every XCD works on one contiguous run of work items: neighbours share halo
+// rows and gather targets, which then stay in one L2.
+__device__ __forceinline__ int xcd_contiguous(int bid, int per_xcd) {
+  return (bid % kXcds) * per_xcd + bid / kXcds;
+}
+
+template <int V> struct GlobalRows {
+  const float *__restrict__ base;
+  int ld;    // row stride in floats
+  int coff;  // this lane's first column
+  __device__ __forceinline__ fvec<V> load(int row) const {
+    return *reinterpret_cast<const fvec<V> *>(base + (size_t)row * ld + coff);
+  }
+};
+template <int V> struct LdsRows {
+  const float *base;  // slab; row r of the intermediate is at (r - first) * ld
+  int ld, coff, first;
+  __device__ __forceinline__ fvec<V> load(int row) const {
+    return *reinterpret_cast<const fvec<V> *>(base + (row - first) * ld + coff);
+  }
+};
+
+// acc += sum over stored entries k in [kb, ke) of val[k] * src.row(idx[k]), CSR order.
+// All LPR lanes of the group must call this together (it shuffles inside the group).
+template <int V, int LPR, class Src>
+__device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float *__restrict__ val,
+                                        int kb, int ke, int glane, bool col_ok, const Src &src,
+                                        fvec<V> &acc) {
+  for (int k0 = kb; k0 < ke; k0 += LPR) {
+    const int k = k0 + glane;
+    int c = 0;
+    float a = 0.f;
+    if (k < ke) { c = idx[k]; a = val[k]; }
+    const int cnt = min(LPR, ke - k0);
+    int t = 0;
+    for (; t + 4 <= cnt; t += 4) {
+      const int c0 = __shfl(c, t, LPR), c1 = __shfl(c, t + 1, LPR);
+      const int c2 = __shfl(c, t + 2, LPR), c3 = __shfl(c, t + 3, LPR);
+      const float a0 = __shfl(a, t, LPR), a1 = __shfl(a, t + 1, LPR);
+      const float a2 = __shfl(a, t + 2, LPR), a3 = __shfl(a, t + 3, LPR);
+      if (col_ok) {
+        const fvec<V> x0 = src.load(c0), x1 = src.load(c1), x2 = src.load(c2), x3 = src.load(c3);
+        vfma<V>(a0, x0, acc);
+        vfma<V>(a1, x1, acc);
+        vfma<V>(a2, x2, acc);
+        vfma<V>(a3, x3, acc);
+      }
+    }
+    for (; t < cnt; ++t) {
+      const int c0 = __shfl(c, t, LPR);
+      const float a0 = __shfl(a, t, LPR);
+      if (col_ok) vfma<V>(a0, src.load(c0), acc);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Fused SpMM-SpMM tile kernel: one workgroup per tile.
+//   phase 1  T[r,:] = sum_j Bx[j] * C[Bi[j],:]   for r in the tile's producer range -> LDS
+//            (+ HBM for the rows the remainder will read)
+//   phase 2  D[i,:] = sum_k Ax[k] * T[Ai[k],:]   for the tile's fused rows, T read from LDS
+// ---------------------------------------------------------------------------------
+template <int V, int LPR>
+__global__ __launch_bounds__(kBlock) void fused_spmm_spmm_kernel(
+    const TileDesc *__restrict__ tiles, int n_tiles, int per_xcd, const int *__restrict__ fused_ids,
+    const int *__restrict__ Bp, const int *__restrict__ Bi, const float *__restrict__ Bx,
+    const float *__restrict__ C, const int *__restrict__ Ap, const int *__restrict__ Ai,
+    const float *__restrict__ Ax, float *__restrict__ D, float *__restrict__ T, int N, int ldc,
+    int accumulate) {
+  extern __shared__ __align__(16) float slab[];
+  const int tile = xcd_contiguous(blockIdx.x, per_xcd);
+  if (tile >= n_tiles) return;
+  const TileDesc t = tiles[tile];
+  constexpr int G = kBlock / LPR;
+  const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
+  const bool has_cons = t.cons_end > t.cons_begin;
+  for (int c0 = 0; c0 < N; c0 += LPR * V) {
+    const int coff = c0 + glane * V;
+    const bool ok = coff < N;
+    const GlobalRows<V> csrc{C, ldc, ok ? coff : 0};
+    for (int r = t.prod_begin + group; r < t.prod_end; r += G) {
+      fvec<V> acc = vzero<V>();
+      row_dot<V, LPR>(Bi, Bx, Bp[r], Bp[r + 1], glane, ok, csrc, acc);
+      if (ok) {
+        if (has_cons) *reinterpret_cast<fvec<V> *>(slab + (r - t.prod_begin) * N + coff) = acc;
+        if (r >= t.wb_begin && r < t.wb_end)
+          *reinterpret_cast<fvec<V> *>(T + (size_t)r * N + coff) = acc;
+      }
+    }
+    if (!has_cons) continue;
+    __syncthreads();
+    const LdsRows<V> tsrc{slab, N, ok ? coff : 0, t.prod_begin};
+    for (int q = t.cons_begin + group; q < t.cons_end; q += G) {
+      const int i = fused_ids[q];
+      fvec<V> acc = vzero<V>();
+      if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)i * N + coff);
+      row_dot<V, LPR>(Ai, Ax, Ap[i], Ap[i + 1], glane, ok, tsrc, acc);
+      if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)i * N + coff) = acc;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Row-wise SpMM  Y[i,:] = sum_k Ax[k] * X[Ai[k],:]  for i = rows[q] (or i = q when rows
+// is null).  Serves the unfused remainder (X = the intermediate in HBM) and tf_spmm.
+// ---------------------------------------------------------------------------------
+template <int V, int LPR>
+__global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
+    const int *__restrict__ rows, int n_rows, int per_xcd, const int *__restrict__ Ap,
+    const int *__restrict__ Ai, const float *__restrict__ Ax, const float *__restrict__ X, int ldx,
+    float *__restrict__ Y, int N, int accumulate) {
+  constexpr int G = kBlock / LPR;
+  const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
+  const int q = xcd_contiguous(blockIdx.x, per_xcd) * G + group;
+  if (q >= n_rows) return;  // whole lane groups leave together
+  const int i = rows ? rows[q] : q;
+  const int kb = Ap[i], ke = Ap[i + 1];
+  for (int c0 = 0; c0 < N; c0 += LPR * V) {
+    const int coff = c0 + glane * V;
+    const bool ok = coff < N;
+    const GlobalRows<V> src{X, ldx, ok ? coff : 0};
+    fvec<V> acc = vzero<V>();
+    if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
+    row_dot<V, LPR>(Ai, Ax, kb, ke, glane, ok, src, acc);
+    if (ok) *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Long remainder rows.  One workgroup per chunk of a row: lane groups take LPR-entry
+// segments round-robin, partial sums are combined across the groups through LDS in a
+// fixed order, and the chunk's result goes to partial[slot].  A second kernel adds a
+// row's chunks in order, so the result does not depend on scheduling.
+// ---------------------------------------------------------------------------------
+template <int V, int LPR>
+__global__ __launch_bounds__(kBlock) void spmm_long_chunk_kernel(
+    const LongChunk *__restrict__ chunks, const int *__restrict__ Ai, const float *__restrict__ Ax,
+    const float *__restrict__ X, int ldx, float *__restrict__ partial, int N) {
+  constexpr int G = kBlock / LPR;
+  __shared__ __align__(16) float red[G * LPR * V];
+  const LongChunk ch = chunks[blockIdx.x];
+  const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
+  for (int c0 = 0; c0 < N; c0 += LPR * V) {
+    const int coff = c0 + glane * V;
+    const bool ok = coff < N;
+    const GlobalRows<V> src{X, ldx, ok ? coff : 0};
+    fvec<V> acc = vzero<V>();
+    for (int k0 = ch.k_begin + group * LPR; k0 < ch.k_end; k0 += G * LPR)
+      row_dot<V, LPR>(Ai, Ax, k0, min(ch.k_end, k0 + LPR), glane, ok, src, acc);
+    *reinterpret_cast<fvec<V> *>(red + (group * LPR + glane) * V) = acc;
+    __syncthreads();
+    if (group == 0 && ok) {
+      fvec<V> sum = vzero<V>();
+      for (int g = 0; g < G; ++g) vadd<V>(*reinterpret_cast<const fvec<V> *>(red + (g * LPR + glane) * V), sum);
+      *reinterpret_cast<fvec<V> *>(partial + (size_t)ch.slot * N + coff) = sum;
+    }
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void long_row_reduce_kernel(const LongRow *__restrict__ rows,
+                                                                 const float *__restrict__ partial,
+                                                                 float *__restrict__ Y, int N,
+                                                                 int accumulate) {
+  const LongRow lr = rows[blockIdx.x];
+  for (int c = threadIdx.x; c < N; c += kBlock) {
+    float s = accumulate ? Y[(size_t)lr.row * N + c] : 0.f;
+    for (int p = 0; p < lr.count; ++p) s += partial[(size_t)(lr.first + p) * N + c];
+    Y[(size_t)lr.row * N + c] = s;
+  }
+}
+
+__global__ void fill_kernel(float *__restrict__ p, size_t n, float v) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+// ---------------------------------------------------------------------------------
+// Tile GEMM on fp32 MFMA.  A wavefront owns a block of 32 rows and all N = 32*NB
+// columns: NB accumulators of v_mfma_f32_32x32x2_f32.  C (K x N) is staged through LDS
+// kc rows at a time; the rows of B are read straight from HBM, 16 bytes per lane: lane
+// (i = lane%32, h = lane/32) loads B[row0+i][k0+8m+4h .. +4), so one load feeds four
+// MFMA steps whose k index is 8m+4h+t.  The same k is used for the C operand, so the
+// permuted k order inside a group of 8 does not change the product.
+// ---------------------------------------------------------------------------------
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+template <int NB>
+__device__ __forceinline__ void gemm_accumulate_chunk(const float *__restrict__ Xrow, bool row_ok,
+                                                      int kc, const float *stage, int N, int h, int j,
+                                                      v16f (&acc)[NB]) {
+  for (int m = 0; m < kc; m += 8) {
+    fvec<4> a4 = vzero<4>();
+    if (row_ok) a4 = *reinterpret_cast<const fvec<4> *>(Xrow + m + 4 * h);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float *w = stage + (m + 4 * h + t) * N + j;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.v[t], w[nb * 32], acc[nb], 0, 0, 0);
+    }
+  }
+}
+
+// Cooperative copy of rows [k0, k0+kc) of W (K x N, row-major) into LDS.
+__device__ __forceinline__ void stage_weights(const float *__restrict__ W, int N, int k0, int kc, float *stage) {
+  const int n4 = kc * N / 4;
+  const fvec<4> *src = reinterpret_cast<const fvec<4> *>(W + (size_t)k0 * N);
+  fvec<4> *dst = reinterpret_cast<fvec<4> *>(stage);
+  for (int i = threadIdx.x; i < n4; i += kBlock) dst[i] = src[i];
+}
+
+// Computes intermediate rows [p0, p1) = X[p0:p1, :K] * W for the whole workgroup.
+// Results go to `slab` (row r at (r-p0)*N) when slab != null and to T rows in
+// [wb0, wb1) when T != null.  Must be called by all threads of the workgroup.
+template <int NB>
+__device__ __forceinline__ void tile_gemm(const float *__restrict__ X, const float *__restrict__ W, int K,
+                                          int kc, int p0, int p1, float *stage, float *slab,
+                                          float *__restrict__ T, int wb0, int wb1) {
+  constexpr int N = NB * 32;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int h = lane / 32, j = lane % 32;
+  constexpr int W_PER_BLOCK = kBlock / 64;
+  const int nrb = (p1 - p0 + 31) / 32;
+  const int iters = (nrb + W_PER_BLOCK - 1) / W_PER_BLOCK;
+  const bool single = (K <= kc);
+  if (single) {
+    stage_weights(W, N, 0, K, stage);
+    __syncthreads();
+  }
+  for (int it = 0; it < iters; ++it) {
+    const int rb = it * W_PER_BLOCK + wave;
+    const int row = p0 + rb * 32 + j;  // the row this lane feeds as the A operand
+    const bool row_ok = rb < nrb && row < p1;
+    const float *Xrow = X + (size_t)(row_ok ? row : p0) * K;
+    v16f acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
+    if (single) {
+      if (rb < nrb) gemm_accumulate_chunk<NB>(Xrow, row_ok, K, stage, N, h, j, acc);
+    } else {
+      for (int k0 = 0; k0 < K; k0 += kc) {
+        const int cur = min(kc, K - k0);
+        __syncthreads();
+        stage_weights(W, N, k0, cur, stage);
+        __syncthreads();
+        if (rb < nrb) gemm_accumulate_chunk<NB>(Xrow + k0, row_ok, cur, stage, N, h, j, acc);
+      }
+    }
+    if (rb < nrb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int orow = p0 + rb * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+        if (orow < p1) {
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const float v = acc[nb][r];
+            if (slab) slab[(orow - p0) * N + nb * 32 + j] = v;
+            if (T && orow >= wb0 && orow < wb1) T[(size_t)orow * N + nb * 32 + j] = v;
+          }
+        }
+      }
+    }
+  }
+}
+
+// Fused GeMM-SpMM tile kernel: phase 1 is the tile GEMM into the LDS slab, phase 2 the
+// consumer rows out of LDS (same as the SpMM-SpMM kernel).
+template <int NB, int LPR>
+__global__ __launch_bounds__(kBlock) void fused_gemm_spmm_kernel(
+    const TileDesc *__restrict__ tiles, int n_tiles, int per_xcd, const int *__restrict__ fused_ids,
+    const float *__restrict__ B, const float *__restrict__ C, int K, int kc, const int *__restrict__ Ap,
+    const int *__restrict__ Ai, const float *__restrict__ Ax, float *__restrict__ D,
+    float *__restrict__ T, int accumulate) {
+  extern __shared__ __align__(16) float lds[];
+  constexpr int N = NB * 32;
+  constexpr int V = 4;
+  const int tile = xcd_contiguous(blockIdx.x, per_xcd);
+  if (tile >= n_tiles) return;
+  const TileDesc t = tiles[tile];
+  float *stage = lds;
+  float *slab = lds + kc * N;
+  const bool has_cons = t.cons_end > t.cons_begin;
+  tile_gemm<NB>(B, C, K, kc, t.prod_begin, t.prod_end, stage, has_cons ? slab : nullptr,
+                t.wb_end > t.wb_begin ? T : nullptr, t.wb_begin, t.wb_end);
+  if (!has_cons) return;
+  __syncthreads();
+  constexpr int G = kBlock / LPR;
+  const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
+  const int coff = glane * V;
+  const bool ok = coff < N;
+  const LdsRows<V> tsrc{slab, N, ok ? coff : 0, t.prod_begin};
+  for (int q = t.cons_begin + group; q < t.cons_end; q += G) {
+    const int i = fused_ids[q];
+    fvec<V> acc = vzero<V>();
+    if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)i * N + coff);
+    row_dot<V, LPR>(Ai, Ax, Ap[i], Ap[i + 1], glane, ok, tsrc, acc);
+    if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)i * N + coff) = acc;
+  }
+}
+
+// Plain GEMM  Y = X * W  (tf_gemm): 128 rows per workgroup, no slab.
+template <int NB>
+__global__ __launch_bounds__(kBlock) void gemm_kernel(const float *__restrict__ X, const float *__restrict__ W,
+                                                      float *__restrict__ Y, int M, int K, int kc,
+                                                      int per_xcd, int n_blocks) {
+  extern __shared__ __align__(16) float lds[];
+  const int b = xcd_contiguous(blockIdx.x, per_xcd);
+  if (b >= n_blocks) return;
+  const int p0 = b * 128, p1 = min(M, p0 + 128);
+  tile_gemm<NB>(X, W, K, kc, p0, p1, lds, nullptr, Y, p0, p1);
+}
+
+// ---------------------------------------------------------------------------------
+// Host-side launchers
+// ---------------------------------------------------------------------------------
+namespace {
+
+struct Shape { int V, LPR; };
+
+Shape pick_shape(int N) {
+  int V = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+  int lanes = (N + V - 1) / V;
+  int LPR = 8;
+  while (LPR < lanes && LPR < 64) LPR *= 2;
+  return {V, LPR};
+}
+
+inline int per_xcd_of(int n) { return (n + kXcds - 1) / kXcds; }
+
+template <class F> hipError_t allow_lds(F kernel, int bytes) {
+  if (bytes <= 65536) return hipSuccess;
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+#define TF_DISPATCH_VL(V_, L_, CALL)                                         \
+  do {                                                                       \
+    if (V_ == 4) {                                                           \
+      if (L_ == 8) { CALL(4, 8); } else if (L_ == 16) { CALL(4, 16); }       \
+      else if (L_ == 32) { CALL(4, 32); } else { CALL(4, 64); }              \
+    } else if (V_ == 2) {                                                    \
+      if (L_ == 8) { CALL(2, 8); } else if (L_ == 16) { CALL(2, 16); }       \
+      else if (L_ == 32) { CALL(2, 32); } else { CALL(2, 64); }              \
+    } else {                                                                 \
+      if (L_ == 8) { CALL(1, 8); } else if (L_ == 16) { CALL(1, 16); }       \
+      else if (L_ == 32) { CALL(1, 32); } else { CALL(1, 64); }              \
+    }                                                                        \
+  } while (0)
+
+#define TF_DISPATCH_NB(NB_, CALL)                                            \
+  do {                                                                       \
+    switch (NB_) {                                                           \
+      case 1: CALL(1); break; case 2: CALL(2); break; case 3: CALL(3); break; \
+      case 4: CALL(4); break; case 5: CALL(5); break; case 6: CALL(6); break; \
+      case 7: CALL(7); break; default: CALL(8); break;                       \
+    }                                                                        \
+  } while (0)
+
+}  // namespace
+
+hipError_t launch_fused_spmm_spmm(const TileDesc *tiles, int n_tiles, const int *fused_ids,
+                                  const int *Bp, const int *Bi, const float *Bx, const float *C,
+                                  const int *Ap, const int *Ai, const float *Ax, float *D, float *T,
+                                  int N, int lds_bytes, int accumulate, hipStream_t st) {
+  if (n_tiles <= 0) return hipSuccess;
+  const Shape s = pick_shape(N);
+  const int per = per_xcd_of(n_tiles);
+  hipError_t err = hipSuccess;
+#define CALL(V_, L_)                                                                       \
+  err = allow_lds(fused_spmm_spmm_kernel<V_, L_>, lds_bytes);                              \
+  if (err == hipSuccess)                                                                   \
+    hipLaunchKernelGGL((fused_spmm_spmm_kernel<V_, L_>), dim3(per *kXcds), dim3(kBlock),   \
+                       lds_bytes, st, tiles, n_tiles, per, fused_ids, Bp, Bi, Bx, C, Ap, Ai, \
+                       Ax, D, T, N, N, accumulate)
+  TF_DISPATCH_VL(s.V, s.LPR, CALL);
+#undef CALL
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const int *Ai, const float *Ax,
+                            const float *X, float *Y, int N, int accumulate, hipStream_t st) {
+  if (n_rows <= 0) return hipSuccess;
+  const Shape s = pick_shape(N);
+  const int G = kBlock / s.LPR;
+  const int blocks = (n_rows + G - 1) / G;
+  const int per = per_xcd_of(blocks);
+#define CALL(V_, L_)                                                                        \
+  hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(per *kXcds), dim3(kBlock), 0, st, rows, \
+                     n_rows, per, Ap, Ai, Ax, X, N, Y, N, accumulate)
+  TF_DISPATCH_VL(s.V, s.LPR, CALL);
+#undef CALL
+  return hipGetLastError();
+}
+
+hipError_t launch_long_rows(const LongChunk *chunks, int n_chunks, const LongRow *rows, int n_long,
+                            const int *Ai, const float *Ax, const float *X, float *partial, float *Y,
+                            int N, int accumulate, hipStream_t st) {
+  if (n_chunks <= 0) return hipSuccess;
+  const Shape s = pick_shape(N);
+#define CALL(V_, L_)                                                                          \
+  hipLaunchKernelGGL((spmm_long_chunk_kernel<V_, L_>), dim3(n_chunks), dim3(kBlock), 0, st,   \
+                     chunks, Ai, Ax, X, N, partial, N)
+  TF_DISPATCH_VL(s.V, s.LPR, CALL);
+#undef CALL
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  hipLaunchKernelGGL(long_row_reduce_kernel, dim3(n_long), dim3(kBlock), 0, st, rows, partial, Y, N,
+                     accumulate);
+  return hipGetLastError();
+}
+
+hipError_t launch_fused_gemm_spmm(const TileDesc *tiles, int n_tiles, const int *fused_ids,
+                                  const float *B, const float *C, int K, int kc, const int *Ap,
+                                  const int *Ai, const float *Ax, float *D, float *T, int N,
+                                  int lds_bytes, int accumulate, hipStream_t st) {
+  if (n_tiles <= 0) return hipSuccess;
+  const int per = per_xcd_of(n_tiles);
+  const int NB = N / 32;
+  const int LPR = pick_shape(N).LPR;
+  hipError_t err = hipSuccess;
+#define CALL2(NB_, L_)                                                                      \
+  err = allow_lds(fused_gemm_spmm_kernel<NB_, L_>, lds_bytes);                              \
+  if (err == hipSuccess)                                                                    \
+    hipLaunchKernelGGL((fused_gemm_spmm_kernel<NB_, L_>), dim3(per *kXcds), dim3(kBlock),   \
+                       lds_bytes, st, tiles, n_tiles, per, fused_ids, B, C, K, kc, Ap, Ai, Ax, \
+                       D, T, accumulate)
+#define CALL(NB_)                                                         \
+  do {                                                                    \
+    if (LPR == 8) { CALL2(NB_, 8); } else if (LPR == 16) { CALL2(NB_, 16); } \
+    else if (LPR == 32) { CALL2(NB_, 32); } else { CALL2(NB_, 64); }      \
+  } while (0)
+  TF_DISPATCH_NB(NB, CALL);
+#undef CALL
+#undef CALL2
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+hipError_t launch_gemm(const float *X, const float *W, float *Y, int M, int K, int N, int kc,
+                       hipStream_t st) {
+  if (M <= 0) return hipSuccess;
+  const int blocks = (M + 127) / 128;
+  const int per = per_xcd_of(blocks);
+  const int lds_bytes = kc * N * 4;
+  const int NB = N / 32;
+  hipError_t err = hipSuccess;
+#define CALL(NB_)                                                                               \
+  err = allow_lds(gemm_kernel<NB_>, lds_bytes);                                                 \
+  if (err == hipSuccess)                                                                        \
+    hipLaunchKernelGGL((gemm_kernel<NB_>), dim3(per *kXcds), dim3(kBlock), lds_bytes, st, X, W, \
+                       Y, M, K, kc, per, blocks)
+  TF_DISPATCH_NB(NB, CALL);
+#undef CALL
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+hipError_t launch_fill(float *p, size_t n, float v, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  const int blocks = (int)std::min<size_t>((n + 255) / 256, 65536);
+  hipLaunchKernelGGL(fill_kernel, dim3(blocks), dim3(256), 0, st, p, n, v);
+  return hipGetLastError();
+}
+
+}  // namespace tf
