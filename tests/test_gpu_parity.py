@@ -1,0 +1,316 @@
+"""Parity of the HIP executors with the CPU oracle, through the C ABI, on a real MI355X.
+
+SpMM-SpMM is bit-exact (same fma sequence per output element as the reference's AVX2
+kernels); GeMM-SpMM and split long rows are held to max|got - want| / max|want| <= 1e-4
+(the fp32 MFMA GEMM and the chunked rows sum in a different order), and are exact on
+integer-valued operands."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+def run_spmm_spmm(tf, A, B, Cd, accumulate=False, D0=None, **kw):
+    Ah = tf.CsrMatrix.from_scipy(A)
+    Bh = Ah if B is A else tf.CsrMatrix.from_scipy(B)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=Cd.shape[1], **kw)
+    S.validate()
+    D = tf.DenseMatrix(A.shape[0], Cd.shape[1], D0) if D0 is not None else tf.DenseMatrix(A.shape[0], Cd.shape[1])
+    if D0 is None:
+        D.fill(float("nan"))  # overwrite mode must not read D
+    tf.spmm_spmm(Ah, Bh, tf.DenseMatrix.from_numpy(Cd), D, S, accumulate=accumulate)
+    tf.device_synchronize()
+    return D.to_numpy(), S.info()
+
+
+def run_gemm_spmm(tf, A, B, Cd, accumulate=False, D0=None, **kw):
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=Cd.shape[1], K=B.shape[1], **kw)
+    S.validate()
+    D = tf.DenseMatrix(A.shape[0], Cd.shape[1], D0) if D0 is not None else tf.DenseMatrix(A.shape[0], Cd.shape[1])
+    if D0 is None:
+        D.fill(float("nan"))
+    tf.gemm_spmm(Ah, tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(Cd), D, S, accumulate=accumulate)
+    tf.device_synchronize()
+    return D.to_numpy(), S.info()
+
+
+def oracle_spmm_spmm(orc, A, B, Cd):
+    return orc.spmm_spmm(A, B, Cd, orc.unfused_schedule(max(A.shape[0], B.shape[0])) if A.shape[0] == B.shape[0]
+                         else _two_level(A.shape[0], B.shape[0], orc), nthreads=8)[0]
+
+
+def _two_level(L, M, orc):
+    ids = np.concatenate([np.arange(M), np.arange(L)]).astype(np.int32)
+    typ = np.concatenate([np.zeros(M), np.ones(L)]).astype(np.int32)
+    return orc.Schedule(2, [0, 1, 2], [0, M, M + L], [M, M, M, M + L], ids, typ)
+
+
+# ---- SpMM-SpMM ----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("N", [128, 64, 32, 256, 8, 20, 6, 5, 320])
+def test_spmm_spmm_banded_bit_exact(gpu, tf, orc, N):
+    say(f"spmm_spmm banded N={N}")
+    A = tf.workloads.banded_random(3000, 32, 16, seed=31)
+    Cd = tf.workloads.uniform((3000, N), 32)
+    want = oracle_spmm_spmm(orc, A, A, Cd)
+    for kw in (dict(), dict(max_redundancy=1.0), dict(lds_budget_bytes=163840, tile_rows=200), dict(tile_rows=7)):
+        got, info = run_spmm_spmm(tf, A, A, Cd, **kw)
+        assert np.array_equal(got, want), (N, kw, orc.rel_err(got, want))
+    assert info["n_fused_rows"] > 0
+
+
+@pytest.mark.parametrize("idx,scale", [(2, 0.05), (5, 0.004), (5, 0.03)])
+def test_spmm_spmm_configs_bit_exact(gpu, tf, orc, idx, scale):
+    cfg = tf.workloads.make_config(idx, scale)
+    say(f"spmm_spmm {cfg['name']} scale={scale} rows={cfg['A'].shape[0]}")
+    want = oracle_spmm_spmm(orc, cfg["A"], cfg["A"], cfg["C"])
+    got, info = run_spmm_spmm(tf, cfg["A"], cfg["A"], cfg["C"])
+    assert np.array_equal(got, want)
+    f64 = cfg["A"].astype(np.float64) @ (cfg["A"].astype(np.float64) @ cfg["C"].astype(np.float64))
+    assert orc.rel_err(got, f64) <= TOL
+
+
+def test_spmm_spmm_two_matrices_rectangular_unsorted_empty(gpu, tf, orc):
+    """A != B, B rectangular, A with unsorted columns and empty rows."""
+    say("spmm_spmm A != B rectangular")
+    rng = np.random.default_rng(40)
+    L, M, Kc, N = 900, 700, 500, 64
+    A = sp.random(L, M, density=0.01, format="csr", random_state=rng, dtype=np.float32)
+    A.data = rng.uniform(-1, 1, A.nnz).astype(np.float32)
+    lil = A.tolil()
+    for i in range(0, L, 9):
+        lil.rows[i], lil.data[i] = [], []
+    A = sp.csr_matrix(lil, dtype=np.float32)
+    for i in range(L):  # scramble column order inside rows
+        s, e = A.indptr[i], A.indptr[i + 1]
+        p = rng.permutation(e - s)
+        A.indices[s:e], A.data[s:e] = A.indices[s:e][p], A.data[s:e][p]
+    B = sp.random(M, Kc, density=0.02, format="csr", random_state=rng, dtype=np.float32)
+    B.data = rng.uniform(-1, 1, B.nnz).astype(np.float32)
+    Cd = rng.uniform(-1, 1, (Kc, N)).astype(np.float32)
+    want = orc.spmm_spmm(A, B, Cd, _two_level(L, M, orc))[0]
+    got, _ = run_spmm_spmm(tf, A, B, Cd)
+    assert np.array_equal(got, want)
+
+
+def test_spmm_spmm_accumulate(gpu, tf, orc):
+    say("spmm_spmm accumulate")
+    A = tf.workloads.laplacian_2d(40)
+    Cd = tf.workloads.uniform((1600, 64), 41)
+    D0 = tf.workloads.uniform((1600, 64), 42)
+    base = oracle_spmm_spmm(orc, A, A, Cd)
+    for kw in (dict(), dict(max_redundancy=1.0, tile_rows=128)):
+        got, _ = run_spmm_spmm(tf, A, A, Cd, accumulate=True, D0=D0, **kw)
+        assert orc.rel_err(got, D0.astype(np.float64) + base) <= 1e-6
+        got0, _ = run_spmm_spmm(tf, A, A, Cd, accumulate=True, D0=np.zeros_like(D0), **kw)
+        assert np.array_equal(got0, base)  # zeroed D, the reference's calling convention
+
+
+def test_spmm_spmm_long_rows(gpu, tf, orc):
+    """Hub rows longer than long_row_nnz are cut into chunks and tree-reduced."""
+    say("spmm_spmm long rows")
+    rng = np.random.default_rng(43)
+    M, N = 6000, 128
+    A = tf.workloads.banded_random(M, 32, 16, seed=44).tolil()
+    for hub, deg in ((17, 5000), (3000, 2100), (5999, 700)):
+        cols = np.sort(rng.choice(M, deg, replace=False))
+        A.rows[hub] = cols.tolist()
+        A.data[hub] = rng.uniform(-1, 1, deg).astype(np.float32).tolist()
+    A = sp.csr_matrix(A, dtype=np.float32)
+    Cd = tf.workloads.uniform((M, N), 45)
+    want = A.astype(np.float64) @ (A.astype(np.float64) @ Cd.astype(np.float64))
+    got, info = run_spmm_spmm(tf, A, A, Cd, long_row_nnz=512)
+    assert info["n_long_rows"] == 3 and info["n_long_chunks"] == 10 + 5 + 2
+    assert orc.rel_err(got, want) <= TOL
+    ok = np.ones(M, bool)
+    ok[[17, 3000, 5999]] = False
+    assert np.array_equal(got[ok], oracle_spmm_spmm(orc, A, A, Cd)[ok])  # unsplit rows stay bit-exact
+
+
+def test_laplacian_all_ones_exact_full_size(gpu, tf):
+    """The 128^3 Laplacian with an all-ones dense operand (the reference's own input,
+    fusion/example/SpMM_SpMM_Demo_Utils.h:53-59): integers throughout, so D must equal the
+    7-point stencil applied twice on the grid, exactly, at the benchmark's full size."""
+    say("spmm_spmm 3D Laplacian 128^3 all ones")
+    g, N = 128, 64
+    A = tf.workloads.laplacian_3d(g)
+    ones = np.ones((g ** 3, N), np.float32)
+    got, info = run_spmm_spmm(tf, A, A, ones)
+
+    def st(u):
+        out = 6.0 * u
+        out[:, :, 1:] -= u[:, :, :-1]; out[:, :, :-1] -= u[:, :, 1:]
+        out[:, 1:, :] -= u[:, :-1, :]; out[:, :-1, :] -= u[:, 1:, :]
+        out[1:, :, :] -= u[:-1, :, :]; out[:-1, :, :] -= u[1:, :, :]
+        return out
+    want = st(st(np.ones((g, g, g), np.float32))).reshape(-1)
+    assert np.array_equal(got, np.repeat(want[:, None], N, axis=1))
+
+
+def test_full_size_banded_linearity_and_roundtrip(gpu, tf, orc):
+    """Benchmark size (65,536 rows, N = 128): bit-exact against the oracle, and linear in C."""
+    say("spmm_spmm cfg2 full size")
+    cfg = tf.workloads.make_config(2)
+    A, Cd = cfg["A"], cfg["C"]
+    got, info = run_spmm_spmm(tf, A, A, Cd)
+    assert info["n_fused_rows"] == A.shape[0]
+    assert np.array_equal(got, oracle_spmm_spmm(orc, A, A, Cd))
+    C2 = tf.workloads.uniform(Cd.shape, 99)
+    g2, _ = run_spmm_spmm(tf, A, A, C2)
+    g12, _ = run_spmm_spmm(tf, A, A, Cd + C2)
+    assert orc.rel_err(g12, got.astype(np.float64) + g2) <= 1e-5
+
+
+# ---- GeMM-SpMM ----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("K,N", [(64, 64), (128, 128), (256, 128), (8, 32), (72, 96), (40, 256), (512, 64)])
+def test_gemm_spmm_shapes(gpu, tf, orc, K, N):
+    say(f"gemm_spmm K={K} N={N}")
+    n = 36
+    A = tf.workloads.laplacian_2d(n)
+    M = n * n
+    rng = np.random.default_rng(50 + K + N)
+    B = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    Cd = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    want, _ = orc.gemm_spmm(A, B, Cd, orc.unfused_schedule(M), nthreads=8)
+    for kw in (dict(), dict(tile_rows=160, max_redundancy=2.0, lds_budget_bytes=163840), dict(max_redundancy=1.0, tile_rows=96)):
+        got, info = run_gemm_spmm(tf, A, B, Cd, **kw)
+        assert orc.rel_err(got, want) <= TOL, (K, N, kw)
+    Bi = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    Ci = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    exact = (A.astype(np.int64) @ (Bi.astype(np.int64) @ Ci.astype(np.int64))).astype(np.float32)
+    got, info = run_gemm_spmm(tf, A, Bi, Ci, tile_rows=160, max_redundancy=2.0, lds_budget_bytes=163840)
+    assert info["n_fused_rows"] > 0
+    assert np.array_equal(got, exact)  # integer operands: exact whatever the summation order
+
+
+@pytest.mark.parametrize("idx,scale", [(1, 1.0), (3, 0.02), (4, 2.0 ** -6)])
+def test_gemm_spmm_configs(gpu, tf, orc, idx, scale):
+    cfg = tf.workloads.make_config(idx, scale)
+    say(f"gemm_spmm {cfg['name']} scale={scale} rows={cfg['A'].shape[0]}")
+    A = cfg["A"]
+    want, _ = orc.gemm_spmm(A, cfg["B"], cfg["C"], orc.unfused_schedule(A.shape[0]), nthreads=8)
+    got, info = run_gemm_spmm(tf, A, cfg["B"], cfg["C"])
+    assert orc.rel_err(got, want) <= TOL
+    if idx == 4:
+        assert info["n_long_rows"] >= 1
+
+
+def test_gemm_spmm_reductions_and_accumulate(gpu, tf, orc):
+    say("gemm_spmm reductions")
+    M, K, N = 1000, 64, 64
+    rng = np.random.default_rng(60)
+    B = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    Cd = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    eye = sp.identity(M, format="csr", dtype=np.float32)
+    got, info = run_gemm_spmm(tf, eye, B, Cd)  # A = I: D = B*C, every row fused
+    assert info["n_fused_rows"] == M
+    assert orc.rel_err(got, B.astype(np.float64) @ Cd.astype(np.float64)) <= 1e-6
+    A = tf.workloads.banded_random(M, 32, 16, seed=61)
+    got, _ = run_gemm_spmm(tf, A, B, np.eye(K, dtype=np.float32))  # C = I: D = A*B exactly
+    assert np.array_equal(got, orc.spmm(A, B))
+    D0 = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    base, _ = run_gemm_spmm(tf, A, B, Cd)
+    acc, _ = run_gemm_spmm(tf, A, B, Cd, accumulate=True, D0=D0)
+    assert orc.rel_err(acc, D0.astype(np.float64) + base) <= 1e-6
+
+
+def test_power_law_row_sums_full_size(gpu, tf):
+    """2^21-node R-MAT, row-normalised: with all-ones B (M x 128) and C (128 x 128) the
+    intermediate is 128 everywhere, so D is 128 on every non-empty row and 0 on empty ones."""
+    say("gemm_spmm R-MAT 2^21 all ones")
+    cfg = tf.workloads.make_config(4)
+    A = cfg["A"]
+    M = A.shape[0]
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128)
+    S.validate()
+    B = tf.DenseMatrix(M, 128); B.fill(1.0)
+    Cm = tf.DenseMatrix(128, 128); Cm.fill(1.0)
+    D = tf.DenseMatrix(M, 128); D.fill(float("nan"))
+    tf.gemm_spmm(Ah, B, Cm, D, S)
+    tf.device_synchronize()
+    got = D.to_numpy()
+    empty = np.diff(A.indptr) == 0
+    assert np.all(got[empty] == 0.0)
+    rs = np.asarray(A.astype(np.float64).sum(axis=1)).ravel()
+    assert np.abs(got[~empty] - 128.0 * rs[~empty][:, None]).max() <= 128.0 * TOL
+    assert np.abs(got[~empty] - 128.0).max() <= 128.0 * TOL
+
+
+# ---- building blocks, the C++ API, error behaviour ---------------------------------------
+
+def test_unfused_building_blocks(gpu, tf, orc):
+    say("tf_spmm / tf_gemm")
+    A = tf.workloads.banded_random(2000, 64, 9, seed=70)
+    X = tf.workloads.uniform((2000, 96), 71)
+    Y = tf.DenseMatrix(2000, 96)
+    tf.spmm(tf.CsrMatrix.from_scipy(A), tf.DenseMatrix.from_numpy(X), Y)
+    assert np.array_equal(Y.to_numpy(), orc.spmm(A, X))
+    W = tf.workloads.uniform((96, 64), 72)
+    Z = tf.DenseMatrix(2000, 64)
+    tf.gemm(tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W), Z)
+    assert orc.rel_err(Z.to_numpy(), X.astype(np.float64) @ W.astype(np.float64)) <= 1e-6
+
+
+def test_cpp_readme_api(gpu):
+    say("C++ README API program")
+    exe = os.path.join(ROOT, "tests", "cpp", "api_check")
+    assert os.path.exists(exe), "tests/cpp/api_check is not built (run build())"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "api_check ok" in r.stdout, r.stdout + r.stderr
+
+
+def test_error_behaviour(gpu, tf):
+    say("error paths")
+    A = tf.workloads.banded_random(512, 32, 16, seed=80)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64)
+    Cd = tf.DenseMatrix(512, 64); Cd.fill(1.0)
+    D = tf.DenseMatrix(512, 64)
+    with pytest.raises(tf.TileFusionError) as e:  # schedule built for another N
+        tf.spmm_spmm(Ah, Ah, tf.DenseMatrix(512, 32), tf.DenseMatrix(512, 32), S)
+    assert e.value.status == -4
+    with pytest.raises(tf.TileFusionError) as e:  # schedule built for the other operation
+        tf.gemm_spmm(Ah, Cd, tf.DenseMatrix(64, 64), D, S)
+    assert e.value.status == -4
+    other = tf.CsrMatrix.from_scipy(tf.workloads.laplacian_2d(16))
+    with pytest.raises(tf.TileFusionError) as e:  # schedule built for another pattern
+        tf.spmm_spmm(other, other, tf.DenseMatrix(256, 64), tf.DenseMatrix(256, 64), S)
+    assert e.value.status == -4
+    with pytest.raises(tf.TileFusionError) as e:  # D with the wrong row count
+        tf.spmm_spmm(Ah, Ah, Cd, tf.DenseMatrix(100, 64), S)
+    assert e.value.status == -1
+    tf.spmm_spmm(Ah, Ah, Cd, D, S)  # and the handle is still usable afterwards
+    tf.device_synchronize()
+    assert np.isfinite(D.to_numpy()).all()
+
+
+def test_streams_and_wrapped_buffers(gpu, tf, orc):
+    """A caller-provided stream and a dense operand wrapped around foreign device memory."""
+    say("streams / wrapped device pointers")
+    A = tf.workloads.banded_random(1024, 32, 16, seed=81)
+    Cd = tf.workloads.uniform((1024, 128), 82)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128)
+    owner = tf.DenseMatrix(1024, 128)
+    D = tf.DenseMatrix.wrap_device(1024, 128, owner.device_ptr())
+    st = tf.Stream()
+    e0, e1 = tf.Event(), tf.Event()
+    e0.record(st)
+    tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(Cd), D, S, stream=st)
+    e1.record(st)
+    e1.synchronize()
+    assert e0.elapsed_ms(e1) > 0.0
+    assert np.array_equal(owner.to_numpy(), oracle_spmm_spmm(orc, A, A, Cd))

@@ -1,0 +1,172 @@
+"""The gfx950 inspector (tf_inspect) on the CPU: schedules are checked exactly by an
+independent validator written here, by the library's own validator, and against
+hand-derived fused sets on banded and stencil patterns."""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+
+def validate(view, info, A, lds_budget):
+    """Independent of the library: every first-op row owned once, every second-op row
+    scheduled once, fused rows read only rows their tile computes, remainder rows read
+    only rows some tile writes back, slabs fit the LDS budget."""
+    L, M = A.shape
+    tr, wb = view["tile_range"], view["writeback"]
+    nt = len(tr)
+    assert view["n1_"] == 2 and view["ptr1_"][0] == 0 and view["ptr1_"][1] == nt
+    P = view["ptr1_"][2]
+    ptr2, kb, ids, typ = view["ptr2_"], view["ker_begin_"], view["id_"], view["type_"]
+    assert len(ptr2) == P + 1 and ptr2[0] == 0 and ptr2[P] == len(ids) == M + L
+    assert np.array_equal(np.sort(ids[typ == 0]), np.arange(M))
+    assert np.array_equal(np.sort(ids[typ == 1]), np.arange(L))
+    stored = np.zeros(M, bool)
+    fused_rows = 0
+    end = 0
+    for t in range(nt):
+        pb, pe, ob, oe = tr[t]
+        assert ob == end and oe > ob and pb <= ob and pe >= oe and 0 <= pb and pe <= M
+        end = oe
+        own = ids[ptr2[t]:kb[2 * t]]
+        fused = ids[kb[2 * t]:kb[2 * t + 1]]
+        assert kb[2 * t + 1] == ptr2[t + 1]
+        assert np.array_equal(own, np.arange(ob, oe))
+        assert np.all(typ[ptr2[t]:kb[2 * t]] == 0) and np.all(typ[kb[2 * t]:kb[2 * t + 1]] == 1)
+        if len(fused):
+            assert (pe - pb) * info["N"] * 4 <= lds_budget
+        for i in fused:
+            cols = A.indices[A.indptr[i]:A.indptr[i + 1]]
+            if len(cols):
+                assert cols.min() >= pb and cols.max() < pe, f"fused row {i} leaves tile {t}"
+        fused_rows += len(fused)
+        assert ob <= wb[t][0] <= wb[t][1] <= oe
+        stored[wb[t][0]:wb[t][1]] = True
+    assert end == M
+    assert fused_rows == info["n_fused_rows"] and fused_rows + info["n_remainder_rows"] == L
+    for p in range(nt, P):
+        rows = ids[ptr2[p]:ptr2[p + 1]]
+        assert 0 < len(rows) <= 64 and kb[2 * p] == ptr2[p] and kb[2 * p + 1] == ptr2[p + 1]
+        for i in rows:
+            cols = A.indices[A.indptr[i]:A.indptr[i + 1]]
+            assert np.all(stored[cols]), f"remainder row {i} reads a row nobody stores"
+    assert info["n_writeback_rows"] == int(sum(b - a for a, b in wb))
+
+
+def inspect(tf, A, **kw):
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, **kw)
+    S.validate()
+    return S, S.view(), S.info()
+
+
+@pytest.mark.parametrize("idx,scale", [(1, 1.0), (2, 0.1), (3, 0.02), (4, 2.0 ** -7), (5, 0.004)])
+def test_configs_validate(tf, idx, scale):
+    cfg = tf.workloads.make_config(idx, scale)
+    op = tf.OP_GEMM_SPMM if cfg["op"] == "gemm_spmm" else tf.OP_SPMM_SPMM
+    for budget in (32768, 65536, 163840):
+        S, view, info = inspect(tf, cfg["A"], op=op, N=cfg["N"], K=cfg["K"], lds_budget_bytes=budget)
+        validate(view, info, cfg["A"], budget)
+
+
+def test_banded_halo_fuses_everything(tf):
+    """Half-bandwidth 16: with recomputation every row fuses and nothing is written back;
+    each tile computes its owned rows plus at most 16 halo rows per side."""
+    A = tf.workloads.banded_random(4096, 32, 16, seed=3)
+    S, view, info = inspect(tf, A, op=tf.OP_SPMM_SPMM, N=128, lds_budget_bytes=65536)
+    validate(view, info, A, 65536)
+    assert info["n_fused_rows"] == 4096 and info["n_remainder_rows"] == 0 and info["n_writeback_rows"] == 0
+    tr = view["tile_range"]
+    assert np.all(tr[:, 2] - tr[:, 0] <= 16) and np.all(tr[:, 1] - tr[:, 3] <= 16)
+    assert np.all(tr[:, 1] - tr[:, 0] <= 65536 // (128 * 4))
+
+
+def test_no_recomputation_matches_reference_rule(tf):
+    """max_redundancy = 1 is the reference's tiling: a row fuses iff all its columns are
+    rows of its own tile (Fusion_Inspector.h:885-891, without the sorted-columns shortcut)."""
+    n = 32
+    A = tf.workloads.laplacian_2d(n)
+    S, view, info = inspect(tf, A, op=tf.OP_SPMM_SPMM, N=64, lds_budget_bytes=65536, tile_rows=256, max_redundancy=1.0)
+    validate(view, info, A, 65536)
+    tr = view["tile_range"]
+    assert np.array_equal(tr[:, 0], tr[:, 2]) and np.array_equal(tr[:, 1], tr[:, 3])
+    assert np.all(tr[:, 3] - tr[:, 2] == 256)
+    ids, kb = view["id_"], view["ker_begin_"]
+    M = n * n
+    for t, (s, e, _, _) in enumerate(tr):
+        want = [i for i in range(s, e) if (i - n < 0 or i - n >= s) and (i + n >= M or i + n < e)
+                and (i % n == 0 or i - 1 >= s) and (i % n == n - 1 or i + 1 < e)]
+        assert ids[kb[2 * t]:kb[2 * t + 1]].tolist() == want
+    # remainder rows = n rows either side of every interior boundary -> their reads force write-back
+    assert info["n_remainder_rows"] == 2 * n * (len(tr) - 1)
+    assert info["n_writeback_rows"] > 0
+
+
+def test_unsorted_columns_and_empty_rows(tf):
+    """Columns in any order, rows without entries, and a row that reaches across the
+    matrix (never fusable) are all scheduled exactly once."""
+    rng = np.random.default_rng(0)
+    M = 700
+    rows, cols = [], []
+    for i in range(M):
+        if i % 7 == 3:
+            continue
+        c = np.unique(np.clip(i + rng.integers(-5, 6, 4), 0, M - 1))
+        rng.shuffle(c)
+        rows += [i] * len(c)
+        cols += c.tolist()
+    rows += [350, 350]
+    cols += [0, M - 1]
+    A = sp.csr_matrix((np.ones(len(rows), np.float32), (rows, cols)), shape=(M, M))
+    A.has_sorted_indices = False
+    perm_A = A.copy()
+    for i in range(M):  # scramble each row's column order
+        s, e = perm_A.indptr[i], perm_A.indptr[i + 1]
+        p = rng.permutation(e - s)
+        perm_A.indices[s:e] = perm_A.indices[s:e][p]
+    S, view, info = inspect(tf, perm_A, op=tf.OP_SPMM_SPMM, N=32, lds_budget_bytes=16384)
+    validate(view, info, perm_A, 16384)
+    assert 350 in view["id_"][view["ptr2_"][view["ptr1_"][1]]:]  # the far-reaching row is a remainder row
+    assert info["n_remainder_rows"] >= 1
+
+
+def test_long_rows_are_chunked(tf):
+    M = 4096
+    hub = sp.csr_matrix((np.ones(3000, np.float32), (np.zeros(3000, int), np.arange(3000))), shape=(M, M))
+    A = sp.csr_matrix(hub + sp.identity(M, dtype=np.float32, format="csr"))
+    S, view, info = inspect(tf, A, op=tf.OP_SPMM_SPMM, N=64, long_row_nnz=512)
+    validate(view, info, A, 65536)
+    assert info["n_long_rows"] == 1 and info["n_long_chunks"] == 6  # ceil(3000 / 512)
+
+
+def test_rectangular_and_bad_arguments(tf):
+    A = sp.random(300, 200, density=0.02, format="csr", random_state=np.random.default_rng(1), dtype=np.float32)
+    S, view, info = inspect(tf, A, op=tf.OP_SPMM_SPMM, N=16)
+    validate(view, info, A, 65536)
+    A2 = sp.random(200, 300, density=0.02, format="csr", random_state=np.random.default_rng(2), dtype=np.float32)
+    S, view, info = inspect(tf, A2, op=tf.OP_SPMM_SPMM, N=16)
+    validate(view, info, A2, 65536)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    for kw in (dict(op=7, N=16), dict(op=tf.OP_SPMM_SPMM, N=0), dict(op=tf.OP_GEMM_SPMM, N=64, K=0),
+               dict(op=tf.OP_SPMM_SPMM, N=16, lds_budget_bytes=1 << 20), dict(op=tf.OP_SPMM_SPMM, N=4096, lds_budget_bytes=16384)):
+        with pytest.raises(tf.TileFusionError) as e:
+            tf.inspector(Ah, 1, **kw)
+        assert e.value.status == -1
+    with pytest.raises(tf.TileFusionError) as e:
+        tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=48, K=64)
+    assert e.value.status == -5
+    bad = tf.CsrMatrix(4, 4, [0, 1, 2, 3, 4], [0, 1, 9, 3], [1, 1, 1, 1])
+    with pytest.raises(tf.TileFusionError):
+        tf.inspector(bad, 1, op=tf.OP_SPMM_SPMM, N=8)
+
+
+def test_validator_rejects_a_schedule_for_another_pattern(tf):
+    A = tf.workloads.banded_random(1024, 32, 16, seed=1)
+    B = tf.workloads.laplacian_2d(32)
+    S = tf.inspector(tf.CsrMatrix.from_scipy(A), 1, op=tf.OP_SPMM_SPMM, N=64)
+    with pytest.raises(tf.TileFusionError) as e:
+        S.validate(tf.CsrMatrix.from_scipy(B))
+    assert e.value.status == -4
+    A2 = A.copy()
+    A2.indices[A2.indptr[500]] = 0  # same size, one dependence moved far away
+    with pytest.raises(tf.TileFusionError) as e:
+        S.validate(tf.CsrMatrix.from_scipy(A2))
+    assert e.value.status == -4 and "row 500" in str(e.value)

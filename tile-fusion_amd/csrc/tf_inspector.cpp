@@ -62,7 +62,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   // LDS the tile GEMM needs for staging C, before any slab row.
   int gemm_kc = 0, staging = 0;
   if (o.op == TF_OP_GEMM_SPMM) {
-    gemm_kc = std::min(o.K, std::max(8, (32768 / (4 * o.N)) / 8 * 8));
+    const int stage_cap = std::min(32768, o.lds_budget_bytes / 2);
+    gemm_kc = std::min(o.K, std::max(8, (stage_cap / (4 * o.N)) / 8 * 8));
     staging = gemm_kc * o.N * 4;
   }
   const int row_bytes = o.N * 4;
