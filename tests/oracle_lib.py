@@ -122,10 +122,6 @@ def inspect_fixed_tiles(A, iter_per_partition, num_threads):
     return Schedule.from_struct(s)
 
 
-def _unused():
-    pass
-
-
 def unfused_schedule(M, rows_per_part=64):
     """Two levels without any fusion: level 0 = all first-op rows, level 1 = all second-op rows."""
     nparts = (M + rows_per_part - 1) // rows_per_part
