@@ -81,6 +81,8 @@ def main():
     ap.add_argument("--lds", type=int, default=0, help="LDS budget per tile in bytes (0 = library default)")
     ap.add_argument("--tile-rows", type=int, default=0)
     ap.add_argument("--max-redundancy", type=float, default=0.0)
+    ap.add_argument("--strip", type=int, default=0, help="columns per strip of windowed tiles (32 or 64)")
+    ap.add_argument("--no-window", action="store_true", help="do not build windowed tiles")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the result check")
     args = ap.parse_args()
@@ -98,8 +100,9 @@ def main():
 
     Ah = tf.CsrMatrix.from_scipy(A).to_device()
     t0 = time.perf_counter()
+    inner = Ah if (op == tf.OP_SPMM_SPMM and cfg["B"] is A and not args.no_window) else None
     S = tf.inspector(Ah, 1, op=op, N=N, K=K, lds_budget_bytes=args.lds, tile_rows=args.tile_rows,
-                     max_redundancy=args.max_redundancy)
+                     max_redundancy=args.max_redundancy, inner=inner, strip_cols=args.strip)
     inspect_s = time.perf_counter() - t0
     S.validate()
     info = S.info()
@@ -153,14 +156,15 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": cfg["name"], "op": cfg["op"], "rows": int(A.shape[0]), "nnz": int(A.nnz), "N": N, "K": K,
-                   "lds_budget_bytes": info["lds_bytes"], "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
+                   "lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
                    "remainder_rows": info["n_remainder_rows"], "recomputed_rows": info["n_producer_rows"] - A.shape[1],
                    "writeback_rows": info["n_writeback_rows"], "kernels_per_step": n_kernels,
                    "inspector_s": round(inspect_s, 4), "rel_err_vs_f64": check, "device": dev["arch"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes": int(alg_bytes), "kernel_ms": round(dev_ms, 5),
-                     "kernel": "fused_spmm_spmm_kernel" if op == tf.OP_SPMM_SPMM else "fused_gemm_spmm_kernel",
+                     "kernel": ("fused_spmm_spmm_window_kernel" if info["windowed"] else "fused_spmm_spmm_kernel")
+                     if op == tf.OP_SPMM_SPMM else "fused_gemm_spmm_kernel",
                      "note": "kernel_ms = HIP-event time on the launch stream / steps (all kernels of a step)"},
     }
     if op == tf.OP_GEMM_SPMM:

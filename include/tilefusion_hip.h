@@ -105,7 +105,8 @@ typedef struct {
   int K;                 /* GeMM-SpMM: columns of dense B = rows of C (FeatureDim); else 0   */
   int lds_budget_bytes;  /* LDS one fused tile may take; plays the role of the cache budget
                             ScheduleParameters::TileM of the reference's variable-tile
-                            inspector.  Default 65536, max 163840.                            */
+                            inspector.  Default 65536 (81920 when an inner pattern is
+                            given), max 163840.                                               */
   int tile_rows;         /* cap on the rows a tile owns; default: sized so that the launch
                             has about four tiles per compute unit                             */
   float max_redundancy;  /* a tile may compute up to this many intermediate rows per owned
@@ -115,6 +116,16 @@ typedef struct {
   int long_row_nnz;      /* remainder rows with more stored entries than this are split into
                             chunks reduced by a wavefront-level tree; default 2048           */
   int compute_units;     /* sizing hint; default: the current device, or 256 with no device  */
+  /* SpMM-SpMM only, optional: sparsity pattern of the inner matrix B (M x inner_cols, host
+     arrays).  In every run of the reference B is A (fusion/example/SpMM_SpMM_Demo_Utils.h:
+     53-54); pass A's arrays again for that case.  With it the inspector can tell when the rows
+     of C a tile reads form a small contiguous window and then stages that window in LDS
+     ("windowed" tiles: both products run out of LDS).  Null = unknown, C is gathered from HBM. */
+  const int *inner_Ap;
+  const int *inner_Ai;
+  int inner_cols;
+  int strip_cols;        /* windowed tiles work on this many columns of C/D at a time (32 or 64);
+                            default 32                                                         */
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -144,6 +155,8 @@ typedef struct {
   int n_writeback_rows;  /* intermediate rows that are written to HBM               */
   int max_tile_producer_rows;
   int lds_bytes;         /* dynamic LDS of the fused-tile kernel                    */
+  int windowed;          /* 1 when tiles stage their window of C in LDS             */
+  int strip_cols;        /* columns per strip of the windowed kernel, else 0        */
   long long fused_nnz;   /* stored entries of A in fused rows (getFusedNnzNum)      */
   long long workspace_bytes; /* device memory the executor keeps (intermediate + partials) */
 } tf_schedule_info;

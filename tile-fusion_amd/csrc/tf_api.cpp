@@ -31,6 +31,7 @@ struct DeviceSchedule {
   int device = -1;
   TileDesc *tiles = nullptr;
   int *fused_ids = nullptr;
+  int *win = nullptr;
   int *rem_rows = nullptr;
   LongChunk *long_chunks = nullptr;
   LongRow *long_rows = nullptr;
@@ -42,6 +43,9 @@ struct DeviceSchedule {
 hipError_t launch_fused_spmm_spmm(const TileDesc *, int, const int *, const int *, const int *,
                                   const float *, const float *, const int *, const int *,
                                   const float *, float *, float *, int, int, int, hipStream_t);
+hipError_t launch_fused_spmm_spmm_window(const TileDesc *, const int *, int, const int *, const int *,
+                                         const int *, const float *, const float *, float *, int, int,
+                                         int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
                             float *, int, int, hipStream_t);
 hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const int *, const float *,
@@ -83,7 +87,7 @@ int default_compute_units() {
 
 void release_device_schedule(DeviceSchedule *d) {
   if (!d) return;
-  (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->rem_rows);
+  (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows);
   (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows);
   (void)hipFree(d->inter); (void)hipFree(d->partial);
   delete d;
@@ -113,6 +117,7 @@ static tf_status ensure_device(tf_schedule *s) {
   d->device = dev;
   tf_status rc = upload_vec(s->tiles, &d->tiles);
   if (!rc) rc = upload_vec(s->fused_ids, &d->fused_ids);
+  if (!rc) rc = upload_vec(s->win, &d->win);
   if (!rc) rc = upload_vec(s->rem_rows, &d->rem_rows);
   if (!rc) rc = upload_vec(s->long_chunks, &d->long_chunks);
   if (!rc) rc = upload_vec(s->long_rows, &d->long_rows);
@@ -359,9 +364,24 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
   const tf::DeviceSchedule *d = s->dev;
+  if (s->windowed) {
+    if (B->nnz != s->inner_nnz || B->N != s->opts.inner_cols)
+      return fail(TF_ESCHEDULE, "tf_spmm_spmm: schedule was built for an inner pattern with %lld entries and %d columns, B has %d and %d",
+                  s->inner_nnz, s->opts.inner_cols, B->nnz, B->N);
+    // The windowed kernel walks one staged CSR chunk for both products: B must be A.
+    const bool same = (B == A) || (B->p == A->p && B->i == A->i && B->x == A->x);
+    if (same) {
+      TF_HIP(tf::launch_fused_spmm_spmm_window(d->tiles, d->win, (int)s->tiles.size(), d->fused_ids, A->p,
+                                               A->i, A->x, C->d, D->d, s->opts.N, s->opts.strip_cols,
+                                               s->lds_bytes, acc, st));
+      return TF_OK;
+    }
+    if (s->lds_bytes_general > 163840)
+      return fail(TF_ESCHEDULE, "tf_spmm_spmm: this schedule needs B to be the same matrix as A");
+  }
   TF_HIP(tf::launch_fused_spmm_spmm(d->tiles, (int)s->tiles.size(), d->fused_ids, B->p, B->i, B->x,
                                     C->d, A->p, A->i, A->x, D->d, d->inter, s->opts.N,
-                                    s->lds_bytes, acc, st));
+                                    s->windowed ? s->lds_bytes_general : s->lds_bytes, acc, st));
   return tf::run_remainder(A, D, s, acc, st);
 }
 

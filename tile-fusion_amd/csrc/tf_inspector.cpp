@@ -51,7 +51,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   } else {
     o.K = 0;
   }
-  if (o.lds_budget_bytes <= 0) o.lds_budget_bytes = 65536;
+  const bool has_inner = o.op == TF_OP_SPMM_SPMM && o.inner_Ap != nullptr;
+  if (o.lds_budget_bytes <= 0) o.lds_budget_bytes = has_inner ? 81920 : 65536;  // two workgroups per CU either way
   if (o.lds_budget_bytes > kMaxLds)
     return tf::fail(TF_EINVAL, "tf_inspect: lds_budget_bytes %d exceeds %d", o.lds_budget_bytes, kMaxLds);
   if (o.max_redundancy <= 0.f) o.max_redundancy = (o.op == TF_OP_GEMM_SPMM) ? 1.5f : 3.0f;
@@ -71,6 +72,11 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   if (p_max < 8)
     return tf::fail(TF_EINVAL, "tf_inspect: LDS budget %d holds only %d intermediate rows of N=%d",
                     o.lds_budget_bytes, p_max, o.N);
+  if (o.strip_cols <= 0) o.strip_cols = 32;
+  if (o.strip_cols != 32 && o.strip_cols != 64)
+    return tf::fail(TF_EINVAL, "tf_inspect: strip_cols must be 32 or 64");
+  const bool want_window = o.op == TF_OP_SPMM_SPMM && o.inner_Ap && (o.inner_Ai || o.inner_Ap[M] == 0) &&
+                           o.inner_cols > 0 && o.N % o.strip_cols == 0;
   int r_cap = o.tile_rows > 0 ? o.tile_rows : ceil_div(M, 2 * o.compute_units);
   if (o.op == TF_OP_GEMM_SPMM) r_cap = ceil_div(r_cap, 32) * 32;
   r_cap = std::max(r_cap, o.tile_rows > 0 ? 1 : 32);
@@ -81,6 +87,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   if (!S) return tf::fail(TF_ENOMEM, "tf_inspect: out of host memory");
   try {
     S->opts = o;
+    S->opts.inner_Ap = nullptr;  // the caller's arrays are not kept
+    S->opts.inner_Ai = nullptr;
     S->L = L;
     S->M = M;
     S->nnz = nnz;
@@ -103,14 +111,88 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       lo[i] = a;
       hi[i] = b + 1;
     }
+    std::vector<char> fused(L, 0);
+
+    // ---- windowed tiles (SpMM-SpMM with a known inner pattern) -------------------------
+    // Every row must fuse, and the rows of C that a tile's producer rows read must form a
+    // window small enough to sit in LDS next to the slab, one strip of columns at a time.
+    bool windowed = false;
+    if (want_window) {
+      const int *Bp = o.inner_Ap, *Bi = o.inner_Ai;
+      const int SW = o.strip_cols;
+      std::vector<int> blo(M), bhi(M);
+      bool ok = (Bp[0] == 0);
+      for (int r = 0; r < M && ok; ++r) {
+        int a = INT_MAX, b = -1;
+        if (Bp[r + 1] < Bp[r]) { ok = false; break; }
+        for (int k = Bp[r]; k < Bp[r + 1]; ++k) {
+          const int c = Bi[k];
+          if (c < 0 || c >= o.inner_cols) { ok = false; break; }
+          a = std::min(a, c);
+          b = std::max(b, c);
+        }
+        blo[r] = a;      // INT_MAX / 0 for an empty row: no constraint
+        bhi[r] = b + 1;
+      }
+      auto a16 = [](long long x) { return (x + 15) / 16 * 16; };
+      auto lds_of = [&](int P, int R, long long nz, int Wc) {
+        return a16(4LL * (P + 1)) + a16(4LL * R) + a16(8LL * (nz + 2LL * P)) + 4LL * SW * ((long long)Wc + P);  // 2 = pad slots per staged row
+      };
+      std::vector<tf::TileDesc> tiles;
+      std::vector<int> ids, win;
+      long long prod_rows = 0;
+      int lds_max = 0, slab = 0;
+      int s = 0;
+      while (ok && s < M) {
+        int wlo = s, whi = s, clo = INT_MAX, chi = 0, e = s;
+        while (e < M && e - s < r_cap) {
+          int nlo = std::min(wlo, e), nhi = std::max(whi, e + 1);
+          if (e < L) { nlo = std::min(nlo, lo[e]); nhi = std::max(nhi, hi[e]); }
+          int nclo = clo, nchi = chi;
+          for (int r = nlo; r < wlo; ++r) { nclo = std::min(nclo, blo[r]); nchi = std::max(nchi, bhi[r]); }
+          for (int r = std::max(whi, nlo); r < nhi; ++r) { nclo = std::min(nclo, blo[r]); nchi = std::max(nchi, bhi[r]); }
+          const int Wc = nchi > nclo ? nchi - nclo : 0;
+          if (lds_of(nhi - nlo, e + 1 - s, (long long)Bp[nhi] - Bp[nlo], Wc) > o.lds_budget_bytes) break;
+          wlo = nlo; whi = nhi; clo = nclo; chi = nchi; ++e;
+        }
+        if (e == s || (e - s < std::min(r_cap, 16) && e != M) ||
+            (float)(whi - wlo) > o.max_redundancy * (float)(e - s)) { ok = false; break; }
+        tf::TileDesc t{};
+        t.own_begin = s; t.own_end = e; t.prod_begin = wlo; t.prod_end = whi;
+        t.wb_begin = t.wb_end = s;
+        t.cons_begin = (int)ids.size();
+        for (int i = s; i < e && i < L; ++i) ids.push_back(i);
+        t.cons_end = (int)ids.size();
+        if (chi <= clo) { clo = 0; chi = 0; }
+        win.push_back(clo); win.push_back(chi);
+        lds_max = std::max<long long>(lds_max, lds_of(whi - wlo, e - s, (long long)Bp[whi] - Bp[wlo], chi - clo));
+        slab = std::max(slab, whi - wlo);
+        prod_rows += whi - wlo;
+        tiles.push_back(t);
+        s = e;
+      }
+      if (ok && L <= M) {
+        windowed = true;
+        S->inner_nnz = Bp[M];
+        S->tiles.swap(tiles);
+        S->fused_ids.swap(ids);
+        S->win.swap(win);
+        S->n_producer_rows = prod_rows;
+        S->slab_rows = slab;
+        S->lds_bytes = lds_max;
+        std::fill(fused.begin(), fused.end(), 1);
+      }
+    }
+    S->windowed = windowed;
+    if (!windowed) S->opts.strip_cols = 0;
+
     // A row whose own reach (itself plus its columns) exceeds the slab can never fuse.
     auto reach_lo = [&](int i) { return std::min(lo[i], std::min(i, M - 1)); };
     auto reach_hi = [&](int i) { return std::max(hi[i], std::min(i, M - 1) + 1); };
     auto never = [&](int i) { return reach_hi(i) - reach_lo(i) > p_max; };
 
-    std::vector<char> fused(L, 0);
-    int slab_rows = 0;
-    int s = 0;
+    int slab_rows = windowed ? S->slab_rows : 0;
+    int s = windowed ? M : 0;
     while (s < M) {
       tf::TileDesc t{};
       // 1. grow a tile whose producer window covers every fusable row it owns
@@ -169,7 +251,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       if (a >= 0) { t.wb_begin = a; t.wb_end = b; S->n_writeback_rows += b - a; }
     }
     S->slab_rows = slab_rows;
-    S->lds_bytes = slab_rows * row_bytes + staging;
+    S->lds_bytes_general = slab_rows * row_bytes + staging;
+    if (!windowed) S->lds_bytes = S->lds_bytes_general;
 
     // MultiDimensionalSet-layout view (Fusion_Inspector.h:959-1010).
     const int nt = (int)S->tiles.size();
@@ -234,6 +317,8 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   info->n_writeback_rows = s->n_writeback_rows;
   info->max_tile_producer_rows = s->slab_rows;
   info->lds_bytes = s->lds_bytes;
+  info->windowed = s->windowed ? 1 : 0;
+  info->strip_cols = s->windowed ? s->opts.strip_cols : 0;
   info->fused_nnz = s->fused_nnz;
   long long ws = 0;
   if (s->n_writeback_rows > 0) ws += (long long)s->M * s->opts.N * 4;
@@ -271,7 +356,7 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
     prev_end = t.own_end;
     if (t.prod_begin > t.own_begin || t.prod_end < t.own_end || t.prod_begin < 0 || t.prod_end > M)
       return tf::fail(TF_ESCHEDULE, "tile %zu: producer range [%d,%d) does not cover owned rows [%d,%d)", ti, t.prod_begin, t.prod_end, t.own_begin, t.own_end);
-    if (t.cons_end > t.cons_begin &&
+    if (!s->windowed && t.cons_end > t.cons_begin &&
         (long long)(t.prod_end - t.prod_begin) * row_bytes > s->opts.lds_budget_bytes)
       return tf::fail(TF_ESCHEDULE, "tile %zu: slab of %d rows exceeds the LDS budget", ti, t.prod_end - t.prod_begin);
     if (t.wb_begin < t.own_begin || t.wb_end > t.own_end || t.wb_end < t.wb_begin)

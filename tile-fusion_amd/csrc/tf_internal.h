@@ -41,6 +41,10 @@ struct tf_schedule {
   tf_inspect_opts opts{};  // resolved (no zero "default" fields left)
   int L = 0, M = 0;
   int lds_bytes = 0;          // dynamic LDS of the fused kernel: intermediate slab (+ GEMM staging)
+  int lds_bytes_general = 0;  // the same for the kernel that gathers C from HBM (fallback of windowed tiles)
+  bool windowed = false;      // tiles stage their window of C in LDS (win holds the windows)
+  long long inner_nnz = 0;    // stored entries of the inner pattern the windows were built from
+  std::vector<int> win;       // [2*n_tiles] first,last+1 row of C read by the tile's producer rows
   int slab_rows = 0;          // max producer rows of any tile
   int gemm_kc = 0;            // rows of C staged in LDS per step (GeMM-SpMM)
   std::vector<tf::TileDesc> tiles;

@@ -14,7 +14,10 @@
 
 namespace tf {
 
-constexpr int kBlock = 256;  // threads per workgroup of every kernel in this file
+#ifndef TF_BLOCK
+#define TF_BLOCK 256
+#endif
+constexpr int kBlock = TF_BLOCK;  // threads per workgroup of every kernel in this file
 constexpr int kXcds = 8;     // workgroup ids are dealt round-robin over the 8 XCDs
 
 template <int V> struct alignas(4 * V) fvec { float v[V]; };
@@ -133,6 +136,141 @@ __global__ __launch_bounds__(kBlock) void fused_spmm_spmm_kernel(
       if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)i * N + coff);
       row_dot<V, LPR>(Ai, Ax, Ap[i], Ap[i + 1], glane, ok, tsrc, acc);
       if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)i * N + coff) = acc;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Windowed fused SpMM-SpMM tile kernel (inner matrix == outer matrix, the reference's
+// setting).  Everything a tile touches more than once is staged in LDS first:
+//   * the CSR chunk of its producer rows, as (byte offset into the window, value) pairs,
+//     one pad entry per row so that the rows a wavefront walks start in different banks;
+//   * then, strip by strip (SW columns of C/D at a time): the window of C rows the
+//     producer rows read, the slab of intermediate rows, and out of it the fused rows.
+// A lane group of SW/4 lanes owns one row; both products read only LDS, HBM sees each
+// C row about once per tile and each D row once.  Same fma sequence per element as
+// fused_spmm_spmm_kernel, hence the same bits.
+// ---------------------------------------------------------------------------------
+constexpr int kWinPad = 2;  // pad slots after each staged row (keeps 8 rows' reads in 8 bank groups)
+
+__device__ __forceinline__ int align16i(int x) { return (x + 15) & ~15; }
+
+// acc += sum_k val[k] * row(off[k]) over staged entries [kb, ke), in order.  The entry
+// reads of the next four are issued before the fmas of the current four.
+__device__ __forceinline__ fvec<4> lds_row_dot(const int2 *__restrict__ ent, int kb, int ke,
+                                               const char *base, fvec<4> acc) {
+  int k = kb;
+  if (k + 4 <= ke) {
+    int2 e0 = ent[k], e1 = ent[k + 1], e2 = ent[k + 2], e3 = ent[k + 3];
+    k += 4;
+    for (;;) {
+      const fvec<4> x0 = *reinterpret_cast<const fvec<4> *>(base + e0.x);
+      const fvec<4> x1 = *reinterpret_cast<const fvec<4> *>(base + e1.x);
+      const fvec<4> x2 = *reinterpret_cast<const fvec<4> *>(base + e2.x);
+      const fvec<4> x3 = *reinterpret_cast<const fvec<4> *>(base + e3.x);
+      const bool more = k + 4 <= ke;
+      int2 n0 = e0, n1 = e1, n2 = e2, n3 = e3;
+      if (more) { n0 = ent[k]; n1 = ent[k + 1]; n2 = ent[k + 2]; n3 = ent[k + 3]; }
+      vfma<4>(__int_as_float(e0.y), x0, acc);
+      vfma<4>(__int_as_float(e1.y), x1, acc);
+      vfma<4>(__int_as_float(e2.y), x2, acc);
+      vfma<4>(__int_as_float(e3.y), x3, acc);
+      if (!more) break;
+      e0 = n0; e1 = n1; e2 = n2; e3 = n3;
+      k += 4;
+    }
+  }
+  for (; k < ke; ++k) {
+    const int2 e0 = ent[k];
+    vfma<4>(__int_as_float(e0.y), *reinterpret_cast<const fvec<4> *>(base + e0.x), acc);
+  }
+  return acc;
+}
+
+// One 16-byte unit of a strip of the window of C (unit u = row-in-window * LPR + quad).
+// Threads past the end re-read unit 0, which always exists; the value is not used.
+template <int LPR>
+__device__ __forceinline__ fvec<4> window_unit(const float *__restrict__ C, int first_row, int N, int c0,
+                                               int n4, int u) {
+  const int uu = u < n4 ? u : 0;
+  return *reinterpret_cast<const fvec<4> *>(C + (size_t)(first_row + uu / LPR) * N + c0 + (uu % LPR) * 4);
+}
+
+template <int SW, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
+    const TileDesc *__restrict__ tiles, const int2 *__restrict__ win, int n_tiles, int per_xcd,
+    const int *__restrict__ fused_ids, const int *__restrict__ Bp, const int *__restrict__ Bi,
+    const float *__restrict__ Bx, const float *__restrict__ C, float *__restrict__ D, int N,
+    int accumulate) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int LPR = SW / 4;           // lanes per row
+  constexpr int G = BLOCK / LPR;        // rows in flight per workgroup
+  constexpr int ROWB = SW * 4;          // bytes of one strip row
+  const int tile = xcd_contiguous(blockIdx.x, per_xcd);
+  if (tile >= n_tiles) return;
+  const TileDesc t = tiles[tile];
+  const int2 w = win[tile];
+  const int P = t.prod_end - t.prod_begin, R = t.cons_end - t.cons_begin, Wc = w.y - w.x;
+  const int k0 = Bp[t.prod_begin];
+  const int nz = Bp[t.prod_end] - k0;
+  int *rp = reinterpret_cast<int *>(smem);
+  int *cons = reinterpret_cast<int *>(smem + align16i(4 * (P + 1)));
+  int2 *ent = reinterpret_cast<int2 *>(reinterpret_cast<unsigned char *>(cons) + align16i(4 * R));
+  float *Cbuf = reinterpret_cast<float *>(reinterpret_cast<unsigned char *>(ent) + align16i(8 * (nz + kWinPad * P)));
+  float *Tbuf = Cbuf + Wc * SW;
+  const int tid = threadIdx.x, group = tid / LPR, glane = tid % LPR;
+
+  const int n4 = Wc * LPR;  // 16-byte units in one strip of the window
+  // The next strip of the window is fetched into registers while the current one is being
+  // worked on, and dropped into LDS once the current strip's first product is done.
+  constexpr int UPT = 4;  // register-prefetched 16-byte units per thread
+  fvec<4> pre0 = window_unit<LPR>(C, w.x, N, 0, n4, tid);
+  fvec<4> pre1 = window_unit<LPR>(C, w.x, N, 0, n4, tid + BLOCK);
+  fvec<4> pre2 = window_unit<LPR>(C, w.x, N, 0, n4, tid + 2 * BLOCK);
+  fvec<4> pre3 = window_unit<LPR>(C, w.x, N, 0, n4, tid + 3 * BLOCK);
+  // row pointers: entry j of row i sits at rp[i] + j, kWinPad unused slots follow every row
+  for (int i = tid; i <= P; i += BLOCK) rp[i] = Bp[t.prod_begin + i] - k0 + kWinPad * i;
+  for (int i = tid; i < R; i += BLOCK) cons[i] = fused_ids[t.cons_begin + i] - t.prod_begin;
+  // entries: one lane group per row
+  for (int r = group; r < P; r += G) {
+    const int kb = Bp[t.prod_begin + r], ke = Bp[t.prod_begin + r + 1];
+    const int dst = kb - k0 + kWinPad * r;
+    for (int k = kb + glane; k < ke; k += LPR)
+      ent[dst + (k - kb)] = make_int2((Bi[k] - w.x) * ROWB, __float_as_int(Bx[k]));
+  }
+  const char *cbase = reinterpret_cast<const char *>(Cbuf) + glane * 16;
+  // a consumer's column c lives in the slab at row c - prod_begin = (c - w.x) + (w.x - prod_begin)
+  const char *tbase = reinterpret_cast<const char *>(Tbuf) + (w.x - t.prod_begin) * ROWB + glane * 16;
+  for (int c0 = 0; c0 < N; c0 += SW) {
+    __syncthreads();  // previous strip fully consumed (and, first time, staging visible)
+    {
+      fvec<4> *cb = reinterpret_cast<fvec<4> *>(Cbuf);
+      if (tid < n4) cb[tid] = pre0;
+      if (tid + BLOCK < n4) cb[tid + BLOCK] = pre1;
+      if (tid + 2 * BLOCK < n4) cb[tid + 2 * BLOCK] = pre2;
+      if (tid + 3 * BLOCK < n4) cb[tid + 3 * BLOCK] = pre3;
+      for (int u = tid + UPT * BLOCK; u < n4; u += BLOCK)  // windows beyond the prefetch capacity
+        cb[u] = window_unit<LPR>(C, w.x, N, c0, n4, u);
+    }
+    if (c0 + SW < N) {
+      pre0 = window_unit<LPR>(C, w.x, N, c0 + SW, n4, tid);
+      pre1 = window_unit<LPR>(C, w.x, N, c0 + SW, n4, tid + BLOCK);
+      pre2 = window_unit<LPR>(C, w.x, N, c0 + SW, n4, tid + 2 * BLOCK);
+      pre3 = window_unit<LPR>(C, w.x, N, c0 + SW, n4, tid + 3 * BLOCK);
+    }
+    __syncthreads();
+    for (int r = group; r < P; r += G) {
+      const fvec<4> acc = lds_row_dot(ent, rp[r], rp[r + 1] - kWinPad, cbase, vzero<4>());
+      *reinterpret_cast<fvec<4> *>(Tbuf + r * SW + glane * 4) = acc;
+    }
+    __syncthreads();
+    for (int q = group; q < R; q += G) {
+      const int r = cons[q];
+      float *dst = D + (size_t)(t.prod_begin + r) * N + c0 + glane * 4;
+      fvec<4> acc = vzero<4>();
+      if (accumulate) acc = *reinterpret_cast<const fvec<4> *>(dst);
+      acc = lds_row_dot(ent, rp[r], rp[r + 1] - kWinPad, tbase, acc);
+      *reinterpret_cast<fvec<4> *>(dst) = acc;
     }
   }
 }
@@ -413,6 +551,32 @@ hipError_t launch_fused_spmm_spmm(const TileDesc *tiles, int n_tiles, const int 
                        Ax, D, T, N, N, accumulate)
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
 #undef CALL
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+#ifndef TF_WIN_BLOCK
+#define TF_WIN_BLOCK 512
+#endif
+hipError_t launch_fused_spmm_spmm_window(const TileDesc *tiles, const int *win, int n_tiles,
+                                         const int *fused_ids, const int *Bp, const int *Bi,
+                                         const float *Bx, const float *C, float *D, int N, int strip,
+                                         int lds_bytes, int accumulate, hipStream_t st) {
+  if (n_tiles <= 0) return hipSuccess;
+  constexpr int BLOCK = TF_WIN_BLOCK;
+  const int per = per_xcd_of(n_tiles);
+  const int2 *w2 = reinterpret_cast<const int2 *>(win);
+  hipError_t err;
+  if (strip == 32) {
+    err = allow_lds(fused_spmm_spmm_window_kernel<32, BLOCK>, lds_bytes);
+    if (err == hipSuccess)
+      hipLaunchKernelGGL((fused_spmm_spmm_window_kernel<32, BLOCK>), dim3(per * kXcds), dim3(BLOCK), lds_bytes,
+                         st, tiles, w2, n_tiles, per, fused_ids, Bp, Bi, Bx, C, D, N, accumulate);
+  } else {
+    err = allow_lds(fused_spmm_spmm_window_kernel<64, BLOCK>, lds_bytes);
+    if (err == hipSuccess)
+      hipLaunchKernelGGL((fused_spmm_spmm_window_kernel<64, BLOCK>), dim3(per * kXcds), dim3(BLOCK), lds_bytes,
+                         st, tiles, w2, n_tiles, per, fused_ids, Bp, Bi, Bx, C, D, N, accumulate);
+  }
   return err != hipSuccess ? err : hipGetLastError();
 }
 
