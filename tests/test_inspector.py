@@ -48,7 +48,12 @@ def validate(view, info, A, lds_budget):
         for i in rows:
             cols = A.indices[A.indptr[i]:A.indptr[i + 1]]
             assert np.all(stored[cols]), f"remainder row {i} reads a row nobody stores"
-    assert info["n_writeback_rows"] == int(sum(b - a for a, b in wb))
+    # rows actually stored: at least every row a remainder row reads, at most the write-back ranges
+    needed = np.zeros(M, bool)
+    for p in range(nt, P):
+        for i in ids[ptr2[p]:ptr2[p + 1]]:
+            needed[A.indices[A.indptr[i]:A.indptr[i + 1]]] = True
+    assert int(needed.sum()) <= info["n_writeback_rows"] <= int(sum(b - a for a, b in wb))
 
 
 def inspect(tf, A, **kw):

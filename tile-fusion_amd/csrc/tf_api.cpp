@@ -33,6 +33,7 @@ struct DeviceSchedule {
   int *fused_ids = nullptr;
   int *win = nullptr;
   int *rem_rows = nullptr;
+  int *plain_rows = nullptr;
   LongChunk *long_chunks = nullptr;
   LongRow *long_rows = nullptr;
   float *inter = nullptr;    // M x N intermediate, only if some tile writes back
@@ -53,7 +54,7 @@ hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const 
 hipError_t launch_fused_gemm_spmm(const TileDesc *, int, const int *, const float *, const float *,
                                   int, int, const int *, const int *, const float *, float *,
                                   float *, int, int, int, hipStream_t);
-hipError_t launch_gemm(const float *, const float *, float *, int, int, int, int, hipStream_t);
+hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t);
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 
 static thread_local char g_err[512] = "";
@@ -87,7 +88,7 @@ int default_compute_units() {
 
 void release_device_schedule(DeviceSchedule *d) {
   if (!d) return;
-  (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows);
+  (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows); (void)hipFree(d->plain_rows);
   (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows);
   (void)hipFree(d->inter); (void)hipFree(d->partial);
   delete d;
@@ -115,10 +116,11 @@ static tf_status ensure_device(tf_schedule *s) {
   auto *d = new (std::nothrow) DeviceSchedule();
   if (!d) return fail(TF_ENOMEM, "out of host memory");
   d->device = dev;
-  tf_status rc = upload_vec(s->tiles, &d->tiles);
+  tf_status rc = upload_vec(s->launch_tiles, &d->tiles);
   if (!rc) rc = upload_vec(s->fused_ids, &d->fused_ids);
   if (!rc) rc = upload_vec(s->win, &d->win);
   if (!rc) rc = upload_vec(s->rem_rows, &d->rem_rows);
+  if (!rc) rc = upload_vec(s->plain_rows, &d->plain_rows);
   if (!rc) rc = upload_vec(s->long_chunks, &d->long_chunks);
   if (!rc) rc = upload_vec(s->long_rows, &d->long_rows);
   if (!rc && s->n_writeback_rows > 0) {
@@ -371,7 +373,7 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
     // The windowed kernel walks one staged CSR chunk for both products: B must be A.
     const bool same = (B == A) || (B->p == A->p && B->i == A->i && B->x == A->x);
     if (same) {
-      TF_HIP(tf::launch_fused_spmm_spmm_window(d->tiles, d->win, (int)s->tiles.size(), d->fused_ids, A->p,
+      TF_HIP(tf::launch_fused_spmm_spmm_window(d->tiles, d->win, (int)s->launch_tiles.size(), d->fused_ids, A->p,
                                                A->i, A->x, C->d, D->d, s->opts.N, s->opts.strip_cols,
                                                s->lds_bytes, acc, st));
       return TF_OK;
@@ -379,9 +381,14 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
     if (s->lds_bytes_general > 163840)
       return fail(TF_ESCHEDULE, "tf_spmm_spmm: this schedule needs B to be the same matrix as A");
   }
-  TF_HIP(tf::launch_fused_spmm_spmm(d->tiles, (int)s->tiles.size(), d->fused_ids, B->p, B->i, B->x,
+  TF_HIP(tf::launch_fused_spmm_spmm(d->tiles, (int)s->launch_tiles.size(), d->fused_ids, B->p, B->i, B->x,
                                     C->d, A->p, A->i, A->x, D->d, d->inter, s->opts.N,
                                     s->windowed ? s->lds_bytes_general : s->lds_bytes, acc, st));
+  if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
+    const bool all = (int)s->plain_rows.size() == s->M;
+    TF_HIP(tf::launch_spmm_rows(all ? nullptr : d->plain_rows, (int)s->plain_rows.size(), B->p, B->i, B->x,
+                                C->d, d->inter, s->opts.N, 0, st));
+  }
   return tf::run_remainder(A, D, s, acc, st);
 }
 
@@ -398,9 +405,14 @@ extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_d
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
   const tf::DeviceSchedule *d = s->dev;
-  TF_HIP(tf::launch_fused_gemm_spmm(d->tiles, (int)s->tiles.size(), d->fused_ids, B->d, C->d,
+  TF_HIP(tf::launch_fused_gemm_spmm(d->tiles, (int)s->launch_tiles.size(), d->fused_ids, B->d, C->d,
                                     s->opts.K, s->gemm_kc, A->p, A->i, A->x, D->d, d->inter,
                                     s->opts.N, s->lds_bytes, acc, st));
+  if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
+    const bool all = (int)s->plain_rows.size() == s->M;
+    TF_HIP(tf::launch_gemm(B->d, C->d, d->inter, all ? nullptr : d->plain_rows, (int)s->plain_rows.size(),
+                           s->opts.K, s->opts.N, s->opts.compute_units, st));
+  }
   return tf::run_remainder(A, D, s, acc, st);
 }
 
@@ -420,7 +432,7 @@ extern "C" tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, 
   const int K = X->N, N = W->N;
   if (K % 8 != 0 || N % 32 != 0 || N > 256)
     return fail(TF_EUNSUPPORTED, "tf_gemm: needs K %% 8 == 0, N %% 32 == 0, N <= 256 (K=%d N=%d)", K, N);
-  const int kc = std::min(K, std::max(8, (32768 / (4 * N)) / 8 * 8));
-  TF_HIP(tf::launch_gemm(X->d, W->d, Y->d, X->M, K, N, kc, static_cast<hipStream_t>(stream)));
+  TF_HIP(tf::launch_gemm(X->d, W->d, Y->d, nullptr, X->M, K, N, tf::default_compute_units(),
+                         static_cast<hipStream_t>(stream)));
   return TF_OK;
 }

@@ -244,11 +244,24 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         S->rem_rows.push_back(i);
       }
     }
+    // Tiles that fuse nothing are not launched as tiles: the intermediate rows they own go to
+    // the row kernels (plain SpMM / GEMM), and only those some remainder row reads.  A GEMM
+    // whose weight does not fit LDS has no row-list form; such tiles stay tiles.
+    const bool plain_ok = o.op == TF_OP_SPMM_SPMM || (long long)o.K * o.N * 4 <= 131072;
     for (auto &t : S->tiles) {
-      int a = -1, b = -1;
+      int a = -1, b = -1, cnt = 0;
       for (int r = t.own_begin; r < t.own_end; ++r)
-        if (need[r]) { if (a < 0) a = r; b = r + 1; }
-      if (a >= 0) { t.wb_begin = a; t.wb_end = b; S->n_writeback_rows += b - a; }
+        if (need[r]) { if (a < 0) a = r; b = r + 1; ++cnt; }
+      if (a >= 0) { t.wb_begin = a; t.wb_end = b; }
+      const bool fuses = t.cons_end > t.cons_begin;
+      if (fuses || !plain_ok) {
+        S->launch_tiles.push_back(t);
+        if (a >= 0) S->n_writeback_rows += b - a;
+      } else {
+        for (int r = t.own_begin; r < t.own_end; ++r)
+          if (need[r]) S->plain_rows.push_back(r);
+        S->n_writeback_rows += cnt;
+      }
     }
     S->slab_rows = slab_rows;
     S->lds_bytes_general = slab_rows * row_bytes + staging;

@@ -48,6 +48,9 @@ struct tf_schedule {
   int slab_rows = 0;          // max producer rows of any tile
   int gemm_kc = 0;            // rows of C staged in LDS per step (GeMM-SpMM)
   std::vector<tf::TileDesc> tiles;
+  std::vector<tf::TileDesc> launch_tiles;  // the tiles that fuse something: one workgroup each
+  std::vector<int> plain_rows;      // intermediate rows of tiles that fuse nothing, computed by the
+                                    // row kernels -- only the rows some remainder row reads
   std::vector<int> fused_ids;       // second-op rows per tile, tile after tile
   std::vector<int> rem_rows;        // remainder rows handled one row per lane group
   std::vector<tf::LongChunk> long_chunks;

@@ -277,27 +277,135 @@ __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
 
 // ---------------------------------------------------------------------------------
 // Row-wise SpMM  Y[i,:] = sum_k Ax[k] * X[Ai[k],:]  for i = rows[q] (or i = q when rows
-// is null).  Serves the unfused remainder (X = the intermediate in HBM) and tf_spmm.
+// is null).  Serves the unfused remainder (X = the intermediate in HBM), producer rows
+// that no tile fuses, and tf_spmm.
+//
+// A workgroup takes a block of consecutive list positions.  The dependent chain
+// "row pointer -> column indices -> gather" is paid once per block instead of once per
+// row: all row pointers of the block are loaded together, then all (column, value)
+// pairs go to LDS, and only then the lane groups walk their rows, gathering X with
+// several independent loads in flight.  Per-element fma order is CSR order.
 // ---------------------------------------------------------------------------------
+constexpr int kSpmmCap = 4096;  // staged entries per batch: 32 KB of LDS
+
+template <int V, class Src>
+__device__ __forceinline__ void staged_row_dot(const int2 *__restrict__ ent, int kb, int ke, const Src &src,
+                                               fvec<V> &acc) {
+  int k = kb;
+  for (; k + 8 <= ke; k += 8) {
+    int2 e[8];
+    fvec<V> x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) e[u] = ent[k + u];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) x[u] = src.load(e[u].x);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) vfma<V>(__int_as_float(e[u].y), x[u], acc);
+  }
+  if (k + 4 <= ke) {
+    int2 e[4];
+    fvec<V> x[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) e[u] = ent[k + u];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) x[u] = src.load(e[u].x);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) vfma<V>(__int_as_float(e[u].y), x[u], acc);
+    k += 4;
+  }
+  for (; k < ke; ++k) {
+    const int2 e = ent[k];
+    vfma<V>(__int_as_float(e.y), src.load(e.x), acc);
+  }
+}
+
 template <int V, int LPR>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
-    const int *__restrict__ rows, int n_rows, int per_xcd, const int *__restrict__ Ap,
-    const int *__restrict__ Ai, const float *__restrict__ Ax, const float *__restrict__ X, int ldx,
-    float *__restrict__ Y, int N, int accumulate) {
+    const int *__restrict__ rows, int n_rows, int rows_per_block, int per_xcd,
+    const int *__restrict__ Ap, const int *__restrict__ Ai, const float *__restrict__ Ax,
+    const float *__restrict__ X, int ldx, float *__restrict__ Y, int N, int accumulate) {
   constexpr int G = kBlock / LPR;
-  const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
-  const int q = xcd_contiguous(blockIdx.x, per_xcd) * G + group;
-  if (q >= n_rows) return;  // whole lane groups leave together
-  const int i = rows ? rows[q] : q;
-  const int kb = Ap[i], ke = Ap[i + 1];
-  for (int c0 = 0; c0 < N; c0 += LPR * V) {
-    const int coff = c0 + glane * V;
-    const bool ok = coff < N;
-    const GlobalRows<V> src{X, ldx, ok ? coff : 0};
-    fvec<V> acc = vzero<V>();
-    if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
-    row_dot<V, LPR>(Ai, Ax, kb, ke, glane, ok, src, acc);
-    if (ok) *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
+  constexpr int NW = kBlock / 64;
+  __shared__ int2 ent[kSpmmCap];
+  __shared__ int s_row[kBlock], s_kb[kBlock], s_pos[kBlock + 1], s_wsum[NW];
+  const int tid = threadIdx.x, group = tid / LPR, glane = tid % LPR;
+  const int q0 = xcd_contiguous(blockIdx.x, per_xcd) * rows_per_block;
+  if (q0 >= n_rows) return;
+  const int nr = min(rows_per_block, n_rows - q0);  // <= kBlock
+
+  // row ids, first entries and an exclusive scan of the row lengths
+  int len = 0;
+  if (tid < nr) {
+    const int i = rows ? rows[q0 + tid] : q0 + tid;
+    const int kb = Ap[i];
+    len = Ap[i + 1] - kb;
+    s_row[tid] = i;
+    s_kb[tid] = kb;
+  }
+  int incl = len;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up = __shfl_up(incl, d, 64);
+    if ((tid & 63) >= d) incl += up;
+  }
+  if ((tid & 63) == 63) s_wsum[tid >> 6] = incl;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < (tid >> 6); ++w) base += s_wsum[w];
+  if (tid < nr) s_pos[tid] = base + incl - len;
+  if (tid == nr - 1) s_pos[nr] = base + incl;
+  __syncthreads();
+
+  int b0 = 0;
+  while (b0 < nr) {
+    // the longest run of rows [b0, b1) whose entries fit the staging buffer
+    const int p0 = s_pos[b0];
+    int b1 = b0 + 1;
+    {
+      int lo = b0 + 1, hi = nr;  // largest b with s_pos[b] - p0 <= cap
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (s_pos[mid] - p0 <= kSpmmCap) lo = mid; else hi = mid - 1;
+      }
+      b1 = lo;
+    }
+    if (s_pos[b1] - p0 > kSpmmCap) {
+      // a single row longer than the buffer: one lane group walks it straight from HBM
+      if (group == 0) {
+        const int i = s_row[b0], kb = s_kb[b0], ke = kb + (s_pos[b0 + 1] - p0);
+        for (int c0 = 0; c0 < N; c0 += LPR * V) {
+          const int coff = c0 + glane * V;
+          const bool ok = coff < N;
+          const GlobalRows<V> src{X, ldx, ok ? coff : 0};
+          fvec<V> acc = vzero<V>();
+          if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
+          row_dot<V, LPR>(Ai, Ax, kb, ke, glane, ok, src, acc);
+          if (ok) *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
+        }
+      }
+      b0 = b0 + 1;
+      continue;
+    }
+    for (int r = b0 + group; r < b1; r += G) {
+      const int kb = s_kb[r], n = s_pos[r + 1] - s_pos[r], dst = s_pos[r] - p0;
+      for (int j = glane; j < n; j += LPR) ent[dst + j] = make_int2(Ai[kb + j], __float_as_int(Ax[kb + j]));
+    }
+    __syncthreads();
+    for (int r = b0 + group; r < b1; r += G) {
+      const int i = s_row[r], kb = s_pos[r] - p0, ke = s_pos[r + 1] - p0;
+      for (int c0 = 0; c0 < N; c0 += LPR * V) {
+        const int coff = c0 + glane * V;
+        if (coff < N) {
+          const GlobalRows<V> src{X, ldx, coff};
+          fvec<V> acc = vzero<V>();
+          if (accumulate) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
+          staged_row_dot<V>(ent, kb, ke, src, acc);
+          *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
+        }
+      }
+    }
+    __syncthreads();
+    b0 = b1;
   }
 }
 
@@ -475,7 +583,8 @@ __global__ __launch_bounds__(kBlock) void fused_gemm_spmm_kernel(
   }
 }
 
-// Plain GEMM  Y = X * W  (tf_gemm): 128 rows per workgroup, no slab.
+// Plain GEMM  Y = X * W  (tf_gemm) when K*N is too large to keep W in LDS: 128 rows per
+// workgroup, W streamed through LDS in kc-row slices.
 template <int NB>
 __global__ __launch_bounds__(kBlock) void gemm_kernel(const float *__restrict__ X, const float *__restrict__ W,
                                                       float *__restrict__ Y, int M, int K, int kc,
@@ -485,6 +594,109 @@ __global__ __launch_bounds__(kBlock) void gemm_kernel(const float *__restrict__ 
   if (b >= n_blocks) return;
   const int p0 = b * 128, p1 = min(M, p0 + 128);
   tile_gemm<NB>(X, W, K, kc, p0, p1, lds, nullptr, Y, p0, p1);
+}
+
+// Row-list GEMM  Y[r,:] = X[r,:K] * W  for r = rows[q] (or r = q when rows is null):
+// intermediate rows that no tile fuses, and tf_gemm.  Persistent: W (K x N) is copied to
+// LDS once per workgroup, then every wavefront walks its own 32-row blocks with no
+// barrier at all; the rows of X for the next 32 values of k are already in flight
+// (16 bytes per lane and load, see tile_gemm for the k permutation) while the MFMAs of
+// the current ones issue.
+constexpr int kGemmBlock = 512;
+
+template <int NB>
+__global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__restrict__ X,
+                                                               const float *__restrict__ W,
+                                                               float *__restrict__ Y,
+                                                               const int *__restrict__ rows, int n_rows,
+                                                               int K) {
+  extern __shared__ __align__(16) float wlds[];
+  constexpr int N = NB * 32;
+  {
+    const int n4 = K * N / 4;
+    const fvec<4> *src = reinterpret_cast<const fvec<4> *>(W);
+    fvec<4> *dst = reinterpret_cast<fvec<4> *>(wlds);
+    for (int i = threadIdx.x; i < n4; i += kGemmBlock) dst[i] = src[i];
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int h = lane / 32, j = lane % 32;
+  const int total_waves = gridDim.x * (kGemmBlock / 64);
+  const int nrb = (n_rows + 31) / 32;
+  const int groups = K / 32;       // groups of four 8-wide k steps
+  const int tail8 = (K % 32) / 8;  // leftover 8-wide steps
+  for (int rb = blockIdx.x * (kGemmBlock / 64) + wave; rb < nrb; rb += total_waves) {
+    const int q = rb * 32 + j;  // list position whose row this lane feeds as the A operand
+    const bool row_ok = q < n_rows;
+    const int arow = row_ok ? (rows ? rows[q] : q) : 0;
+    const float *Xrow = X + (size_t)arow * K + 4 * h;
+    v16f acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
+    fvec<4> c0 = vzero<4>(), c1 = c0, c2 = c0, c3 = c0;
+    if (groups > 0 && row_ok) {
+      c0 = *reinterpret_cast<const fvec<4> *>(Xrow);
+      c1 = *reinterpret_cast<const fvec<4> *>(Xrow + 8);
+      c2 = *reinterpret_cast<const fvec<4> *>(Xrow + 16);
+      c3 = *reinterpret_cast<const fvec<4> *>(Xrow + 24);
+    }
+    for (int g = 0; g < groups; ++g) {
+      fvec<4> n0 = c0, n1 = c1, n2 = c2, n3 = c3;
+      if (g + 1 < groups && row_ok) {
+        const float *nx = Xrow + (g + 1) * 32;
+        n0 = *reinterpret_cast<const fvec<4> *>(nx);
+        n1 = *reinterpret_cast<const fvec<4> *>(nx + 8);
+        n2 = *reinterpret_cast<const fvec<4> *>(nx + 16);
+        n3 = *reinterpret_cast<const fvec<4> *>(nx + 24);
+      }
+      const float *wbase = wlds + (g * 32 + 4 * h) * N + j;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(c0.v[t], wbase[t * N + nb * 32], acc[nb], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(c1.v[t], wbase[(8 + t) * N + nb * 32], acc[nb], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(c2.v[t], wbase[(16 + t) * N + nb * 32], acc[nb], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(c3.v[t], wbase[(24 + t) * N + nb * 32], acc[nb], 0, 0, 0);
+      c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    }
+    for (int m = 0; m < tail8; ++m) {
+      const int kk = groups * 32 + m * 8;
+      fvec<4> a4 = vzero<4>();
+      if (row_ok) a4 = *reinterpret_cast<const fvec<4> *>(Xrow + kk);
+      const float *wbase = wlds + (kk + 4 * h) * N + j;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.v[t], wbase[t * N + nb * 32], acc[nb], 0, 0, 0);
+    }
+    // accumulator register r of lane (h, j) holds output row 8*(r/4) + 4*h + r%4, column j
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int oq = rb * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+      if (oq < n_rows) {
+        const int orow = rows ? rows[oq] : oq;
+        float *dst = Y + (size_t)orow * N + j;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) dst[nb * 32] = acc[nb][r];
+      }
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------------
@@ -585,11 +797,16 @@ hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const in
   if (n_rows <= 0) return hipSuccess;
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
-  const int blocks = (n_rows + G - 1) / G;
+  // rows per workgroup: a few passes of the lane groups, so the staging round trips are
+  // amortised, while the launch still has many more workgroups than compute units
+  int rpb = 4 * G;
+  while (rpb > G && (n_rows + rpb - 1) / rpb < 2048) rpb -= G;
+  rpb = std::min(rpb, kBlock);
+  const int blocks = (n_rows + rpb - 1) / rpb;
   const int per = per_xcd_of(blocks);
 #define CALL(V_, L_)                                                                        \
   hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(per *kXcds), dim3(kBlock), 0, st, rows, \
-                     n_rows, per, Ap, Ai, Ax, X, N, Y, N, accumulate)
+                     n_rows, rpb, per, Ap, Ai, Ax, X, N, Y, N, accumulate)
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
 #undef CALL
   return hipGetLastError();
@@ -638,19 +855,36 @@ hipError_t launch_fused_gemm_spmm(const TileDesc *tiles, int n_tiles, const int 
   return err != hipSuccess ? err : hipGetLastError();
 }
 
-hipError_t launch_gemm(const float *X, const float *W, float *Y, int M, int K, int N, int kc,
-                       hipStream_t st) {
-  if (M <= 0) return hipSuccess;
-  const int blocks = (M + 127) / 128;
-  const int per = per_xcd_of(blocks);
-  const int lds_bytes = kc * N * 4;
+hipError_t launch_gemm(const float *X, const float *W, float *Y, const int *rows, int n_rows, int K,
+                       int N, int compute_units, hipStream_t st) {
+  if (n_rows <= 0) return hipSuccess;
   const int NB = N / 32;
   hipError_t err = hipSuccess;
+  const int w_bytes = K * N * 4;
+  if (w_bytes <= 131072) {
+    // W resident in LDS: persistent workgroups, as many per compute unit as the LDS allows
+    const int per_cu = std::max(1, std::min(2, 163840 / w_bytes));
+    const int nrb = (n_rows + 31) / 32;
+    const int grid = std::max(1, std::min(compute_units * per_cu, (nrb + kGemmBlock / 64 - 1) / (kGemmBlock / 64)));
+#define CALL(NB_)                                                                               \
+  err = allow_lds(gemm_rows_kernel<NB_>, w_bytes);                                              \
+  if (err == hipSuccess)                                                                        \
+    hipLaunchKernelGGL((gemm_rows_kernel<NB_>), dim3(grid), dim3(kGemmBlock), w_bytes, st, X, W, Y, \
+                       rows, n_rows, K)
+    TF_DISPATCH_NB(NB, CALL);
+#undef CALL
+    return err != hipSuccess ? err : hipGetLastError();
+  }
+  if (rows) return hipErrorInvalidValue;  // the streamed-W kernel takes contiguous rows only
+  const int kc = std::min(K, std::max(8, (32768 / (4 * N)) / 8 * 8));
+  const int blocks = (n_rows + 127) / 128;
+  const int per = per_xcd_of(blocks);
+  const int lds_bytes = kc * N * 4;
 #define CALL(NB_)                                                                               \
   err = allow_lds(gemm_kernel<NB_>, lds_bytes);                                                 \
   if (err == hipSuccess)                                                                        \
     hipLaunchKernelGGL((gemm_kernel<NB_>), dim3(per *kXcds), dim3(kBlock), lds_bytes, st, X, W, \
-                       Y, M, K, kc, per, blocks)
+                       Y, n_rows, K, kc, per, blocks)
   TF_DISPATCH_NB(NB, CALL);
 #undef CALL
   return err != hipSuccess ? err : hipGetLastError();
