@@ -113,8 +113,9 @@ typedef struct {
                             row (halo rows recomputed so that boundary rows still fuse);
                             1.0 disables recomputation = the reference's tiling.
                             Default 3.0 for SpMM-SpMM, 1.5 for GeMM-SpMM.                    */
-  int long_row_nnz;      /* remainder rows with more stored entries than this are split into
-                            chunks reduced by a wavefront-level tree; default 2048           */
+  int long_row_nnz;      /* remainder rows with more stored entries than this are worked on by a
+                            whole workgroup each (in chunks of max(this, 1024) entries, partial
+                            sums added in a fixed order); default 128, max 2048               */
   int compute_units;     /* sizing hint; default: the current device, or 256 with no device  */
   /* SpMM-SpMM only, optional: sparsity pattern of the inner matrix B (M x inner_cols, host
      arrays).  In every run of the reference B is A (fusion/example/SpMM_SpMM_Demo_Utils.h:

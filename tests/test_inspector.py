@@ -139,7 +139,7 @@ def test_long_rows_are_chunked(tf):
     A = sp.csr_matrix(hub + sp.identity(M, dtype=np.float32, format="csr"))
     S, view, info = inspect(tf, A, op=tf.OP_SPMM_SPMM, N=64, long_row_nnz=512)
     validate(view, info, A, 65536)
-    assert info["n_long_rows"] == 1 and info["n_long_chunks"] == 6  # ceil(3000 / 512)
+    assert info["n_long_rows"] == 1 and info["n_long_chunks"] == 3  # ceil(3000 / max(512, 1024))
 
 
 def test_rectangular_and_bad_arguments(tf):

@@ -57,7 +57,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     return tf::fail(TF_EINVAL, "tf_inspect: lds_budget_bytes %d exceeds %d", o.lds_budget_bytes, kMaxLds);
   if (o.max_redundancy <= 0.f) o.max_redundancy = (o.op == TF_OP_GEMM_SPMM) ? 1.5f : 3.0f;
   if (o.max_redundancy < 1.f) o.max_redundancy = 1.f;
-  if (o.long_row_nnz <= 0) o.long_row_nnz = 2048;
+  if (o.long_row_nnz <= 0) o.long_row_nnz = 128;
+  if (o.long_row_nnz > 2048) o.long_row_nnz = 2048;  // a row must fit one staging batch of the row kernel
   if (o.compute_units <= 0) o.compute_units = tf::default_compute_units();
 
   // LDS the tile GEMM needs for staging C, before any slab row.
@@ -218,6 +219,17 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
           if (lo[i] >= s && hi[i] <= e) { S->fused_ids.push_back(i); fused[i] = 1; }
       }
       t.cons_end = (int)S->fused_ids.size();
+      {  // rows without entries fuse trivially; a tile that would fuse only such rows fuses nothing
+        // and one that would fuse less than a quarter of its rows is not worth a workgroup of its own
+        int useful = 0;
+        for (int q = t.cons_begin; q < t.cons_end; ++q)
+          useful += Ap[S->fused_ids[q] + 1] > Ap[S->fused_ids[q]];
+        if (4 * useful < t.own_end - t.own_begin) {
+          for (int q = t.cons_begin; q < t.cons_end; ++q) fused[S->fused_ids[q]] = 0;
+          S->fused_ids.resize(t.cons_begin);
+          t.cons_end = t.cons_begin;
+        }
+      }
       if (t.cons_end > t.cons_begin) slab_rows = std::max(slab_rows, t.prod_end - t.prod_begin);
       else { t.prod_begin = t.own_begin; t.prod_end = t.own_end; }  // nothing to fuse: no halo
       t.wb_begin = t.wb_end = t.own_begin;
@@ -226,7 +238,9 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       s = e;
     }
 
-    // Remainder: rows not fused; long ones are cut into chunks.
+    // Remainder: rows not fused; long ones are cut into chunks of up to chunk_nnz entries, each
+    // worked on by a whole workgroup.
+    const int chunk_nnz = std::max(o.long_row_nnz, 1024);
     std::vector<char> need(M, 0);
     for (int i = 0; i < L; ++i) {
       if (fused[i]) { S->fused_nnz += Ap[i + 1] - Ap[i]; continue; }
@@ -234,8 +248,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       const int len = Ap[i + 1] - Ap[i];
       if (len > o.long_row_nnz) {
         tf::LongRow lr{i, (int)S->long_chunks.size(), 0, 0};
-        for (int k = Ap[i]; k < Ap[i + 1]; k += o.long_row_nnz) {
-          tf::LongChunk c{i, k, std::min(Ap[i + 1], k + o.long_row_nnz), (int)S->long_chunks.size()};
+        for (int k = Ap[i]; k < Ap[i + 1]; k += chunk_nnz) {
+          tf::LongChunk c{i, k, std::min(Ap[i + 1], k + chunk_nnz), (int)S->long_chunks.size()};
           S->long_chunks.push_back(c);
           ++lr.count;
         }
@@ -244,6 +258,38 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         S->rem_rows.push_back(i);
       }
     }
+    // Remainder rows of similar length go together: a lane group walks a row alone, so a
+    // workgroup is as slow as its longest row.  Order is kept inside a length class, and a
+    // matrix whose rows all fall in one class keeps its order entirely.
+    {
+      auto cls = [&](int i) {
+        const int len = Ap[i + 1] - Ap[i];
+        return len <= 8 ? 0 : len <= 32 ? 1 : len <= 128 ? 2 : len <= 512 ? 3 : 4;
+      };
+      std::vector<int> byc[5];
+      for (int i : S->rem_rows) byc[cls(i)].push_back(i);
+      S->rem_rows.clear();
+      for (auto &v : byc) S->rem_rows.insert(S->rem_rows.end(), v.begin(), v.end());
+      S->rem_identity = (int)S->rem_rows.size() == L;
+      for (int q = 0; q < L && S->rem_identity; ++q) S->rem_identity = (S->rem_rows[q] == q);
+      // blocks: at most `max_rows` rows and 2048 stored entries (one staging batch) each
+      const int vec = (o.N % 4 == 0) ? 4 : (o.N % 2 == 0) ? 2 : 1;
+      int lpr = 8;
+      while (lpr < (o.N + vec - 1) / vec && lpr < 64) lpr *= 2;
+      const int max_rows = std::min(256, 4 * (256 / lpr));
+      S->rem_blocks.push_back(0);
+      int rows_in = 0, nnz_in = 0, prev_cls = -1;
+      for (size_t q = 0; q < S->rem_rows.size(); ++q) {
+        const int i = S->rem_rows[q], len = Ap[i + 1] - Ap[i], c = cls(i);
+        if (rows_in > 0 && (rows_in >= max_rows || nnz_in + len > 2048 || c != prev_cls)) {
+          S->rem_blocks.push_back((int)q);
+          rows_in = 0; nnz_in = 0;
+        }
+        ++rows_in; nnz_in += len; prev_cls = c;
+      }
+      if (!S->rem_rows.empty()) S->rem_blocks.push_back((int)S->rem_rows.size());
+    }
+
     // Tiles that fuse nothing are not launched as tiles: the intermediate rows they own go to
     // the row kernels (plain SpMM / GEMM), and only those some remainder row reads.  A GEMM
     // whose weight does not fit LDS has no row-list form; such tiles stay tiles.
@@ -410,7 +456,7 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
     for (int c = lr.first; c < lr.first + lr.count; ++c) {
       const auto &ch = s->long_chunks[c];
       if (ch.row != lr.row || ch.k_begin != k || ch.k_end <= ch.k_begin || ch.slot != c ||
-          ch.k_end - ch.k_begin > s->opts.long_row_nnz)
+          ch.k_end - ch.k_begin > std::max(s->opts.long_row_nnz, 1024))
         return tf::fail(TF_ESCHEDULE, "long row %d: chunk %d does not continue at entry %d", lr.row, c, k);
       k = ch.k_end;
     }

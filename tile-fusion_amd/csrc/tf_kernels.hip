@@ -41,6 +41,7 @@ template <int V> __device__ __forceinline__ void vadd(const fvec<V> &x, fvec<V> 
 // that every XCD works on one contiguous run of work items: neighbours share halo
 // rows and gather targets, which then stay in one L2.
 __device__ __forceinline__ int xcd_contiguous(int bid, int per_xcd) {
+  if (per_xcd <= 0) return bid;  // remapping switched off
   return (bid % kXcds) * per_xcd + bid / kXcds;
 }
 
@@ -286,52 +287,54 @@ __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
 // pairs go to LDS, and only then the lane groups walk their rows, gathering X with
 // several independent loads in flight.  Per-element fma order is CSR order.
 // ---------------------------------------------------------------------------------
-constexpr int kSpmmCap = 4096;  // staged entries per batch: 32 KB of LDS
+constexpr int kSpmmCap = 2048;  // staged entries per batch: 16 KB of LDS
+
+// acc += sum over staged entries [kb, ke) of value * src.row(column), in order.  Entries
+// are taken eight (then four) at a time and all gathers of a batch are issued before its
+// first fma.  The last one to three entries go as one batch of four whose unused slots
+// re-read the row's last entry and skip the fma, so that a short row costs one memory
+// round trip instead of one per entry.
+template <int V, int B, class Src>
+__device__ __forceinline__ void staged_batch(const int2 *__restrict__ ent, int k, int ke, const Src &src,
+                                             fvec<V> &acc) {
+  int2 e[B];
+  fvec<V> x[B];
+#pragma unroll
+  for (int u = 0; u < B; ++u) e[u] = ent[min(k + u, ke - 1)];
+#pragma unroll
+  for (int u = 0; u < B; ++u) x[u] = src.load(e[u].x);
+#pragma unroll
+  for (int u = 0; u < B; ++u) {
+    fvec<V> next = acc;
+    vfma<V>(__int_as_float(e[u].y), x[u], next);
+    if (k + u < ke) acc = next;
+  }
+}
 
 template <int V, class Src>
 __device__ __forceinline__ void staged_row_dot(const int2 *__restrict__ ent, int kb, int ke, const Src &src,
                                                fvec<V> &acc) {
   int k = kb;
-  for (; k + 8 <= ke; k += 8) {
-    int2 e[8];
-    fvec<V> x[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) e[u] = ent[k + u];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) x[u] = src.load(e[u].x);
-#pragma unroll
-    for (int u = 0; u < 8; ++u) vfma<V>(__int_as_float(e[u].y), x[u], acc);
-  }
-  if (k + 4 <= ke) {
-    int2 e[4];
-    fvec<V> x[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) e[u] = ent[k + u];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) x[u] = src.load(e[u].x);
-#pragma unroll
-    for (int u = 0; u < 4; ++u) vfma<V>(__int_as_float(e[u].y), x[u], acc);
-    k += 4;
-  }
-  for (; k < ke; ++k) {
-    const int2 e = ent[k];
-    vfma<V>(__int_as_float(e.y), src.load(e.x), acc);
-  }
+  for (; k + 8 <= ke; k += 8) staged_batch<V, 8>(ent, k, ke, src, acc);
+  if (k + 4 <= ke) { staged_batch<V, 4>(ent, k, ke, src, acc); k += 4; }
+  if (k < ke) staged_batch<V, 4>(ent, k, ke, src, acc);
 }
 
 template <int V, int LPR>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
-    const int *__restrict__ rows, int n_rows, int rows_per_block, int per_xcd,
-    const int *__restrict__ Ap, const int *__restrict__ Ai, const float *__restrict__ Ax,
+    const int *__restrict__ rows, int n_rows, const int *__restrict__ blocks, int n_blocks,
+    int rows_per_block, int per_xcd, const int *__restrict__ Ap, const int *__restrict__ Ai, const float *__restrict__ Ax,
     const float *__restrict__ X, int ldx, float *__restrict__ Y, int N, int accumulate) {
   constexpr int G = kBlock / LPR;
   constexpr int NW = kBlock / 64;
   __shared__ int2 ent[kSpmmCap];
   __shared__ int s_row[kBlock], s_kb[kBlock], s_pos[kBlock + 1], s_wsum[NW];
   const int tid = threadIdx.x, group = tid / LPR, glane = tid % LPR;
-  const int q0 = xcd_contiguous(blockIdx.x, per_xcd) * rows_per_block;
-  if (q0 >= n_rows) return;
-  const int nr = min(rows_per_block, n_rows - q0);  // <= kBlock
+  // block = rows [q0, q0 + nr) of the list: given by the cut array, else uniform
+  const int b = xcd_contiguous(blockIdx.x, per_xcd);
+  if (b >= n_blocks) return;
+  const int q0 = blocks ? blocks[b] : b * rows_per_block;
+  const int nr = blocks ? blocks[b + 1] - q0 : min(rows_per_block, n_rows - q0);  // <= kBlock
 
   // row ids, first entries and an exclusive scan of the row lengths
   int len = 0;
@@ -714,7 +717,14 @@ Shape pick_shape(int N) {
   return {V, LPR};
 }
 
-inline int per_xcd_of(int n) { return (n + kXcds - 1) / kXcds; }
+// Work items per XCD for xcd_contiguous; 0 (identity mapping) when the environment variable
+// TF_XCD_REMAP is set to 0.  The grid is sized grid_of(n) either way.
+inline bool xcd_remap_on() {
+  static const bool on = [] { const char *e = getenv("TF_XCD_REMAP"); return !(e && e[0] == '0'); }();
+  return on;
+}
+inline int per_xcd_of(int n) { return xcd_remap_on() ? (n + kXcds - 1) / kXcds : 0; }
+inline int grid_of(int n) { return (n + kXcds - 1) / kXcds * kXcds; }
 
 template <class F> hipError_t allow_lds(F kernel, int bytes) {
   if (bytes <= 65536) return hipSuccess;
@@ -758,7 +768,7 @@ hipError_t launch_fused_spmm_spmm(const TileDesc *tiles, int n_tiles, const int 
 #define CALL(V_, L_)                                                                       \
   err = allow_lds(fused_spmm_spmm_kernel<V_, L_>, lds_bytes);                              \
   if (err == hipSuccess)                                                                   \
-    hipLaunchKernelGGL((fused_spmm_spmm_kernel<V_, L_>), dim3(per *kXcds), dim3(kBlock),   \
+    hipLaunchKernelGGL((fused_spmm_spmm_kernel<V_, L_>), dim3(grid_of(n_tiles)), dim3(kBlock),   \
                        lds_bytes, st, tiles, n_tiles, per, fused_ids, Bp, Bi, Bx, C, Ap, Ai, \
                        Ax, D, T, N, N, accumulate)
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
@@ -781,32 +791,36 @@ hipError_t launch_fused_spmm_spmm_window(const TileDesc *tiles, const int *win, 
   if (strip == 32) {
     err = allow_lds(fused_spmm_spmm_window_kernel<32, BLOCK>, lds_bytes);
     if (err == hipSuccess)
-      hipLaunchKernelGGL((fused_spmm_spmm_window_kernel<32, BLOCK>), dim3(per * kXcds), dim3(BLOCK), lds_bytes,
+      hipLaunchKernelGGL((fused_spmm_spmm_window_kernel<32, BLOCK>), dim3(grid_of(n_tiles)), dim3(BLOCK), lds_bytes,
                          st, tiles, w2, n_tiles, per, fused_ids, Bp, Bi, Bx, C, D, N, accumulate);
   } else {
     err = allow_lds(fused_spmm_spmm_window_kernel<64, BLOCK>, lds_bytes);
     if (err == hipSuccess)
-      hipLaunchKernelGGL((fused_spmm_spmm_window_kernel<64, BLOCK>), dim3(per * kXcds), dim3(BLOCK), lds_bytes,
+      hipLaunchKernelGGL((fused_spmm_spmm_window_kernel<64, BLOCK>), dim3(grid_of(n_tiles)), dim3(BLOCK), lds_bytes,
                          st, tiles, w2, n_tiles, per, fused_ids, Bp, Bi, Bx, C, D, N, accumulate);
   }
   return err != hipSuccess ? err : hipGetLastError();
 }
 
-hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const int *Ai, const float *Ax,
-                            const float *X, float *Y, int N, int accumulate, hipStream_t st) {
+hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *blocks, int n_blocks, const int *Ap,
+                            const int *Ai, const float *Ax, const float *X, float *Y, int N, int accumulate,
+                            hipStream_t st) {
   if (n_rows <= 0) return hipSuccess;
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
-  // rows per workgroup: a few passes of the lane groups, so the staging round trips are
-  // amortised, while the launch still has many more workgroups than compute units
-  int rpb = 4 * G;
-  while (rpb > G && (n_rows + rpb - 1) / rpb < 2048) rpb -= G;
-  rpb = std::min(rpb, kBlock);
-  const int blocks = (n_rows + rpb - 1) / rpb;
-  const int per = per_xcd_of(blocks);
-#define CALL(V_, L_)                                                                        \
-  hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(per *kXcds), dim3(kBlock), 0, st, rows, \
-                     n_rows, rpb, per, Ap, Ai, Ax, X, N, Y, N, accumulate)
+  int rpb = 0;
+  if (!blocks) {
+    // uniform blocks: a few passes of the lane groups per workgroup, so the staging round
+    // trips are amortised, while the launch still has many more workgroups than compute units
+    rpb = 4 * G;
+    while (rpb > G && (n_rows + rpb - 1) / rpb < 2048) rpb -= G;
+    rpb = std::min(rpb, kBlock);
+    n_blocks = (n_rows + rpb - 1) / rpb;
+  }
+  const int per = per_xcd_of(n_blocks);
+#define CALL(V_, L_)                                                                           \
+  hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(grid_of(n_blocks)), dim3(kBlock), 0, st, rows, \
+                     n_rows, blocks, n_blocks, rpb, per, Ap, Ai, Ax, X, N, Y, N, accumulate)
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
 #undef CALL
   return hipGetLastError();
@@ -841,7 +855,7 @@ hipError_t launch_fused_gemm_spmm(const TileDesc *tiles, int n_tiles, const int 
 #define CALL2(NB_, L_)                                                                      \
   err = allow_lds(fused_gemm_spmm_kernel<NB_, L_>, lds_bytes);                              \
   if (err == hipSuccess)                                                                    \
-    hipLaunchKernelGGL((fused_gemm_spmm_kernel<NB_, L_>), dim3(per *kXcds), dim3(kBlock),   \
+    hipLaunchKernelGGL((fused_gemm_spmm_kernel<NB_, L_>), dim3(grid_of(n_tiles)), dim3(kBlock),   \
                        lds_bytes, st, tiles, n_tiles, per, fused_ids, B, C, K, kc, Ap, Ai, Ax, \
                        D, T, accumulate)
 #define CALL(NB_)                                                         \
@@ -883,7 +897,7 @@ hipError_t launch_gemm(const float *X, const float *W, float *Y, const int *rows
 #define CALL(NB_)                                                                               \
   err = allow_lds(gemm_kernel<NB_>, lds_bytes);                                                 \
   if (err == hipSuccess)                                                                        \
-    hipLaunchKernelGGL((gemm_kernel<NB_>), dim3(per *kXcds), dim3(kBlock), lds_bytes, st, X, W, \
+    hipLaunchKernelGGL((gemm_kernel<NB_>), dim3(grid_of(blocks)), dim3(kBlock), lds_bytes, st, X, W, \
                        Y, n_rows, K, kc, per, blocks)
   TF_DISPATCH_NB(NB, CALL);
 #undef CALL
