@@ -83,6 +83,7 @@ def main():
     ap.add_argument("--max-redundancy", type=float, default=0.0)
     ap.add_argument("--strip", type=int, default=0, help="columns per strip of windowed tiles (32 or 64)")
     ap.add_argument("--no-window", action="store_true", help="do not build windowed tiles")
+    ap.add_argument("--xcd-chunk", type=int, default=0, help="rows per XCD turn of the row kernels (-1 contiguous)")
     ap.add_argument("--long-row", type=int, default=0, help="rows with more entries than this are chunked")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the result check")
@@ -104,7 +105,7 @@ def main():
     inner = Ah if (op == tf.OP_SPMM_SPMM and cfg["B"] is A and not args.no_window) else None
     S = tf.inspector(Ah, 1, op=op, N=N, K=K, lds_budget_bytes=args.lds, tile_rows=args.tile_rows,
                      max_redundancy=args.max_redundancy, inner=inner, strip_cols=args.strip,
-                     long_row_nnz=args.long_row)
+                     long_row_nnz=args.long_row, xcd_chunk_rows=args.xcd_chunk)
     inspect_s = time.perf_counter() - t0
     S.validate()
     info = S.info()

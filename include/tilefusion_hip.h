@@ -115,7 +115,7 @@ typedef struct {
                             Default 3.0 for SpMM-SpMM, 1.5 for GeMM-SpMM.                    */
   int long_row_nnz;      /* remainder rows with more stored entries than this are worked on by a
                             whole workgroup each (in chunks of max(this, 1024) entries, partial
-                            sums added in a fixed order); default 128, max 2048               */
+                            sums added in a fixed order); default 32, max 2048                */
   int compute_units;     /* sizing hint; default: the current device, or 256 with no device  */
   /* SpMM-SpMM only, optional: sparsity pattern of the inner matrix B (M x inner_cols, host
      arrays).  In every run of the reference B is A (fusion/example/SpMM_SpMM_Demo_Utils.h:
@@ -127,6 +127,9 @@ typedef struct {
   int inner_cols;
   int strip_cols;        /* windowed tiles work on this many columns of C/D at a time (32 or 64);
                             default 32                                                         */
+  int xcd_chunk_rows;    /* the row kernels deal rows to the 8 XCDs in chunks of this many rows;
+                            0 = choose (an eighth of a dominant far stencil distance, else one
+                            contiguous run per XCD), -1 = always contiguous                   */
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -158,6 +161,7 @@ typedef struct {
   int lds_bytes;         /* dynamic LDS of the fused-tile kernel                    */
   int windowed;          /* 1 when tiles stage their window of C in LDS             */
   int strip_cols;        /* columns per strip of the windowed kernel, else 0        */
+  int xcd_chunk_rows;    /* rows per XCD turn chosen for the row kernels (0: contiguous) */
   long long fused_nnz;   /* stored entries of A in fused rows (getFusedNnzNum)      */
   long long workspace_bytes; /* device memory the executor keeps (intermediate + partials) */
 } tf_schedule_info;

@@ -166,11 +166,66 @@ def test_full_size_banded_linearity_and_roundtrip(gpu, tf, orc):
     A, Cd = cfg["A"], cfg["C"]
     got, info = run_spmm_spmm(tf, A, A, Cd)
     assert info["n_fused_rows"] == A.shape[0]
-    assert np.array_equal(got, oracle_spmm_spmm(orc, A, A, Cd))
+    want = oracle_spmm_spmm(orc, A, A, Cd)
+    assert np.array_equal(got, want)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128, inner=Ah)  # the benchmark's schedule
+    assert S.info()["windowed"] == 1
+    D = tf.DenseMatrix(A.shape[0], 128)
+    tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(Cd), D, S)
+    assert np.array_equal(D.to_numpy(), want)
     C2 = tf.workloads.uniform(Cd.shape, 99)
     g2, _ = run_spmm_spmm(tf, A, A, C2)
     g12, _ = run_spmm_spmm(tf, A, A, Cd + C2)
     assert orc.rel_err(g12, got.astype(np.float64) + g2) <= 1e-5
+
+
+@pytest.mark.parametrize("N,strip", [(128, 32), (128, 64), (64, 32), (256, 64), (32, 32), (96, 32)])
+def test_spmm_spmm_windowed_bit_exact(gpu, tf, orc, N, strip):
+    """Windowed tiles (inner pattern given, B is A): CSR chunk, window of C and slab all in
+    LDS, strip by strip.  Same fma order as the reference, hence the same bits."""
+    say(f"spmm_spmm windowed N={N} strip={strip}")
+    for A in (tf.workloads.banded_random(5000, 32, 16, seed=33), tf.workloads.laplacian_2d(40, 70)):
+        M = A.shape[0]
+        Cd = tf.workloads.uniform((M, N), 34)
+        want = oracle_spmm_spmm(orc, A, A, Cd)
+        Ah = tf.CsrMatrix.from_scipy(A)
+        small = 65536 if strip == 32 else 131072
+        for kw in (dict(lds_budget_bytes=0 if strip == 32 else 163840), dict(lds_budget_bytes=163840, tile_rows=200),
+                   dict(tile_rows=48, lds_budget_bytes=small)):
+            S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N, inner=Ah, strip_cols=strip, **kw)
+            S.validate()
+            info = S.info()
+            assert info["windowed"] == 1 and info["n_fused_rows"] == M and info["n_writeback_rows"] == 0
+            D = tf.DenseMatrix(M, N)
+            D.fill(float("nan"))
+            tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(Cd), D, S)
+            tf.device_synchronize()
+            assert np.array_equal(D.to_numpy(), want), (N, strip, kw)
+        D0 = tf.workloads.uniform((M, N), 35)
+        D = tf.DenseMatrix.from_numpy(D0)
+        tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(Cd), D, S, accumulate=True)
+        assert orc.rel_err(D.to_numpy(), D0.astype(np.float64) + want) <= 1e-6
+
+
+def test_spmm_spmm_windowed_schedule_with_other_inner_matrix(gpu, tf, orc):
+    """A windowed schedule used with B != A falls back to the kernel that gathers C from
+    HBM (same tiles), and refuses an inner matrix of another size."""
+    say("spmm_spmm windowed schedule, B != A")
+    A = tf.workloads.banded_random(3000, 32, 16, seed=36)
+    B2 = A.copy()
+    B2.data = tf.workloads.uniform((A.nnz,), 37)
+    Cd = tf.workloads.uniform((3000, 64), 38)
+    Ah, Bh = tf.CsrMatrix.from_scipy(A), tf.CsrMatrix.from_scipy(B2)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah)
+    assert S.info()["windowed"] == 1
+    D = tf.DenseMatrix(3000, 64)
+    tf.spmm_spmm(Ah, Bh, tf.DenseMatrix.from_numpy(Cd), D, S)
+    assert np.array_equal(D.to_numpy(), oracle_spmm_spmm(orc, A, B2, Cd))
+    other = tf.CsrMatrix.from_scipy(tf.workloads.banded_random(3000, 32, 8, seed=39))
+    with pytest.raises(tf.TileFusionError) as e:
+        tf.spmm_spmm(Ah, other, tf.DenseMatrix.from_numpy(Cd), D, S)
+    assert e.value.status == -4
 
 
 # ---- GeMM-SpMM ----------------------------------------------------------------------------

@@ -175,3 +175,31 @@ def test_validator_rejects_a_schedule_for_another_pattern(tf):
     with pytest.raises(tf.TileFusionError) as e:
         S.validate(tf.CsrMatrix.from_scipy(A2))
     assert e.value.status == -4 and "row 500" in str(e.value)
+
+
+def test_windowed_tiles(tf):
+    """With the inner pattern given, banded and narrow-grid patterns get windowed tiles:
+    every row fused, nothing written back, and the window of C recorded per tile covers
+    every column the tile's producer rows read."""
+    for A, N in ((tf.workloads.banded_random(4096, 32, 16, seed=3), 128), (tf.workloads.laplacian_2d(48), 64)):
+        Ah = tf.CsrMatrix.from_scipy(A)
+        S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N, inner=Ah)
+        S.validate()
+        info, view = S.info(), S.view()
+        assert info["windowed"] == 1 and info["strip_cols"] == 32
+        assert info["n_fused_rows"] == A.shape[0] and info["n_writeback_rows"] == 0
+        assert info["lds_bytes"] <= 81920
+        validate(view, info, A, 163840)
+    # a pattern whose rows reach across the matrix cannot be windowed
+    R = tf.workloads.erdos_renyi_gcn(4000, 10.0, seed=5)
+    Rh = tf.CsrMatrix.from_scipy(R)
+    assert tf.inspector(Rh, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Rh).info()["windowed"] == 0
+
+
+def test_far_stencil_distance_sets_xcd_chunk(tf):
+    A = tf.workloads.laplacian_3d(40)  # planes 1600 rows apart: below the 2048-row floor
+    assert tf.inspector(tf.CsrMatrix.from_scipy(A), 1, op=tf.OP_SPMM_SPMM, N=64).info()["xcd_chunk_rows"] == 0
+    A = tf.workloads.laplacian_3d(64)  # planes 4096 rows apart -> chunks of 512 rows
+    assert tf.inspector(tf.CsrMatrix.from_scipy(A), 1, op=tf.OP_SPMM_SPMM, N=64).info()["xcd_chunk_rows"] == 512
+    A = tf.workloads.erdos_renyi_gcn(20000, 10.0, seed=5)  # random graph: no dominant distance
+    assert tf.inspector(tf.CsrMatrix.from_scipy(A), 1, op=tf.OP_SPMM_SPMM, N=64).info()["xcd_chunk_rows"] == 0

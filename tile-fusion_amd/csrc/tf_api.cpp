@@ -33,7 +33,6 @@ struct DeviceSchedule {
   int *fused_ids = nullptr;
   int *win = nullptr;
   int *rem_rows = nullptr;
-  int *rem_blocks = nullptr;
   int *plain_rows = nullptr;
   LongChunk *long_chunks = nullptr;
   LongRow *long_rows = nullptr;
@@ -48,8 +47,8 @@ hipError_t launch_fused_spmm_spmm(const TileDesc *, int, const int *, const int 
 hipError_t launch_fused_spmm_spmm_window(const TileDesc *, const int *, int, const int *, const int *,
                                          const int *, const float *, const float *, float *, int, int,
                                          int, int, hipStream_t);
-hipError_t launch_spmm_rows(const int *, int, const int *, int, const int *, const int *, const float *,
-                            const float *, float *, int, int, hipStream_t);
+hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
+                            float *, int, int, int, hipStream_t);
 hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const int *, const float *,
                             const float *, float *, float *, int, int, hipStream_t);
 hipError_t launch_fused_gemm_spmm(const TileDesc *, int, const int *, const float *, const float *,
@@ -89,7 +88,7 @@ int default_compute_units() {
 
 void release_device_schedule(DeviceSchedule *d) {
   if (!d) return;
-  (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows); (void)hipFree(d->rem_blocks); (void)hipFree(d->plain_rows);
+  (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows); (void)hipFree(d->plain_rows);
   (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows);
   (void)hipFree(d->inter); (void)hipFree(d->partial);
   delete d;
@@ -121,7 +120,6 @@ static tf_status ensure_device(tf_schedule *s) {
   if (!rc) rc = upload_vec(s->fused_ids, &d->fused_ids);
   if (!rc) rc = upload_vec(s->win, &d->win);
   if (!rc) rc = upload_vec(s->rem_rows, &d->rem_rows);
-  if (!rc) rc = upload_vec(s->rem_blocks, &d->rem_blocks);
   if (!rc) rc = upload_vec(s->plain_rows, &d->plain_rows);
   if (!rc) rc = upload_vec(s->long_chunks, &d->long_chunks);
   if (!rc) rc = upload_vec(s->long_rows, &d->long_rows);
@@ -146,8 +144,8 @@ static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int
   const int N = s->opts.N;
   if (!s->rem_rows.empty()) {
     // identity list: no indirection needed
-    TF_HIP(launch_spmm_rows(s->rem_identity ? nullptr : d->rem_rows, (int)s->rem_rows.size(), d->rem_blocks,
-                            (int)s->rem_blocks.size() - 1, A->p, A->i, A->x, d->inter, D->d, N, accumulate, st));
+    TF_HIP(launch_spmm_rows(s->rem_identity ? nullptr : d->rem_rows, (int)s->rem_rows.size(), A->p, A->i,
+                            A->x, d->inter, D->d, N, accumulate, s->xcd_chunk_rows, st));
   }
   if (!s->long_chunks.empty())
     TF_HIP(launch_long_rows(d->long_chunks, (int)s->long_chunks.size(), d->long_rows,
@@ -388,8 +386,8 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
                                     s->windowed ? s->lds_bytes_general : s->lds_bytes, acc, st));
   if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
     const bool all = (int)s->plain_rows.size() == s->M;
-    TF_HIP(tf::launch_spmm_rows(all ? nullptr : d->plain_rows, (int)s->plain_rows.size(), nullptr, 0, B->p,
-                                B->i, B->x, C->d, d->inter, s->opts.N, 0, st));
+    TF_HIP(tf::launch_spmm_rows(all ? nullptr : d->plain_rows, (int)s->plain_rows.size(), B->p, B->i, B->x,
+                                C->d, d->inter, s->opts.N, 0, s->xcd_chunk_rows, st));
   }
   return tf::run_remainder(A, D, s, acc, st);
 }
@@ -422,8 +420,8 @@ extern "C" tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, un
   if (!A || !X || !Y) return fail(TF_EINVAL, "tf_spmm: null argument");
   if (X->M != A->N || Y->M != A->M || X->N != Y->N)
     return fail(TF_EINVAL, "tf_spmm: shapes A %d x %d, X %d x %d, Y %d x %d", A->M, A->N, X->M, X->N, Y->M, Y->N);
-  TF_HIP(tf::launch_spmm_rows(nullptr, A->M, nullptr, 0, A->p, A->i, A->x, X->d, Y->d, X->N,
-                              (flags & TF_ACCUMULATE) ? 1 : 0, static_cast<hipStream_t>(stream)));
+  TF_HIP(tf::launch_spmm_rows(nullptr, A->M, A->p, A->i, A->x, X->d, Y->d, X->N,
+                              (flags & TF_ACCUMULATE) ? 1 : 0, 0, static_cast<hipStream_t>(stream)));
   return TF_OK;
 }
 

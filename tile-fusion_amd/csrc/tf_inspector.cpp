@@ -57,7 +57,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     return tf::fail(TF_EINVAL, "tf_inspect: lds_budget_bytes %d exceeds %d", o.lds_budget_bytes, kMaxLds);
   if (o.max_redundancy <= 0.f) o.max_redundancy = (o.op == TF_OP_GEMM_SPMM) ? 1.5f : 3.0f;
   if (o.max_redundancy < 1.f) o.max_redundancy = 1.f;
-  if (o.long_row_nnz <= 0) o.long_row_nnz = 128;
+  if (o.long_row_nnz <= 0) o.long_row_nnz = 32;
   if (o.long_row_nnz > 2048) o.long_row_nnz = 2048;  // a row must fit one staging batch of the row kernel
   if (o.compute_units <= 0) o.compute_units = tf::default_compute_units();
 
@@ -80,7 +80,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
                            o.inner_cols > 0 && o.N % o.strip_cols == 0;
   int r_cap = o.tile_rows > 0 ? o.tile_rows : ceil_div(M, 2 * o.compute_units);
   if (o.op == TF_OP_GEMM_SPMM) r_cap = ceil_div(r_cap, 32) * 32;
-  r_cap = std::max(r_cap, o.tile_rows > 0 ? 1 : 32);
+  r_cap = std::max(r_cap, o.tile_rows > 0 ? 1 : 64);  // smaller tiles spend most of their work on halo rows
   r_cap = std::min(r_cap, p_max);
   o.tile_rows = r_cap;
 
@@ -156,8 +156,9 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
           if (lds_of(nhi - nlo, e + 1 - s, (long long)Bp[nhi] - Bp[nlo], Wc) > o.lds_budget_bytes) break;
           wlo = nlo; whi = nhi; clo = nclo; chi = nchi; ++e;
         }
-        if (e == s || (e - s < std::min(r_cap, 16) && e != M) ||
-            (float)(whi - wlo) > o.max_redundancy * (float)(e - s)) { ok = false; break; }
+        // (the last tile of the matrix may be short, and then has relatively more halo)
+        if (e == s || (e != M && (e - s < std::min(r_cap, 16) ||
+                                  (float)(whi - wlo) > o.max_redundancy * (float)(e - s)))) { ok = false; break; }
         tf::TileDesc t{};
         t.own_begin = s; t.own_end = e; t.prod_begin = wlo; t.prod_end = whi;
         t.wb_begin = t.wb_end = s;
@@ -204,8 +205,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         if (nhi - nlo > p_max) break;
         wlo = nlo; whi = nhi; ++e;
       }
-      const bool halo_ok = (e > s) && (e - s >= std::min(r_cap, 16) || e == M) &&
-                           (float)(whi - wlo) <= o.max_redundancy * (float)(e - s);
+      const bool halo_ok = (e > s) && (e == M || (e - s >= std::min(r_cap, 16) &&
+                                                 (float)(whi - wlo) <= o.max_redundancy * (float)(e - s)));
       t.cons_begin = (int)S->fused_ids.size();
       if (halo_ok) {
         t.own_begin = s; t.own_end = e; t.prod_begin = wlo; t.prod_end = whi;
@@ -272,22 +273,36 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       for (auto &v : byc) S->rem_rows.insert(S->rem_rows.end(), v.begin(), v.end());
       S->rem_identity = (int)S->rem_rows.size() == L;
       for (int q = 0; q < L && S->rem_identity; ++q) S->rem_identity = (S->rem_rows[q] == q);
-      // blocks: at most `max_rows` rows and 2048 stored entries (one staging batch) each
-      const int vec = (o.N % 4 == 0) ? 4 : (o.N % 2 == 0) ? 2 : 1;
-      int lpr = 8;
-      while (lpr < (o.N + vec - 1) / vec && lpr < 64) lpr *= 2;
-      const int max_rows = std::min(256, 4 * (256 / lpr));
-      S->rem_blocks.push_back(0);
-      int rows_in = 0, nnz_in = 0, prev_cls = -1;
-      for (size_t q = 0; q < S->rem_rows.size(); ++q) {
-        const int i = S->rem_rows[q], len = Ap[i + 1] - Ap[i], c = cls(i);
-        if (rows_in > 0 && (rows_in >= max_rows || nnz_in + len > 2048 || c != prev_cls)) {
-          S->rem_blocks.push_back((int)q);
-          rows_in = 0; nnz_in = 0;
+    }
+
+    // Stencil-like patterns read rows a fixed far distance away (the plane above and below).
+    // If one such distance carries a good share of the entries, the row kernels deal rows to
+    // the XCDs in chunks of an eighth of it: every XCD then keeps the same slab of each plane
+    // and finds the neighbouring planes' rows still in its L2.
+    if (o.xcd_chunk_rows > 0) {
+      S->xcd_chunk_rows = o.xcd_chunk_rows;
+    } else if (o.xcd_chunk_rows == 0 && nnz > 0) {
+      std::vector<long long> hist(32, 0);  // entries by floor(log2(|col - row|))
+      std::vector<int> sample(32, 0);      // one distance seen per bucket
+      const int step = (int)std::max<long long>(1, nnz / 4000000);  // sample every step-th row
+      long long seen = 0, total = 0;
+      for (int i = 0; i < L; i += step) {
+        total += Ap[i + 1] - Ap[i];
+        for (int k = Ap[i]; k < Ap[i + 1]; ++k) {
+          const int d = std::abs(Ai[k] - i);
+          if (d < 2048) continue;
+          int b = 0;
+          while ((2 << b) <= d) ++b;
+          ++hist[b]; sample[b] = d; ++seen;
         }
-        ++rows_in; nnz_in += len; prev_cls = c;
       }
-      if (!S->rem_rows.empty()) S->rem_blocks.push_back((int)S->rem_rows.size());
+      int best = -1;
+      for (int b = 31; b >= 0; --b)
+        if (hist[b] * 8 >= total) { best = b; break; }  // the farthest distance with >= 1/8 of the entries
+      if (best >= 0 && seen * 2 <= total * 1) {          // a stencil, not a random graph: most entries are near
+        const int d = sample[best];
+        S->xcd_chunk_rows = std::max(256, d / 8 / 64 * 64);
+      }
     }
 
     // Tiles that fuse nothing are not launched as tiles: the intermediate rows they own go to
@@ -378,6 +393,7 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   info->lds_bytes = s->lds_bytes;
   info->windowed = s->windowed ? 1 : 0;
   info->strip_cols = s->windowed ? s->opts.strip_cols : 0;
+  info->xcd_chunk_rows = s->xcd_chunk_rows;
   info->fused_nnz = s->fused_nnz;
   long long ws = 0;
   if (s->n_writeback_rows > 0) ws += (long long)s->M * s->opts.N * 4;

@@ -54,8 +54,8 @@ struct tf_schedule {
   std::vector<int> fused_ids;       // second-op rows per tile, tile after tile
   std::vector<int> rem_rows;        // remainder rows handled one row per lane group, ordered by
                                     // length class so that a workgroup's rows cost about the same
-  std::vector<int> rem_blocks;      // [n+1] cuts of rem_rows into workgroup blocks (bounded rows and entries)
   bool rem_identity = false;        // rem_rows is 0..L-1 in order
+  int xcd_chunk_rows = 0;           // rows per XCD turn of the row kernels (0: one contiguous run per XCD)
   std::vector<tf::LongChunk> long_chunks;
   std::vector<tf::LongRow> long_rows;
   long long fused_nnz = 0;

@@ -37,12 +37,16 @@ template <int V> __device__ __forceinline__ void vadd(const fvec<V> &x, fvec<V> 
   for (int i = 0; i < V; ++i) acc.v[i] += x.v[i];
 }
 
-// Consecutive workgroup ids land on different XCDs (each with its own L2).  Remap so
-// that every XCD works on one contiguous run of work items: neighbours share halo
-// rows and gather targets, which then stay in one L2.
-__device__ __forceinline__ int xcd_contiguous(int bid, int per_xcd) {
-  if (per_xcd <= 0) return bid;  // remapping switched off
-  return (bid % kXcds) * per_xcd + bid / kXcds;
+// Consecutive workgroup ids land on different XCDs (each with its own 4 MB L2).  Work items
+// are cut into chunks of `bpc` consecutive items and chunk c goes to XCD c % 8, so that an
+// XCD walks whole chunks in order.  With bpc = all items / 8 every XCD gets one contiguous
+// run (neighbouring tiles share halo rows in one L2); with bpc = (a far stencil stride) / 8
+// every XCD keeps the same slab of every plane, so the plane above and below a row are
+// still in its L2 when they are needed again.  bpc <= 0 switches the remapping off.
+__device__ __forceinline__ int xcd_contiguous(int bid, int bpc) {
+  if (bpc <= 0) return bid;
+  const int xcd = bid % kXcds, s = bid / kXcds;
+  return ((s / bpc) * kXcds + xcd) * bpc + (s % bpc);
 }
 
 template <int V> struct GlobalRows {
@@ -63,6 +67,34 @@ template <int V> struct LdsRows {
 
 // acc += sum over stored entries k in [kb, ke) of val[k] * src.row(idx[k]), CSR order.
 // All LPR lanes of the group must call this together (it shuffles inside the group).
+// The group loads up to LPR (column, value) pairs with one coalesced load, then takes them
+// eight (or four) at a time: all gathers of a batch are issued before its first fma, and a
+// short last batch re-reads the last entry in its unused slots and skips their fma, so a
+// short row costs one gather round trip instead of one per entry.
+template <int V, int LPR, int B, class Src>
+__device__ __forceinline__ void row_dot_batch(int c, float a, int t, int cnt, bool col_ok, const Src &src,
+                                              fvec<V> &acc) {
+  int cc[B];
+  float aa[B];
+#pragma unroll
+  for (int u = 0; u < B; ++u) {
+    const int sl = min(t + u, cnt - 1);
+    cc[u] = __shfl(c, sl, LPR);
+    aa[u] = __shfl(a, sl, LPR);
+  }
+  if (col_ok) {
+    fvec<V> x[B];
+#pragma unroll
+    for (int u = 0; u < B; ++u) x[u] = src.load(cc[u]);
+#pragma unroll
+    for (int u = 0; u < B; ++u) {
+      fvec<V> next = acc;
+      vfma<V>(aa[u], x[u], next);
+      if (t + u < cnt) acc = next;
+    }
+  }
+}
+
 template <int V, int LPR, class Src>
 __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float *__restrict__ val,
                                         int kb, int ke, int glane, bool col_ok, const Src &src,
@@ -74,24 +106,10 @@ __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float
     if (k < ke) { c = idx[k]; a = val[k]; }
     const int cnt = min(LPR, ke - k0);
     int t = 0;
-    for (; t + 4 <= cnt; t += 4) {
-      const int c0 = __shfl(c, t, LPR), c1 = __shfl(c, t + 1, LPR);
-      const int c2 = __shfl(c, t + 2, LPR), c3 = __shfl(c, t + 3, LPR);
-      const float a0 = __shfl(a, t, LPR), a1 = __shfl(a, t + 1, LPR);
-      const float a2 = __shfl(a, t + 2, LPR), a3 = __shfl(a, t + 3, LPR);
-      if (col_ok) {
-        const fvec<V> x0 = src.load(c0), x1 = src.load(c1), x2 = src.load(c2), x3 = src.load(c3);
-        vfma<V>(a0, x0, acc);
-        vfma<V>(a1, x1, acc);
-        vfma<V>(a2, x2, acc);
-        vfma<V>(a3, x3, acc);
-      }
-    }
-    for (; t < cnt; ++t) {
-      const int c0 = __shfl(c, t, LPR);
-      const float a0 = __shfl(a, t, LPR);
-      if (col_ok) vfma<V>(a0, src.load(c0), acc);
-    }
+    if constexpr (LPR >= 8)
+      for (; t + 8 <= cnt; t += 8) row_dot_batch<V, LPR, 8>(c, a, t, cnt, col_ok, src, acc);
+    if (t + 4 <= cnt) { row_dot_batch<V, LPR, 4>(c, a, t, cnt, col_ok, src, acc); t += 4; }
+    if (t < cnt) row_dot_batch<V, LPR, 4>(c, a, t, cnt, col_ok, src, acc);
   }
 }
 
@@ -279,136 +297,30 @@ __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
 // ---------------------------------------------------------------------------------
 // Row-wise SpMM  Y[i,:] = sum_k Ax[k] * X[Ai[k],:]  for i = rows[q] (or i = q when rows
 // is null).  Serves the unfused remainder (X = the intermediate in HBM), producer rows
-// that no tile fuses, and tf_spmm.
-//
-// A workgroup takes a block of consecutive list positions.  The dependent chain
-// "row pointer -> column indices -> gather" is paid once per block instead of once per
-// row: all row pointers of the block are loaded together, then all (column, value)
-// pairs go to LDS, and only then the lane groups walk their rows, gathering X with
-// several independent loads in flight.  Per-element fma order is CSR order.
+// that no tile fuses, and tf_spmm.  One lane group per row and small, short-lived
+// workgroups: what hides the gather latency is the number of rows in flight.
 // ---------------------------------------------------------------------------------
-constexpr int kSpmmCap = 2048;  // staged entries per batch: 16 KB of LDS
-
-// acc += sum over staged entries [kb, ke) of value * src.row(column), in order.  Entries
-// are taken eight (then four) at a time and all gathers of a batch are issued before its
-// first fma.  The last one to three entries go as one batch of four whose unused slots
-// re-read the row's last entry and skip the fma, so that a short row costs one memory
-// round trip instead of one per entry.
-template <int V, int B, class Src>
-__device__ __forceinline__ void staged_batch(const int2 *__restrict__ ent, int k, int ke, const Src &src,
-                                             fvec<V> &acc) {
-  int2 e[B];
-  fvec<V> x[B];
-#pragma unroll
-  for (int u = 0; u < B; ++u) e[u] = ent[min(k + u, ke - 1)];
-#pragma unroll
-  for (int u = 0; u < B; ++u) x[u] = src.load(e[u].x);
-#pragma unroll
-  for (int u = 0; u < B; ++u) {
-    fvec<V> next = acc;
-    vfma<V>(__int_as_float(e[u].y), x[u], next);
-    if (k + u < ke) acc = next;
-  }
-}
-
-template <int V, class Src>
-__device__ __forceinline__ void staged_row_dot(const int2 *__restrict__ ent, int kb, int ke, const Src &src,
-                                               fvec<V> &acc) {
-  int k = kb;
-  for (; k + 8 <= ke; k += 8) staged_batch<V, 8>(ent, k, ke, src, acc);
-  if (k + 4 <= ke) { staged_batch<V, 4>(ent, k, ke, src, acc); k += 4; }
-  if (k < ke) staged_batch<V, 4>(ent, k, ke, src, acc);
-}
-
 template <int V, int LPR>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
-    const int *__restrict__ rows, int n_rows, const int *__restrict__ blocks, int n_blocks,
-    int rows_per_block, int per_xcd, const int *__restrict__ Ap, const int *__restrict__ Ai, const float *__restrict__ Ax,
-    const float *__restrict__ X, int ldx, float *__restrict__ Y, int N, int accumulate) {
+    const int *__restrict__ rows, int n_rows, int n_blocks, int per_xcd, const int *__restrict__ Ap,
+    const int *__restrict__ Ai, const float *__restrict__ Ax, const float *__restrict__ X, int ldx,
+    float *__restrict__ Y, int N, int accumulate) {
   constexpr int G = kBlock / LPR;
-  constexpr int NW = kBlock / 64;
-  __shared__ int2 ent[kSpmmCap];
-  __shared__ int s_row[kBlock], s_kb[kBlock], s_pos[kBlock + 1], s_wsum[NW];
-  const int tid = threadIdx.x, group = tid / LPR, glane = tid % LPR;
-  // block = rows [q0, q0 + nr) of the list: given by the cut array, else uniform
+  const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
   const int b = xcd_contiguous(blockIdx.x, per_xcd);
   if (b >= n_blocks) return;
-  const int q0 = blocks ? blocks[b] : b * rows_per_block;
-  const int nr = blocks ? blocks[b + 1] - q0 : min(rows_per_block, n_rows - q0);  // <= kBlock
-
-  // row ids, first entries and an exclusive scan of the row lengths
-  int len = 0;
-  if (tid < nr) {
-    const int i = rows ? rows[q0 + tid] : q0 + tid;
-    const int kb = Ap[i];
-    len = Ap[i + 1] - kb;
-    s_row[tid] = i;
-    s_kb[tid] = kb;
-  }
-  int incl = len;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int up = __shfl_up(incl, d, 64);
-    if ((tid & 63) >= d) incl += up;
-  }
-  if ((tid & 63) == 63) s_wsum[tid >> 6] = incl;
-  __syncthreads();
-  int base = 0;
-  for (int w = 0; w < (tid >> 6); ++w) base += s_wsum[w];
-  if (tid < nr) s_pos[tid] = base + incl - len;
-  if (tid == nr - 1) s_pos[nr] = base + incl;
-  __syncthreads();
-
-  int b0 = 0;
-  while (b0 < nr) {
-    // the longest run of rows [b0, b1) whose entries fit the staging buffer
-    const int p0 = s_pos[b0];
-    int b1 = b0 + 1;
-    {
-      int lo = b0 + 1, hi = nr;  // largest b with s_pos[b] - p0 <= cap
-      while (lo < hi) {
-        const int mid = (lo + hi + 1) >> 1;
-        if (s_pos[mid] - p0 <= kSpmmCap) lo = mid; else hi = mid - 1;
-      }
-      b1 = lo;
-    }
-    if (s_pos[b1] - p0 > kSpmmCap) {
-      // a single row longer than the buffer: one lane group walks it straight from HBM
-      if (group == 0) {
-        const int i = s_row[b0], kb = s_kb[b0], ke = kb + (s_pos[b0 + 1] - p0);
-        for (int c0 = 0; c0 < N; c0 += LPR * V) {
-          const int coff = c0 + glane * V;
-          const bool ok = coff < N;
-          const GlobalRows<V> src{X, ldx, ok ? coff : 0};
-          fvec<V> acc = vzero<V>();
-          if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
-          row_dot<V, LPR>(Ai, Ax, kb, ke, glane, ok, src, acc);
-          if (ok) *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
-        }
-      }
-      b0 = b0 + 1;
-      continue;
-    }
-    for (int r = b0 + group; r < b1; r += G) {
-      const int kb = s_kb[r], n = s_pos[r + 1] - s_pos[r], dst = s_pos[r] - p0;
-      for (int j = glane; j < n; j += LPR) ent[dst + j] = make_int2(Ai[kb + j], __float_as_int(Ax[kb + j]));
-    }
-    __syncthreads();
-    for (int r = b0 + group; r < b1; r += G) {
-      const int i = s_row[r], kb = s_pos[r] - p0, ke = s_pos[r + 1] - p0;
-      for (int c0 = 0; c0 < N; c0 += LPR * V) {
-        const int coff = c0 + glane * V;
-        if (coff < N) {
-          const GlobalRows<V> src{X, ldx, coff};
-          fvec<V> acc = vzero<V>();
-          if (accumulate) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
-          staged_row_dot<V>(ent, kb, ke, src, acc);
-          *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
-        }
-      }
-    }
-    __syncthreads();
-    b0 = b1;
+  const int q = b * G + group;
+  if (q >= n_rows) return;  // whole lane groups leave together
+  const int i = rows ? rows[q] : q;
+  const int kb = Ap[i], ke = Ap[i + 1];
+  for (int c0 = 0; c0 < N; c0 += LPR * V) {
+    const int coff = c0 + glane * V;
+    const bool ok = coff < N;
+    const GlobalRows<V> src{X, ldx, ok ? coff : 0};
+    fvec<V> acc = vzero<V>();
+    if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
+    row_dot<V, LPR>(Ai, Ax, kb, ke, glane, ok, src, acc);
+    if (ok) *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
   }
 }
 
@@ -725,6 +637,9 @@ inline bool xcd_remap_on() {
 }
 inline int per_xcd_of(int n) { return xcd_remap_on() ? (n + kXcds - 1) / kXcds : 0; }
 inline int grid_of(int n) { return (n + kXcds - 1) / kXcds * kXcds; }
+// The same for chunks of `bpc` items per XCD turn (see xcd_contiguous).
+inline int chunk_bpc(int n, int bpc) { return !xcd_remap_on() ? 0 : (bpc <= 0 || bpc * kXcds >= n) ? (n + kXcds - 1) / kXcds : bpc; }
+inline int grid_chunked(int n, int bpc) { return bpc <= 0 ? grid_of(n) : (n + bpc * kXcds - 1) / (bpc * kXcds) * (bpc * kXcds); }
 
 template <class F> hipError_t allow_lds(F kernel, int bytes) {
   if (bytes <= 65536) return hipSuccess;
@@ -802,25 +717,17 @@ hipError_t launch_fused_spmm_spmm_window(const TileDesc *tiles, const int *win, 
   return err != hipSuccess ? err : hipGetLastError();
 }
 
-hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *blocks, int n_blocks, const int *Ap,
-                            const int *Ai, const float *Ax, const float *X, float *Y, int N, int accumulate,
+hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const int *Ai, const float *Ax,
+                            const float *X, float *Y, int N, int accumulate, int xcd_chunk_rows,
                             hipStream_t st) {
   if (n_rows <= 0) return hipSuccess;
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
-  int rpb = 0;
-  if (!blocks) {
-    // uniform blocks: a few passes of the lane groups per workgroup, so the staging round
-    // trips are amortised, while the launch still has many more workgroups than compute units
-    rpb = 4 * G;
-    while (rpb > G && (n_rows + rpb - 1) / rpb < 2048) rpb -= G;
-    rpb = std::min(rpb, kBlock);
-    n_blocks = (n_rows + rpb - 1) / rpb;
-  }
-  const int per = per_xcd_of(n_blocks);
-#define CALL(V_, L_)                                                                           \
-  hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(grid_of(n_blocks)), dim3(kBlock), 0, st, rows, \
-                     n_rows, blocks, n_blocks, rpb, per, Ap, Ai, Ax, X, N, Y, N, accumulate)
+  const int n_blocks = (n_rows + G - 1) / G;
+  const int bpc = chunk_bpc(n_blocks, xcd_chunk_rows > 0 ? std::max(1, xcd_chunk_rows / G) : 0);
+#define CALL(V_, L_)                                                                                   \
+  hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(grid_chunked(n_blocks, bpc)), dim3(kBlock), 0, st, \
+                     rows, n_rows, n_blocks, bpc, Ap, Ai, Ax, X, N, Y, N, accumulate)
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
 #undef CALL
   return hipGetLastError();
