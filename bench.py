@@ -72,6 +72,24 @@ def cpu_baseline(cfg, budget_s=20.0):
             "ms": round(best * 1e3, 3)}
 
 
+def calibrate(tf, rows=1 << 20, N=128, reps=5):
+    """A plain copy of known size: Y = I * X through tf_spmm reads X (rows*N*4 bytes) plus the
+    CSR of the identity (12 bytes a row + 4) and writes Y (rows*N*4 bytes), with no reuse.
+    Run under `rocprofv3 --pmc FETCH_SIZE` (then WRITE_SIZE): the ratio of the counter to
+    these byte counts is the factor the counter has to be scaled by."""
+    import scipy.sparse as sp
+    eye = sp.identity(rows, dtype=np.float32, format="csr")
+    A = tf.CsrMatrix.from_scipy(eye).to_device()
+    X = tf.DenseMatrix(rows, N)
+    X.fill(1.0)
+    Y = tf.DenseMatrix(rows, N)
+    for _ in range(reps):
+        tf.spmm(A, X, Y)
+    tf.device_synchronize()
+    print(json.dumps({"calibration_kernel": "spmm_rows_kernel", "launches": reps,
+                      "read_bytes_per_launch": rows * N * 4 + 12 * rows + 4, "write_bytes_per_launch": rows * N * 4}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -87,6 +105,8 @@ def main():
     ap.add_argument("--long-row", type=int, default=0, help="rows with more entries than this are chunked")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the result check")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="run a copy of known size instead (scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
@@ -96,6 +116,9 @@ def main():
     tf = importlib.import_module("tile-fusion_amd")
     w = tf.workloads
     dev = tf.device_init(0)
+    if args.calibrate:
+        calibrate(tf)
+        return
     cfg = w.make_config(args.config)
     A, N, K = cfg["A"], cfg["N"], cfg["K"]
     op = tf.OP_GEMM_SPMM if cfg["op"] == "gemm_spmm" else tf.OP_SPMM_SPMM
