@@ -519,6 +519,21 @@ __global__ __launch_bounds__(kBlock) void gemm_kernel(const float *__restrict__ 
 // the current ones issue.
 constexpr int kGemmBlock = 512;
 
+template <int NB> struct alignas((NB == 1 || NB == 2 || NB == 4) ? 4 * NB : (NB == 8 ? 16 : 4)) wvec { float v[NB]; };
+
+// W in LDS is interleaved so that the NB values a lane feeds to the NB column blocks of one
+// k step are adjacent: element (k, nb*32 + j) sits at (k*32 + j)*NB + nb.  One LDS read per
+// k step then serves all NB MFMAs (16 bytes when NB = 4), and the reads for the next eight
+// values of k are issued before the MFMAs of the current eight.
+template <int NB>
+__device__ __forceinline__ void mfma_step8(const fvec<4> &a, const wvec<NB> (&bw)[4], v16f (&acc)[NB]) {
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[t], bw[t].v[nb], acc[nb], 0, 0, 0);
+}
+
 template <int NB>
 __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__restrict__ X,
                                                                const float *__restrict__ W,
@@ -528,77 +543,113 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
   extern __shared__ __align__(16) float wlds[];
   constexpr int N = NB * 32;
   {
+    // 16 bytes per load, eight loads in flight per thread, then the scatter into LDS
     const int n4 = K * N / 4;
     const fvec<4> *src = reinterpret_cast<const fvec<4> *>(W);
-    fvec<4> *dst = reinterpret_cast<fvec<4> *>(wlds);
-    for (int i = threadIdx.x; i < n4; i += kGemmBlock) dst[i] = src[i];
+    for (int i0 = threadIdx.x; i0 < n4; i0 += 8 * kGemmBlock) {
+      fvec<4> v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * kGemmBlock;
+        v[u] = src[i < n4 ? i : i0];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * kGemmBlock;
+        if (i < n4) {
+          const int e = i * 4, k = e / N, n = e % N;  // four consecutive columns of one column block
+          float *dst = wlds + (k * 32 + (n % 32)) * NB + n / 32;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) dst[c * NB] = v[u].v[c];
+        }
+      }
+    }
   }
   __syncthreads();
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int h = lane / 32, j = lane % 32;
   const int total_waves = gridDim.x * (kGemmBlock / 64);
   const int nrb = (n_rows + 31) / 32;
-  const int groups = K / 32;       // groups of four 8-wide k steps
-  const int tail8 = (K % 32) / 8;  // leftover 8-wide steps
-  for (int rb = blockIdx.x * (kGemmBlock / 64) + wave; rb < nrb; rb += total_waves) {
-    const int q = rb * 32 + j;  // list position whose row this lane feeds as the A operand
-    const bool row_ok = q < n_rows;
-    const int arow = row_ok ? (rows ? rows[q] : q) : 0;
-    const float *Xrow = X + (size_t)arow * K + 4 * h;
+  const int steps = K / 8;  // 8-wide k steps; this lane's rows of W in step s are 8s + 4h + t
+  const wvec<NB> *wl = reinterpret_cast<const wvec<NB> *>(wlds) + (4 * h) * 32 + j;
+  // every wavefront walks one contiguous run of row blocks; run lengths differ by at most one
+  // and the longer runs are spread evenly over the compute units
+  const int gw = blockIdx.x * (kGemmBlock / 64) + wave;
+  const int rb0 = (int)((long long)gw * nrb / total_waves);
+  const int rb_end = (int)((long long)(gw + 1) * nrb / total_waves);
+  // A operand: four 8-wide steps (32 values of k) in registers, the next four in flight --
+  // across row blocks too: the first four steps of the next block are requested before the
+  // current block's results are stored.
+  fvec<4> c0 = vzero<4>(), c1 = c0, c2 = c0, c3 = c0;
+  const float *Xrow = X;
+  bool row_ok = false;
+  if (rb0 < rb_end) {
+    const int q = rb0 * 32 + j;  // list position whose row this lane feeds as the A operand
+    row_ok = q < n_rows;
+    Xrow = X + (size_t)(row_ok ? (rows ? rows[q] : q) : 0) * K + 4 * h;
+    if (row_ok) {
+      c0 = *reinterpret_cast<const fvec<4> *>(Xrow);
+      if (steps > 1) c1 = *reinterpret_cast<const fvec<4> *>(Xrow + 8);
+      if (steps > 2) c2 = *reinterpret_cast<const fvec<4> *>(Xrow + 16);
+      if (steps > 3) c3 = *reinterpret_cast<const fvec<4> *>(Xrow + 24);
+    }
+  }
+  for (int rb = rb0; rb < rb_end; ++rb) {
     v16f acc[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
-    fvec<4> c0 = vzero<4>(), c1 = c0, c2 = c0, c3 = c0;
-    if (groups > 0 && row_ok) {
-      c0 = *reinterpret_cast<const fvec<4> *>(Xrow);
-      c1 = *reinterpret_cast<const fvec<4> *>(Xrow + 8);
-      c2 = *reinterpret_cast<const fvec<4> *>(Xrow + 16);
-      c3 = *reinterpret_cast<const fvec<4> *>(Xrow + 24);
-    }
-    for (int g = 0; g < groups; ++g) {
-      fvec<4> n0 = c0, n1 = c1, n2 = c2, n3 = c3;
-      if (g + 1 < groups && row_ok) {
-        const float *nx = Xrow + (g + 1) * 32;
-        n0 = *reinterpret_cast<const fvec<4> *>(nx);
-        n1 = *reinterpret_cast<const fvec<4> *>(nx + 8);
-        n2 = *reinterpret_cast<const fvec<4> *>(nx + 16);
-        n3 = *reinterpret_cast<const fvec<4> *>(nx + 24);
+    // the row this lane will feed in the wave's next block
+    const int rbn = rb + 1;
+    const int qn = rbn * 32 + j;
+    const bool next_ok = rbn < rb_end && qn < n_rows;
+    const float *Xnext = X + (size_t)(next_ok ? (rows ? rows[qn] : qn) : 0) * K + 4 * h;
+    wvec<NB> bw[4], bn[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) bw[t] = wl[t * 32];
+    for (int s0 = 0; s0 < steps; s0 += 4) {
+      fvec<4> n0 = vzero<4>(), n1 = n0, n2 = n0, n3 = n0;
+      if (s0 + 4 < steps) {
+        if (row_ok) {
+          const float *nx = Xrow + (s0 + 4) * 8;
+          n0 = *reinterpret_cast<const fvec<4> *>(nx);
+          if (s0 + 5 < steps) n1 = *reinterpret_cast<const fvec<4> *>(nx + 8);
+          if (s0 + 6 < steps) n2 = *reinterpret_cast<const fvec<4> *>(nx + 16);
+          if (s0 + 7 < steps) n3 = *reinterpret_cast<const fvec<4> *>(nx + 24);
+        }
+      } else if (next_ok) {  // last group of this block: fetch the next block's first group
+        n0 = *reinterpret_cast<const fvec<4> *>(Xnext);
+        if (steps > 1) n1 = *reinterpret_cast<const fvec<4> *>(Xnext + 8);
+        if (steps > 2) n2 = *reinterpret_cast<const fvec<4> *>(Xnext + 16);
+        if (steps > 3) n3 = *reinterpret_cast<const fvec<4> *>(Xnext + 24);
       }
-      const float *wbase = wlds + (g * 32 + 4 * h) * N + j;
+      // step s0
+      {
+        const int sn = min(s0 + 1, steps - 1);
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < 4; ++t) bn[t] = wl[(8 * sn + t) * 32];
+        mfma_step8<NB>(c0, bw, acc);
+      }
+      if (s0 + 1 < steps) {
+        const int sn = min(s0 + 2, steps - 1);
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(c0.v[t], wbase[t * N + nb * 32], acc[nb], 0, 0, 0);
+        for (int t = 0; t < 4; ++t) bw[t] = wl[(8 * sn + t) * 32];
+        mfma_step8<NB>(c1, bn, acc);
+      }
+      if (s0 + 2 < steps) {
+        const int sn = min(s0 + 3, steps - 1);
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < 4; ++t) bn[t] = wl[(8 * sn + t) * 32];
+        mfma_step8<NB>(c2, bw, acc);
+      }
+      if (s0 + 3 < steps) {
+        const int sn = min(s0 + 4, steps - 1);
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(c1.v[t], wbase[(8 + t) * N + nb * 32], acc[nb], 0, 0, 0);
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(c2.v[t], wbase[(16 + t) * N + nb * 32], acc[nb], 0, 0, 0);
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(c3.v[t], wbase[(24 + t) * N + nb * 32], acc[nb], 0, 0, 0);
+        for (int t = 0; t < 4; ++t) bw[t] = wl[(8 * sn + t) * 32];
+        mfma_step8<NB>(c3, bn, acc);
+      }
       c0 = n0; c1 = n1; c2 = n2; c3 = n3;
-    }
-    for (int m = 0; m < tail8; ++m) {
-      const int kk = groups * 32 + m * 8;
-      fvec<4> a4 = vzero<4>();
-      if (row_ok) a4 = *reinterpret_cast<const fvec<4> *>(Xrow + kk);
-      const float *wbase = wlds + (kk + 4 * h) * N + j;
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.v[t], wbase[t * N + nb * 32], acc[nb], 0, 0, 0);
     }
     // accumulator register r of lane (h, j) holds output row 8*(r/4) + 4*h + r%4, column j
 #pragma unroll
@@ -611,6 +662,8 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
         for (int nb = 0; nb < NB; ++nb) dst[nb * 32] = acc[nb][r];
       }
     }
+    Xrow = Xnext;
+    row_ok = next_ok;
   }
 }
 
@@ -784,7 +837,7 @@ hipError_t launch_gemm(const float *X, const float *W, float *Y, const int *rows
   const int w_bytes = K * N * 4;
   if (w_bytes <= 131072) {
     // W resident in LDS: persistent workgroups, as many per compute unit as the LDS allows
-    const int per_cu = std::max(1, std::min(2, 163840 / w_bytes));
+    const int per_cu = 1;  // register use (accumulators + both operand pipelines) allows one 8-wave workgroup
     const int nrb = (n_rows + 31) / 32;
     const int grid = std::max(1, std::min(compute_units * per_cu, (nrb + kGemmBlock / 64 - 1) / (kGemmBlock / 64)));
 #define CALL(NB_)                                                                               \
