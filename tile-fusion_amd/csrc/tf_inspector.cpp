@@ -156,9 +156,9 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
           if (lds_of(nhi - nlo, e + 1 - s, (long long)Bp[nhi] - Bp[nlo], Wc) > o.lds_budget_bytes) break;
           wlo = nlo; whi = nhi; clo = nclo; chi = nchi; ++e;
         }
-        // (the last tile of the matrix may be short, and then has relatively more halo)
-        if (e == s || (e != M && (e - s < std::min(r_cap, 16) ||
-                                  (float)(whi - wlo) > o.max_redundancy * (float)(e - s)))) { ok = false; break; }
+        // (the last tile of the matrix may be short, and then has relatively more halo: 1.5x the limit)
+        if (e == s || (e != M && e - s < std::min(r_cap, 16)) ||
+            (float)(whi - wlo) > (e == M ? 1.5f : 1.0f) * o.max_redundancy * (float)(e - s)) { ok = false; break; }
         tf::TileDesc t{};
         t.own_begin = s; t.own_end = e; t.prod_begin = wlo; t.prod_end = whi;
         t.wb_begin = t.wb_end = s;
@@ -205,8 +205,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         if (nhi - nlo > p_max) break;
         wlo = nlo; whi = nhi; ++e;
       }
-      const bool halo_ok = (e > s) && (e == M || (e - s >= std::min(r_cap, 16) &&
-                                                 (float)(whi - wlo) <= o.max_redundancy * (float)(e - s)));
+      const bool halo_ok = (e > s) && (e == M || e - s >= std::min(r_cap, 16)) &&
+                           (float)(whi - wlo) <= (e == M ? 1.5f : 1.0f) * o.max_redundancy * (float)(e - s);
       t.cons_begin = (int)S->fused_ids.size();
       if (halo_ok) {
         t.own_begin = s; t.own_end = e; t.prod_begin = wlo; t.prod_end = whi;
