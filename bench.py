@@ -193,6 +193,14 @@ def main():
                      if op == tf.OP_SPMM_SPMM else "fused_gemm_spmm_kernel",
                      "note": "kernel_ms = HIP-event time on the launch stream / steps (all kernels of a step)"},
     }
+    try:  # measured HBM traffic of the dominant kernel, if a committed profile covers this schedule
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            t = json.load(f).get(f"cfg{args.config}")
+        if t and t["kernel"] == out["roofline"]["kernel"] and t["tiles"] == info["n_tiles"]:
+            out["roofline"]["traffic"] = t["fetch_bytes"] + t["write_bytes"]
+            out["roofline"]["traffic_source"] = t["source"]
+    except (OSError, ValueError, KeyError):
+        pass
     if op == tf.OP_GEMM_SPMM:
         gemm_flops = 2.0 * A.shape[1] * K * N
         out["roofline"]["mfma_frac_if_gemm_only"] = round(gemm_flops / (dev_ms * 1e-3) / 1e12 / MFMA_FP32_PEAK_TF, 4)
