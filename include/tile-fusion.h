@@ -128,13 +128,18 @@ class FusedSchedule {
     st_->base = base;
   }
   // The schedule for this operation and these widths (built once, then cached).
-  tf_schedule *get(int op, int N, int K) {
+  // inner_is_outer: SpMM-SpMM whose inner matrix B is A itself (every run of the reference,
+  // fusion/example/SpMM_SpMM_Demo_Utils.h:53-54); lets the inspector build windowed tiles.
+  tf_schedule *get(int op, int N, int K, bool inner_is_outer = false) {
     if (!st_) throw std::runtime_error("FusedSchedule: empty schedule (call inspector first)");
-    auto key = std::make_tuple(op, N, K);
+    auto key = std::make_tuple(op, N, inner_is_outer ? -1 : K);
     auto it = st_->built.find(key);
     if (it == st_->built.end()) {
       tf_inspect_opts o = st_->base;
       o.op = op; o.N = N; o.K = K;
+      if (inner_is_outer && st_->L == st_->M) {
+        o.inner_Ap = st_->Ap.data(); o.inner_Ai = st_->Ai.data(); o.inner_cols = st_->M;
+      }
       tf_schedule *s = nullptr;
       detail::check(tf_inspect(st_->L, st_->M, st_->Ap.data(), st_->Ai.data(), &o, &s), "inspector");
       it = st_->built.emplace(key, std::shared_ptr<tf_schedule>(s, tf_schedule_free)).first;
@@ -212,9 +217,10 @@ struct StagedDense {
 inline void spMMSpMMExecutor(def::CSRMatrix A, def::CSRMatrix B, def::Matrix C, def::Matrix D,
                              def::FusedSchedule schedule, int NumThreads) {
   (void)NumThreads;
-  tf_schedule *s = schedule.get(TF_OP_SPMM_SPMM, C.N, 0);
+  const bool same_arrays = (B.Ap == A.Ap && B.Ai == A.Ai && B.Ax == A.Ax && B.M == A.M && B.N == A.N);
+  tf_schedule *s = schedule.get(TF_OP_SPMM_SPMM, C.N, 0, same_arrays);
   detail_exec::StagedCsr a(A);
-  const bool same = (B.Ap == A.Ap && B.Ai == A.Ai && B.Ax == A.Ax && !B.onDevice());
+  const bool same = same_arrays && (!B.onDevice() || B.device() == A.device());
   detail_exec::StagedCsr b(same ? A : B);
   const tf_csr *bh = same ? a.h : b.h;
   detail_exec::StagedDense c(C), d(D);

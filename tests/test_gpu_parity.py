@@ -139,6 +139,22 @@ def test_spmm_spmm_long_rows(gpu, tf, orc):
     assert np.array_equal(got[ok], oracle_spmm_spmm(orc, A, A, Cd)[ok])  # unsplit rows stay bit-exact
 
 
+def test_spmm_spmm_xcd_chunked_rows(gpu, tf, orc):
+    """3D stencil whose plane distance makes the inspector deal rows to the XCDs in chunks:
+    same bits as the contiguous mapping and as the oracle."""
+    say("spmm_spmm 3D Laplacian, chunked XCD mapping")
+    g, N = 52, 64  # planes 2704 rows apart -> chunks of 320 rows
+    A = tf.workloads.laplacian_3d(g)
+    Cd = tf.workloads.uniform((g ** 3, N), 46)
+    want = oracle_spmm_spmm(orc, A, A, Cd)
+    got, info = run_spmm_spmm(tf, A, A, Cd)
+    assert info["xcd_chunk_rows"] == 320 and info["n_fused_rows"] == 0
+    assert np.array_equal(got, want)
+    for chunk in (-1, 64, 4096):
+        got, info = run_spmm_spmm(tf, A, A, Cd, xcd_chunk_rows=chunk)
+        assert np.array_equal(got, want), chunk
+
+
 def test_laplacian_all_ones_exact_full_size(gpu, tf):
     """The 128^3 Laplacian with an all-ones dense operand (the reference's own input,
     fusion/example/SpMM_SpMM_Demo_Utils.h:53-59): integers throughout, so D must equal the
