@@ -106,7 +106,7 @@ typedef struct {
   int lds_budget_bytes;  /* LDS one fused tile may take; plays the role of the cache budget
                             ScheduleParameters::TileM of the reference's variable-tile
                             inspector.  Default 65536 (81920 when an inner pattern is
-                            given), max 163840.                                               */
+                            given, 131072 for GeMM-SpMM), max 163840.                                               */
   int tile_rows;         /* cap on the rows a tile owns; default: sized so that the launch
                             has about four tiles per compute unit                             */
   float max_redundancy;  /* a tile may compute up to this many intermediate rows per owned

@@ -53,7 +53,7 @@ hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const 
                             const float *, float *, float *, int, int, hipStream_t);
 hipError_t launch_fused_gemm_spmm(const TileDesc *, int, const int *, const float *, const float *,
                                   int, int, const int *, const int *, const float *, float *,
-                                  float *, int, int, int, hipStream_t);
+                                  float *, int, int, int, int, hipStream_t);
 hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t);
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 
@@ -407,7 +407,7 @@ extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_d
   const tf::DeviceSchedule *d = s->dev;
   TF_HIP(tf::launch_fused_gemm_spmm(d->tiles, (int)s->launch_tiles.size(), d->fused_ids, B->d, C->d,
                                     s->opts.K, s->gemm_kc, A->p, A->i, A->x, D->d, d->inter,
-                                    s->opts.N, s->lds_bytes, acc, st));
+                                    s->opts.N, s->lds_bytes, acc, s->opts.compute_units, st));
   if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
     const bool all = (int)s->plain_rows.size() == s->M;
     TF_HIP(tf::launch_gemm(B->d, C->d, d->inter, all ? nullptr : d->plain_rows, (int)s->plain_rows.size(),

@@ -52,7 +52,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     o.K = 0;
   }
   const bool has_inner = o.op == TF_OP_SPMM_SPMM && o.inner_Ap != nullptr;
-  if (o.lds_budget_bytes <= 0) o.lds_budget_bytes = has_inner ? 81920 : 65536;  // two workgroups per CU either way
+  if (o.lds_budget_bytes <= 0)  // two workgroups per CU for the sparse kernels, one for the MFMA tile kernel
+    o.lds_budget_bytes = o.op == TF_OP_GEMM_SPMM ? 131072 : has_inner ? 81920 : 65536;
   if (o.lds_budget_bytes > kMaxLds)
     return tf::fail(TF_EINVAL, "tf_inspect: lds_budget_bytes %d exceeds %d", o.lds_budget_bytes, kMaxLds);
   if (o.max_redundancy <= 0.f) o.max_redundancy = (o.op == TF_OP_GEMM_SPMM) ? 1.5f : 3.0f;
@@ -64,8 +65,12 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   // LDS the tile GEMM needs for staging C, before any slab row.
   int gemm_kc = 0, staging = 0;
   if (o.op == TF_OP_GEMM_SPMM) {
-    const int stage_cap = std::min(32768, o.lds_budget_bytes / 2);
-    gemm_kc = std::min(o.K, std::max(8, (stage_cap / (4 * o.N)) / 8 * 8));
+    if ((long long)o.K * o.N * 4 <= o.lds_budget_bytes / 2) {
+      gemm_kc = o.K;  // W stays resident in LDS next to the slab
+    } else {
+      const int stage_cap = std::min(32768, o.lds_budget_bytes / 2);
+      gemm_kc = std::min(o.K, std::max(8, (stage_cap / (4 * o.N)) / 8 * 8));
+    }
     staging = gemm_kc * o.N * 4;
   }
   const int row_bytes = o.N * 4;
