@@ -106,7 +106,9 @@ typedef struct {
   int lds_budget_bytes;  /* LDS one fused tile may take; plays the role of the cache budget
                             ScheduleParameters::TileM of the reference's variable-tile
                             inspector.  Default 65536 (81920 when an inner pattern is
-                            given, 131072 for GeMM-SpMM), max 163840.                                               */
+                            given; GeMM-SpMM: 163840 when the streamed kernel applies, that
+                            is K <= 256, N <= 128 or K <= 128, and a ring of 256 rows fits),
+                            max 163840.                                                       */
   int tile_rows;         /* cap on the rows a tile owns; default: sized so that the launch
                             has about four tiles per compute unit                             */
   float max_redundancy;  /* a tile may compute up to this many intermediate rows per owned
@@ -162,6 +164,8 @@ typedef struct {
   int windowed;          /* 1 when tiles stage their window of C in LDS             */
   int strip_cols;        /* columns per strip of the windowed kernel, else 0        */
   int xcd_chunk_rows;    /* rows per XCD turn chosen for the row kernels (0: contiguous) */
+  int streamed;          /* 1 when GeMM-SpMM tiles are long runs streamed through an LDS ring */
+  int ring_rows;         /* intermediate rows the ring holds, else 0                 */
   long long fused_nnz;   /* stored entries of A in fused rows (getFusedNnzNum)      */
   long long workspace_bytes; /* device memory the executor keeps (intermediate + partials) */
 } tf_schedule_info;

@@ -45,7 +45,8 @@ class ScheduleInfo(C.Structure):
                 ("n_remainder_rows", C.c_int), ("n_long_rows", C.c_int), ("n_long_chunks", C.c_int),
                 ("n_producer_rows", C.c_int), ("n_writeback_rows", C.c_int),
                 ("max_tile_producer_rows", C.c_int), ("lds_bytes", C.c_int), ("windowed", C.c_int),
-                ("strip_cols", C.c_int), ("xcd_chunk_rows", C.c_int), ("fused_nnz", C.c_longlong), ("workspace_bytes", C.c_longlong)]
+                ("strip_cols", C.c_int), ("xcd_chunk_rows", C.c_int), ("streamed", C.c_int), ("ring_rows", C.c_int),
+                ("fused_nnz", C.c_longlong), ("workspace_bytes", C.c_longlong)]
 
 
 class ScheduleView(C.Structure):

@@ -34,6 +34,9 @@ struct DeviceSchedule {
   int *win = nullptr;
   int *rem_rows = nullptr;
   int *plain_rows = nullptr;
+  int *step_begin = nullptr;  // streamed GeMM-SpMM: per launched tile, first entry in step_ptr
+  int *step_ptr = nullptr;
+  int *fused_rec = nullptr;
   LongChunk *long_chunks = nullptr;
   LongRow *long_rows = nullptr;
   float *inter = nullptr;    // M x N intermediate, only if some tile writes back
@@ -53,7 +56,10 @@ hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const 
                             const float *, float *, float *, int, int, hipStream_t);
 hipError_t launch_fused_gemm_spmm(const TileDesc *, int, const int *, const float *, const float *,
                                   int, int, const int *, const int *, const float *, float *,
-                                  float *, int, int, int, int, hipStream_t);
+                                  float *, int, int, int, int, int, hipStream_t);
+hipError_t launch_fused_gemm_spmm_stream(const TileDesc *, int, const int *, const int *, const int *,
+                                         const float *, const float *, int, int, int, const int *,
+                                         const float *, float *, float *, int, int, hipStream_t);
 hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t);
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 
@@ -90,6 +96,7 @@ void release_device_schedule(DeviceSchedule *d) {
   if (!d) return;
   (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows); (void)hipFree(d->plain_rows);
   (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows);
+  (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
   (void)hipFree(d->inter); (void)hipFree(d->partial);
   delete d;
 }
@@ -121,6 +128,9 @@ static tf_status ensure_device(tf_schedule *s) {
   if (!rc) rc = upload_vec(s->win, &d->win);
   if (!rc) rc = upload_vec(s->rem_rows, &d->rem_rows);
   if (!rc) rc = upload_vec(s->plain_rows, &d->plain_rows);
+  if (!rc) rc = upload_vec(s->launch_step, &d->step_begin);
+  if (!rc) rc = upload_vec(s->step_ptr, &d->step_ptr);
+  if (!rc) rc = upload_vec(s->fused_rec, &d->fused_rec);
   if (!rc) rc = upload_vec(s->long_chunks, &d->long_chunks);
   if (!rc) rc = upload_vec(s->long_rows, &d->long_rows);
   if (!rc && s->n_writeback_rows > 0) {
@@ -405,9 +415,14 @@ extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_d
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
   const tf::DeviceSchedule *d = s->dev;
+  if (s->gemm_stream)
+    TF_HIP(tf::launch_fused_gemm_spmm_stream(d->tiles, (int)s->launch_tiles.size(), d->step_begin, d->step_ptr,
+                                             d->fused_rec, B->d, C->d, s->opts.K, s->opts.N, s->ring_rows,
+                                             A->i, A->x, D->d, d->inter, s->lds_bytes, acc, st));
+  else
   TF_HIP(tf::launch_fused_gemm_spmm(d->tiles, (int)s->launch_tiles.size(), d->fused_ids, B->d, C->d,
                                     s->opts.K, s->gemm_kc, A->p, A->i, A->x, D->d, d->inter,
-                                    s->opts.N, s->lds_bytes, acc, s->opts.compute_units, st));
+                                    s->opts.N, s->lds_bytes, acc, s->opts.compute_units, s->gemm_regw ? 1 : 0, st));
   if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
     const bool all = (int)s->plain_rows.size() == s->M;
     TF_HIP(tf::launch_gemm(B->d, C->d, d->inter, all ? nullptr : d->plain_rows, (int)s->plain_rows.size(),

@@ -52,8 +52,24 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     o.K = 0;
   }
   const bool has_inner = o.op == TF_OP_SPMM_SPMM && o.inner_Ap != nullptr;
-  if (o.lds_budget_bytes <= 0)  // two workgroups per CU for the sparse kernels, one for the MFMA tile kernel
-    o.lds_budget_bytes = o.op == TF_OP_GEMM_SPMM ? 131072 : has_inner ? 81920 : 65536;
+  // GeMM-SpMM tiles keep C in registers when a wavefront's K x 16 slice (two slices when
+  // N > 128) fits 64 registers per lane; LDS then holds only the slab, rows padded by 4 floats.
+  const bool gemm_regw = o.op == TF_OP_GEMM_SPMM && o.K <= 256 &&
+                         (o.K <= 64 ? 4 : o.K <= 128 ? 8 : 16) * (o.N > 128 ? 2 : 1) <= 16;
+  // ... and stream: one workgroup per compute unit walks a long run of rows and keeps the last
+  // ring_rows intermediate rows in LDS (a power of two, at least 256: 64 rows being written,
+  // 64 of alignment slack and a reach of 128 or more).
+  const int stream_fixed = 2 * 64 * 36 * 4 + ((o.K <= 128 && o.N <= 128) ? 8 : 4) * 64 * 8 + (1024 + 4) * 4;  // X staging + consumer scratch + step table (<= 1024 steps)
+  auto ring_for = [&](int budget) {
+    int r = 0;
+    for (int c = 256; c <= 4096 && stream_fixed + (long long)c * (o.N + 4) * 4 <= budget; c *= 2) r = c;
+    return r;
+  };
+  const int ring_rows = gemm_regw ? ring_for(o.lds_budget_bytes > 0 ? o.lds_budget_bytes : kMaxLds) : 0;
+  const bool gemm_stream = ring_rows > 0;
+  if (o.lds_budget_bytes <= 0)  // two workgroups per CU, except for the kernels that own a compute unit
+    o.lds_budget_bytes = o.op == TF_OP_GEMM_SPMM ? (gemm_stream ? kMaxLds : gemm_regw ? 81920 : 131072)
+                                                 : has_inner ? 81920 : 65536;
   if (o.lds_budget_bytes > kMaxLds)
     return tf::fail(TF_EINVAL, "tf_inspect: lds_budget_bytes %d exceeds %d", o.lds_budget_bytes, kMaxLds);
   if (o.max_redundancy <= 0.f) o.max_redundancy = (o.op == TF_OP_GEMM_SPMM) ? 1.5f : 3.0f;
@@ -64,7 +80,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
 
   // LDS the tile GEMM needs for staging C, before any slab row.
   int gemm_kc = 0, staging = 0;
-  if (o.op == TF_OP_GEMM_SPMM) {
+  if (gemm_regw) staging = 2 * 64 * 36 * 4;  // the two X staging buffers of the register-W tile kernel
+  if (o.op == TF_OP_GEMM_SPMM && !gemm_regw) {
     if ((long long)o.K * o.N * 4 <= o.lds_budget_bytes / 2) {
       gemm_kc = o.K;  // W stays resident in LDS next to the slab
     } else {
@@ -73,7 +90,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     }
     staging = gemm_kc * o.N * 4;
   }
-  const int row_bytes = o.N * 4;
+  // (the register-W tile kernel also keeps 16 bytes per fused row behind the slab)
+  const int row_bytes = gemm_regw ? (o.N + 4) * 4 + 16 : o.N * 4;
   const int p_max = (o.lds_budget_bytes - staging) / row_bytes;
   if (p_max < 8)
     return tf::fail(TF_EINVAL, "tf_inspect: LDS budget %d holds only %d intermediate rows of N=%d",
@@ -99,6 +117,10 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     S->M = M;
     S->nnz = nnz;
     S->gemm_kc = gemm_kc;
+    S->gemm_regw = gemm_regw;
+    S->gemm_stream = gemm_stream;
+    S->ring_rows = ring_rows;
+    S->slab_ld = gemm_regw ? o.N + 4 : o.N;
 
     // Column extent of every second-op row (columns need not be sorted).
     std::vector<int> lo(L), hi(L);
@@ -200,6 +222,59 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
 
     int slab_rows = windowed ? S->slab_rows : 0;
     int s = windowed ? M : 0;
+
+    // ---- streamed runs (GeMM-SpMM, C in registers) ----------------------------------------
+    // One run per compute unit.  A run produces the rows [prod_begin, prod_end) in steps of 64
+    // and keeps the last ring_rows of them; a fused row is computed during the step after the
+    // one that produced its last column, and by then its first column must still be in the
+    // ring: with q(c) = (c - prod_begin) / 64 that is q(last) - q(first) <= ring_rows/64 - 2.
+    if (gemm_stream) {
+      int own = std::max(user->tile_rows > 0 ? user->tile_rows : ceil_div(ceil_div(M, o.compute_units), 64) * 64, 64);
+      own = std::min(own, 1000 * 64 - 2 * ring_rows);  // a run's step table holds 1024 steps
+      const int qspan = ring_rows / 64 - 2;
+      while (s < M) {
+        const int e = std::min(M, s + own);
+        tf::TileDesc t{};
+        t.own_begin = s; t.own_end = e; t.prod_begin = s; t.prod_end = e;
+        t.cons_begin = t.cons_end = (int)S->fused_ids.size();
+        t.wb_begin = t.wb_end = s;
+        int hlo = INT_MAX, hhi = -1, useful = 0;
+        auto candidate = [&](int i) {
+          return Ap[i + 1] > Ap[i] && hi[i] - lo[i] <= ring_rows - 64 && lo[i] >= s - ring_rows && hi[i] <= e + ring_rows;
+        };
+        for (int i = s; i < e && i < L; ++i)
+          if (candidate(i)) { hlo = std::min(hlo, lo[i]); hhi = std::max(hhi, hi[i]); }
+        if (hhi > hlo) {
+          const int pb = std::min(hlo, s), pe = std::max(hhi, e);
+          const int steps = ceil_div(pe - pb, 64);
+          std::vector<std::vector<int>> by_step(steps + 1);
+          for (int i = s; i < e && i < L; ++i) {
+            if (!candidate(i)) continue;
+            const int qf = (lo[i] - pb) / 64, ql = (hi[i] - 1 - pb) / 64;
+            if (ql - qf <= qspan) { by_step[ql + 1].push_back(i); ++useful; }
+          }
+          if (4 * useful >= e - s && (float)(steps * 64) <= o.max_redundancy * (float)std::max(e - s, 64)) {
+            t.prod_begin = pb; t.prod_end = pe;
+            S->tile_step.push_back((int)S->step_ptr.size());
+            for (int q = 0; q <= steps; ++q) {
+              S->step_ptr.push_back((int)S->fused_ids.size());
+              for (int i : by_step[q]) { S->fused_ids.push_back(i); fused[i] = 1; }
+            }
+            S->step_ptr.push_back((int)S->fused_ids.size());
+            t.cons_end = (int)S->fused_ids.size();
+            slab_rows = std::max(slab_rows, pe - pb);
+          }
+        }
+        if (t.cons_end == t.cons_begin) S->tile_step.push_back(-1);
+        S->n_producer_rows += t.prod_end - t.prod_begin;
+        S->tiles.push_back(t);
+        s = e;
+      }
+      S->fused_rec.reserve(4 * S->fused_ids.size());
+      for (int i : S->fused_ids) {
+        S->fused_rec.push_back(i); S->fused_rec.push_back(Ap[i]); S->fused_rec.push_back(Ap[i + 1]); S->fused_rec.push_back(0);
+      }
+    }
     while (s < M) {
       tf::TileDesc t{};
       // 1. grow a tile whose producer window covers every fusable row it owns
@@ -322,6 +397,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       const bool fuses = t.cons_end > t.cons_begin;
       if (fuses || !plain_ok) {
         S->launch_tiles.push_back(t);
+        if (gemm_stream) S->launch_step.push_back(S->tile_step[&t - S->tiles.data()]);
         if (a >= 0) S->n_writeback_rows += b - a;
       } else {
         for (int r = t.own_begin; r < t.own_end; ++r)
@@ -330,7 +406,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       }
     }
     S->slab_rows = slab_rows;
-    S->lds_bytes_general = slab_rows * row_bytes + staging;
+    S->lds_bytes_general = gemm_stream ? stream_fixed + ring_rows * (o.N + 4) * 4 : slab_rows * row_bytes + staging;
     if (!windowed) S->lds_bytes = S->lds_bytes_general;
 
     // MultiDimensionalSet-layout view (Fusion_Inspector.h:959-1010).
@@ -397,6 +473,8 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   info->max_tile_producer_rows = s->slab_rows;
   info->lds_bytes = s->lds_bytes;
   info->windowed = s->windowed ? 1 : 0;
+  info->streamed = s->gemm_stream ? 1 : 0;
+  info->ring_rows = s->ring_rows;
   info->strip_cols = s->windowed ? s->opts.strip_cols : 0;
   info->xcd_chunk_rows = s->xcd_chunk_rows;
   info->fused_nnz = s->fused_nnz;
@@ -425,7 +503,7 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
   if (L != s->L || M != s->M || Ap[L] != s->nnz)
     return tf::fail(TF_ESCHEDULE, "schedule was built for %d x %d with %lld entries, got %d x %d with %d",
                     s->L, s->M, s->nnz, L, M, Ap[L]);
-  const int row_bytes = s->opts.N * 4;
+  const int row_bytes = (s->slab_ld > 0 ? s->slab_ld : s->opts.N) * 4 + (s->gemm_regw ? 16 : 0);
   std::vector<int> owner(M, -1), done(L, 0);
   std::vector<char> stored(M, 0);
   int prev_end = 0;
@@ -436,7 +514,32 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
     prev_end = t.own_end;
     if (t.prod_begin > t.own_begin || t.prod_end < t.own_end || t.prod_begin < 0 || t.prod_end > M)
       return tf::fail(TF_ESCHEDULE, "tile %zu: producer range [%d,%d) does not cover owned rows [%d,%d)", ti, t.prod_begin, t.prod_end, t.own_begin, t.own_end);
-    if (!s->windowed && t.cons_end > t.cons_begin &&
+    if (s->gemm_stream && t.cons_end > t.cons_begin) {
+      // rows of step q are computed while rows 64q.. are produced: all their columns were produced
+      // in earlier steps and are still among the last ring_rows - 64 rows
+      const int st = ti < s->tile_step.size() ? s->tile_step[ti] : -1;
+      const int steps = (t.prod_end - t.prod_begin + 63) / 64;
+      if (st < 0 || steps > 1024 || st + steps + 2 > (int)s->step_ptr.size() || s->step_ptr[st] != t.cons_begin ||
+          s->step_ptr[st + steps + 1] != t.cons_end)
+        return tf::fail(TF_ESCHEDULE, "tile %zu: bad step table", ti);
+      for (int q = 0; q <= steps; ++q) {
+        if (s->step_ptr[st + q + 1] < s->step_ptr[st + q])
+          return tf::fail(TF_ESCHEDULE, "tile %zu: step table not monotone at step %d", ti, q);
+        for (int x = s->step_ptr[st + q]; x < s->step_ptr[st + q + 1]; ++x) {
+          const int i = s->fused_ids[x];
+          if (i < 0 || i >= L) return tf::fail(TF_ESCHEDULE, "tile %zu: fused row %d out of range", ti, i);
+          if (s->fused_rec[4 * (size_t)x] != i || s->fused_rec[4 * (size_t)x + 1] != Ap[i] || s->fused_rec[4 * (size_t)x + 2] != Ap[i + 1])
+            return tf::fail(TF_ESCHEDULE, "tile %zu: record of fused row %d does not match the matrix", ti, i);
+          for (int k = Ap[i]; k < Ap[i + 1]; ++k) {
+            if (Ai[k] < t.prod_begin || Ai[k] >= t.prod_end) continue;  // reported below
+            const int qc = (Ai[k] - t.prod_begin) / 64;
+            if (qc > q - 1 || qc < q - s->ring_rows / 64 + 1)
+              return tf::fail(TF_ESCHEDULE, "fused row %d in step %d of tile %zu reads intermediate row %d that is not in the ring then", i, q, ti, Ai[k]);
+          }
+        }
+      }
+    }
+    if (!s->windowed && !s->gemm_stream && t.cons_end > t.cons_begin &&
         (long long)(t.prod_end - t.prod_begin) * row_bytes > s->opts.lds_budget_bytes)
       return tf::fail(TF_ESCHEDULE, "tile %zu: slab of %d rows exceeds the LDS budget", ti, t.prod_end - t.prod_begin);
     if (t.wb_begin < t.own_begin || t.wb_end > t.own_end || t.wb_end < t.wb_begin)

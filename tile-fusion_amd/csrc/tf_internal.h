@@ -47,6 +47,15 @@ struct tf_schedule {
   std::vector<int> win;       // [2*n_tiles] first,last+1 row of C read by the tile's producer rows
   int slab_rows = 0;          // max producer rows of any tile
   int gemm_kc = 0;            // rows of C staged in LDS per step (GeMM-SpMM)
+  bool gemm_regw = false;     // GeMM-SpMM tiles keep C in registers (no staging; slab rows padded)
+  int slab_ld = 0;            // floats between two slab rows of the general / GeMM-SpMM tile kernels
+  bool gemm_stream = false;   // GeMM-SpMM tiles are long runs streamed through a ring of ring_rows slab rows
+  int ring_rows = 0;
+  std::vector<int> tile_step;    // per tile: first entry of its steps in step_ptr (-1: fuses nothing)
+  std::vector<int> launch_step;  // the same for launch_tiles
+  std::vector<int> step_ptr;     // per streamed tile steps+2 offsets into fused_ids: rows of step q are
+                                 // [step_ptr[q], step_ptr[q+1]), computed while rows 64q.. are produced
+  std::vector<int> fused_rec;    // (row, first entry, end, 0) per fused id of a streamed schedule
   std::vector<tf::TileDesc> tiles;
   std::vector<tf::TileDesc> launch_tiles;  // the tiles that fuse something: one workgroup each
   std::vector<int> plain_rows;      // intermediate rows of tiles that fuse nothing, computed by the

@@ -49,6 +49,13 @@ __device__ __forceinline__ int xcd_contiguous(int bid, int bpc) {
   return ((s / bpc) * kXcds + xcd) * bpc + (s % bpc);
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// global load and store of the wavefront, which would cut off the loads a kernel issues
+// ahead of time for a later phase; kernels that prefetch across barriers use this instead.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <int V> struct GlobalRows {
   const float *__restrict__ base;
   int ld;    // row stride in floats
@@ -95,6 +102,17 @@ __device__ __forceinline__ void row_dot_batch(int c, float a, int t, int cnt, bo
   }
 }
 
+// The same for cnt <= LPR entries already in registers: lane g of the group holds entry g.
+template <int V, int LPR, class Src>
+__device__ __forceinline__ void row_dot_loaded(int c, float a, int cnt, bool col_ok, const Src &src,
+                                               fvec<V> &acc) {
+  int t = 0;
+  if constexpr (LPR >= 8)
+    for (; t + 8 <= cnt; t += 8) row_dot_batch<V, LPR, 8>(c, a, t, cnt, col_ok, src, acc);
+  if (t + 4 <= cnt) { row_dot_batch<V, LPR, 4>(c, a, t, cnt, col_ok, src, acc); t += 4; }
+  if (t < cnt) row_dot_batch<V, LPR, 4>(c, a, t, cnt, col_ok, src, acc);
+}
+
 template <int V, int LPR, class Src>
 __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float *__restrict__ val,
                                         int kb, int ke, int glane, bool col_ok, const Src &src,
@@ -104,12 +122,7 @@ __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float
     int c = 0;
     float a = 0.f;
     if (k < ke) { c = idx[k]; a = val[k]; }
-    const int cnt = min(LPR, ke - k0);
-    int t = 0;
-    if constexpr (LPR >= 8)
-      for (; t + 8 <= cnt; t += 8) row_dot_batch<V, LPR, 8>(c, a, t, cnt, col_ok, src, acc);
-    if (t + 4 <= cnt) { row_dot_batch<V, LPR, 4>(c, a, t, cnt, col_ok, src, acc); t += 4; }
-    if (t < cnt) row_dot_batch<V, LPR, 4>(c, a, t, cnt, col_ok, src, acc);
+    row_dot_loaded<V, LPR>(c, a, min(LPR, ke - k0), col_ok, src, acc);
   }
 }
 
@@ -792,6 +805,407 @@ __global__ __launch_bounds__(kGemmBlock) void fused_gemm_spmm_resident_kernel(
   }
 }
 
+// Fused GeMM-SpMM tile kernel with W in registers.  v_mfma_f32_16x16x4_f32: a wavefront
+// owns 16 output columns (CPW such column blocks when N > 128) and keeps its K x 16 slice of
+// W in registers for the whole tile -- lane (j = lane%16, h = lane/16) holds
+// W[16m + 4h + u][16*cb + j] in w[4m + u] -- so LDS holds the slab of intermediate rows and
+// a small staging buffer for X, and two workgroups share a compute unit: one runs its MFMA
+// phase while the other gathers its fused rows out of LDS.
+// X reaches the MFMAs through LDS: the workgroup copies 64 rows x 32 values of k at a time
+// (one 16-byte load per thread, whole cache lines per row) into one of two buffers, two
+// chunks ahead in registers; every wavefront then reads its A operands from there, 16 bytes
+// per lane and four MFMA steps per read: lane (j, h) reads X[row0 + j][16m + 4h .. +4), and
+// both operands use the same permuted k order.  The slab's row stride is N + 4 floats and
+// the staging buffer's 36, which keeps the lanes of a read or store in different banks.
+typedef float v4f __attribute__((ext_vector_type(4)));
+constexpr int kSlabPad = 4;
+constexpr int kXRows = 64, kXChunk = 32, kXLd = kXChunk + 4;
+constexpr int kXStageFloats = 2 * kXRows * kXLd;  // both buffers
+
+template <int KS, int CPW, int LPR>
+__global__ __launch_bounds__(kGemmBlock) void fused_gemm_spmm_regw_kernel(
+    const TileDesc *__restrict__ tiles, int n_tiles, int per_xcd, const int *__restrict__ fused_ids,
+    const float *__restrict__ B, const float *__restrict__ W, int K, int N, const int *__restrict__ Ap,
+    const int *__restrict__ Ai, const float *__restrict__ Ax, float *__restrict__ D, float *__restrict__ T,
+    int accumulate) {
+  extern __shared__ __align__(16) float lds[];
+  static_assert(kGemmBlock * 4 == kXRows * kXChunk, "one 16-byte unit of a chunk per thread");
+  const int tile = xcd_contiguous(blockIdx.x, per_xcd);
+  if (tile >= n_tiles) return;
+  const TileDesc t = tiles[tile];
+  constexpr int NW = kGemmBlock / 64;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int j = lane % 16, h = lane / 16;
+  const int CB = N / 16;  // column blocks
+  // N <= 64 (LPR <= 16): RG wavefronts share a column block and split the four row blocks of a chunk
+  constexpr int RG = CPW == 1 ? (LPR == 8 ? 4 : LPR == 16 ? 2 : 1) : 1;
+  const int cb0 = RG > 1 ? wave % (NW / RG) : wave;
+  const int rg = RG > 1 ? wave / (NW / RG) : 0;
+  const int ld = N + kSlabPad;
+  const int P = t.prod_end - t.prod_begin;
+  const int R = t.cons_end - t.cons_begin;
+  const bool has_cons = R > 0;
+  constexpr int V = 4;
+  constexpr int G = kGemmBlock / LPR;
+  constexpr int RND = 8;  // fused rows per lane group whose entries are fetched ahead of the MFMA phase
+  const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
+  float *xbuf = lds;
+  float *slab = lds + kXStageFloats;
+  // (row, first entry, end) of every fused row of the tile, behind the slab
+  int4 *cinfo = reinterpret_cast<int4 *>(slab + P * ld);
+  for (int x = threadIdx.x; x < R; x += kGemmBlock) {
+    const int i = fused_ids[t.cons_begin + x];
+    cinfo[x] = make_int4(i, Ap[i], Ap[i + 1], 0);
+  }
+
+  // staging role of this thread: 16 bytes of row sr of every chunk
+  const int sr = threadIdx.x / 8, sk = (threadIdx.x % 8) * 4;
+  const int nkc = (K + kXChunk - 1) / kXChunk;
+  const int nchunks = ((P + kXRows - 1) / kXRows) * nkc;
+  auto chunk_unit = [&](int ch) -> fvec<4> {
+    const int q = ch / nkc, k = (ch % nkc) * kXChunk + sk;
+    const int row = t.prod_begin + min(q * kXRows + sr, P - 1);  // rows past the end repeat the last one
+    return (ch < nchunks && k < K) ? *reinterpret_cast<const fvec<4> *>(B + (size_t)row * K + k) : vzero<4>();
+  };
+  fvec<4> x0 = chunk_unit(0), x1 = chunk_unit(1), x2 = chunk_unit(2);
+
+  float w[CPW][KS * 4];
+  if (cb0 < CB) {  // uniform per wavefront
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      const int cb = cb0 + NW * c;
+#pragma unroll
+      for (int m = 0; m < KS; ++m)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int k = 16 * m + 4 * h + u;
+          w[c][4 * m + u] = (cb < CB && k < K) ? W[(size_t)k * N + 16 * cb + j] : 0.f;
+        }
+    }
+  }
+  *reinterpret_cast<fvec<4> *>(xbuf + sr * kXLd + sk) = x0;
+  x0 = x1;
+  x1 = x2;
+  __syncthreads();  // chunk 0 and cinfo visible
+  // The first LPR entries of the rows this lane group will compute are requested now and used
+  // after the MFMA phase: their latency is covered by it.
+  int pc[RND];
+  float pa[RND];
+#pragma unroll
+  for (int r = 0; r < RND; ++r) {
+    pc[r] = 0;
+    pa[r] = 0.f;
+    const int x = r * G + group;
+    if (x < R) {
+      const int4 ci = cinfo[x];
+      const int k = ci.y + glane;
+      if (k < ci.z) { pc[r] = Ai[k]; pa[r] = Ax[k]; }
+    }
+  }
+
+  int ch = 0;
+  for (int r0 = 0; r0 < P; r0 += kXRows) {
+    v4f acc[CPW][4];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) acc[c][b] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kc = 0; kc < KS / 2; ++kc) {
+      if (kc * kXChunk < K) {  // uniform
+        x2 = chunk_unit(ch + 3);
+        const float *xb = xbuf + (ch & 1) * (kXRows * kXLd);
+        if (cb0 < CB) {
+#pragma unroll
+          for (int m2 = 0; m2 < 2; ++m2) {
+            fvec<4> a[4];
+#pragma unroll
+            for (int bi = 0; bi < 4; ++bi)
+              if (bi * RG < 4)
+                a[bi] = *reinterpret_cast<const fvec<4> *>(xb + (16 * (rg + RG * bi) + j) * kXLd + 16 * m2 + 4 * h);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+              for (int bi = 0; bi < 4; ++bi)
+                if (bi * RG < 4) {
+#pragma unroll
+                  for (int c = 0; c < CPW; ++c)
+                    acc[c][bi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[bi].v[u], w[c][4 * (2 * kc + m2) + u],
+                                                                      acc[c][bi], 0, 0, 0);
+                }
+          }
+        }
+        if (ch + 1 < nchunks)
+          *reinterpret_cast<fvec<4> *>(xbuf + ((ch + 1) & 1) * (kXRows * kXLd) + sr * kXLd + sk) = x0;
+        x0 = x1;
+        x1 = x2;
+        ++ch;
+        __syncthreads();
+      }
+    }
+    // accumulator register r of lane (j, h) is output row 4h + r, column j of its block
+    if (cb0 < CB) {
+#pragma unroll
+      for (int bi = 0; bi < 4; ++bi)
+        if (bi * RG < 4) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int lr = r0 + 16 * (rg + RG * bi) + 4 * h + r;
+            if (lr < P) {
+              const int row = t.prod_begin + lr;
+              const bool wb = row >= t.wb_begin && row < t.wb_end;
+#pragma unroll
+              for (int c = 0; c < CPW; ++c) {
+                const int col = 16 * (cb0 + NW * c) + j;
+                if (col < N) {
+                  if (has_cons) slab[lr * ld + col] = acc[c][bi][r];
+                  if (wb) T[(size_t)row * N + col] = acc[c][bi][r];
+                }
+              }
+            }
+          }
+        }
+    }
+  }
+  if (!has_cons) return;
+  __syncthreads();
+  const int coff = glane * V;
+  const bool ok = coff < N;
+  const LdsRows<V> tsrc{slab, ld, ok ? coff : 0, t.prod_begin};
+#pragma unroll
+  for (int r = 0; r < RND; ++r) {
+    const int x = r * G + group;
+    if (x < R) {  // uniform per lane group
+      const int4 ci = cinfo[x];
+      fvec<V> acc = vzero<V>();
+      if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)ci.x * N + coff);
+      row_dot_loaded<V, LPR>(pc[r], pa[r], min(LPR, ci.z - ci.y), ok, tsrc, acc);
+      row_dot<V, LPR>(Ai, Ax, ci.y + LPR, ci.z, glane, ok, tsrc, acc);
+      if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)ci.x * N + coff) = acc;
+    }
+  }
+  for (int x = RND * G + group; x < R; x += G) {
+    const int4 ci = cinfo[x];
+    fvec<V> acc = vzero<V>();
+    if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)ci.x * N + coff);
+    row_dot<V, LPR>(Ai, Ax, ci.y, ci.z, glane, ok, tsrc, acc);
+    if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)ci.x * N + coff) = acc;
+  }
+}
+
+// Streaming fused GeMM-SpMM kernel.  A workgroup walks one long run of intermediate rows,
+// 64 at a time, and keeps only the last `ring_rows` of them in LDS (a ring: row r sits in
+// slot (r - prod_begin) % ring_rows).  Eight producer wavefronts compute the next 64 rows on
+// MFMA exactly as in the tile kernel above (W in registers, X through the staging buffers)
+// while NCW consumer wavefronts compute the fused rows whose last column was produced in
+// the step before -- the schedule lists them step by step -- so the MFMA pipe and the
+// VALU/LDS gather work overlap all the time, W is loaded once per run and no row is computed
+// twice inside a run.  Both kinds of wavefront meet at one barrier per 32 values of k
+// (the staging rhythm: KS/2 intervals per step, the ones past K empty); the consumers spread
+// a step's rows evenly over those intervals.
+// Nothing that is still in flight is ever moved between registers: the staging units
+// alternate between two registers by the parity of the interval, and a consumer lane group
+// keeps one register set per interval of a step -- the (row, first entry, end) record of the
+// row it will compute in the same interval of the next step is requested right after the
+// current row is done, its first LPR entries one interval later.  The entries are turned
+// into (byte offset into the ring, value) pairs in a small per-group LDS area and walked in
+// CSR order with broadcast reads.
+constexpr int kStreamProducers = 8;   // wavefronts
+
+template <int KS, int CPW, int LPR, int NCW>
+__global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm_stream_kernel(
+    const TileDesc *__restrict__ tiles, const int *__restrict__ step_begin, const int *__restrict__ step_ptr,
+    const int4 *__restrict__ fused_rec, const float *__restrict__ B, const float *__restrict__ W, int K, int N,
+    int ring_rows, const int *__restrict__ Ai, const float *__restrict__ Ax, float *__restrict__ D,
+    float *__restrict__ T, int accumulate) {
+  extern __shared__ __align__(16) float lds[];
+  const TileDesc t = tiles[blockIdx.x];
+  constexpr int NW = kStreamProducers;
+  constexpr int NKC = KS / 2;  // intervals per step
+  static_assert(NKC % 2 == 0, "the staging registers alternate by interval parity");
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int ld = N + kSlabPad;
+  const int P = t.prod_end - t.prod_begin;
+  const int S = (P + kXRows - 1) / kXRows;  // production steps
+  float *xbuf = lds;
+  float *ring = lds + kXStageFloats;
+  const int ring_mask = ring_rows - 1;
+  int *sp = reinterpret_cast<int *>(ring + ring_rows * ld) + NCW * 128;  // S + 2 offsets into fused_rec
+  for (int x = threadIdx.x; x < S + 2; x += (NW + NCW) * 64) sp[x] = step_ptr[step_begin[blockIdx.x] + x];
+
+  if (wave < NW) {
+    // ---- producers -------------------------------------------------------------------
+    const int j = lane % 16, h = lane / 16;
+    const int CB = N / 16;
+    constexpr int RG = CPW == 1 ? (LPR == 8 ? 4 : LPR == 16 ? 2 : 1) : 1;
+    const int cb0 = RG > 1 ? wave % (NW / RG) : wave;
+    const int rg = RG > 1 ? wave / (NW / RG) : 0;
+    const int sr = threadIdx.x / 8, sk = (threadIdx.x % 8) * 4;
+    const int nchunks = S * NKC;
+    auto chunk_unit = [&](int ch) -> fvec<4> {
+      const int q = ch / NKC, k = (ch % NKC) * kXChunk + sk;
+      const int row = t.prod_begin + min(q * kXRows + sr, P - 1);
+      return (ch < nchunks && k < K) ? *reinterpret_cast<const fvec<4> *>(B + (size_t)row * K + k) : vzero<4>();
+    };
+    float *const xdst = xbuf + sr * kXLd + sk;
+    {
+      const fvec<4> first = chunk_unit(0);
+      *reinterpret_cast<fvec<4> *>(xdst) = first;
+    }
+    fvec<4> xs[2];  // xs[p]: the unit of the next interval of parity p
+    xs[1] = chunk_unit(1);
+    xs[0] = chunk_unit(2);
+    float w[CPW][KS * 4];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      const int cb = cb0 + NW * c;
+#pragma unroll
+      for (int m = 0; m < KS; ++m)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int k = 16 * m + 4 * h + u;
+          w[c][4 * m + u] = (cb < CB && k < K) ? W[(size_t)k * N + 16 * cb + j] : 0.f;
+        }
+    }
+    lds_barrier();
+    for (int q = 0; q < S; ++q) {
+      v4f acc[CPW][4];
+#pragma unroll
+      for (int c = 0; c < CPW; ++c)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[c][b] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < NKC; ++kc) {
+        const int ch = q * NKC + kc;
+        const float *xb = xbuf + (kc & 1) * (kXRows * kXLd);
+        if (cb0 < CB && kc * kXChunk < K) {  // uniform
+#pragma unroll
+          for (int m2 = 0; m2 < 2; ++m2) {
+            fvec<4> a[4];
+#pragma unroll
+            for (int bi = 0; bi < 4; ++bi)
+              if (bi * RG < 4)
+                a[bi] = *reinterpret_cast<const fvec<4> *>(xb + (16 * (rg + RG * bi) + j) * kXLd + 16 * m2 + 4 * h);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+              for (int bi = 0; bi < 4; ++bi)
+                if (bi * RG < 4) {
+#pragma unroll
+                  for (int c = 0; c < CPW; ++c)
+                    acc[c][bi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[bi].v[u], w[c][4 * (2 * kc + m2) + u],
+                                                                      acc[c][bi], 0, 0, 0);
+                }
+          }
+        }
+        // the unit of the next interval goes to the other buffer, its register takes the unit
+        // three intervals ahead
+        *reinterpret_cast<fvec<4> *>(xdst + ((kc + 1) & 1) * (kXRows * kXLd)) = xs[(kc + 1) & 1];
+        xs[(kc + 1) & 1] = chunk_unit(ch + 3);
+        if (kc == NKC - 1 && cb0 < CB) {
+          // last interval of the step: the 64 new rows go into the ring (and to HBM where the
+          // remainder reads them) before the barrier that lets the consumers at them
+#pragma unroll
+          for (int bi = 0; bi < 4; ++bi)
+            if (bi * RG < 4) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int lr = q * kXRows + 16 * (rg + RG * bi) + 4 * h + r;
+                if (lr < P) {
+                  const int row = t.prod_begin + lr;
+                  const bool wb = row >= t.wb_begin && row < t.wb_end;
+#pragma unroll
+                  for (int c = 0; c < CPW; ++c) {
+                    const int col = 16 * (cb0 + NW * c) + j;
+                    if (col < N) {
+                      ring[(lr & ring_mask) * ld + col] = acc[c][bi][r];
+                      if (wb) T[(size_t)row * N + col] = acc[c][bi][r];
+                    }
+                  }
+                }
+              }
+            }
+        }
+        lds_barrier();
+      }
+    }
+    return;
+  }
+
+  // ---- consumers -----------------------------------------------------------------------
+  constexpr int NG = NCW * 64 / LPR;  // lane groups = fused rows in flight
+  const int ctid = threadIdx.x - NW * 64;
+  const int cg = ctid / LPR, glane = ctid % LPR;
+  const int coff = glane * 4;
+  const bool ok = coff < N;
+  int2 *scratch = reinterpret_cast<int2 *>(ring + ring_rows * ld) + cg * LPR;
+  const char *rbase = reinterpret_cast<const char *>(ring) + (ok ? coff : 0) * 4;
+  // rows of step q handled in its interval kc: an even share of [sp[q], sp[q+1])
+  auto range = [&](int q, int kc, int &b, int &e) {
+    if (q >= S) { b = 0; e = 0; return; }
+    const int c0 = sp[q], len = sp[q + 1] - c0;
+    b = c0 + len * kc / NKC;
+    e = c0 + len * (kc + 1) / NKC;
+  };
+  auto load_rec = [&](int q, int kc) -> int4 {
+    int b, e;
+    range(q, kc, b, e);
+    const int x = b + cg;
+    return x < e ? fused_rec[x] : make_int4(0, 0, 0, 0);
+  };
+  auto row = [&](const int4 rec, int c, float a) {
+    fvec<4> acc = vzero<4>();
+    float *dst = D + (size_t)rec.x * N + coff;
+    if (accumulate && ok) acc = *reinterpret_cast<const fvec<4> *>(dst);
+    for (int k0 = rec.y;;) {
+      scratch[glane] = make_int2(((c - t.prod_begin) & ring_mask) * (ld * 4), __float_as_int(a));
+      acc = lds_row_dot(scratch, 0, min(LPR, rec.z - k0), rbase, acc);
+      k0 += LPR;
+      if (k0 >= rec.z) break;
+      c = 0; a = 0.f;
+      if (k0 + glane < rec.z) { c = Ai[k0 + glane]; a = Ax[k0 + glane]; }
+    }
+    if (ok) *reinterpret_cast<fvec<4> *>(dst) = acc;
+  };
+  auto row_from_memory = [&](int x) {
+    const int4 rec = fused_rec[x];
+    int c = 0;
+    float a = 0.f;
+    if (rec.y + glane < rec.z) { c = Ai[rec.y + glane]; a = Ax[rec.y + glane]; }
+    row(rec, c, a);
+  };
+  lds_barrier();  // step table visible (the producers' first staging unit too)
+  int4 rec[NKC];
+  int pc[NKC];
+  float pa[NKC];
+#pragma unroll
+  for (int kc = 0; kc < NKC; ++kc) rec[kc] = load_rec(0, kc);
+#pragma unroll
+  for (int kc = 0; kc + 1 < NKC; ++kc) {
+    pc[kc] = 0; pa[kc] = 0.f;
+    if (rec[kc].y + glane < rec[kc].z) { pc[kc] = Ai[rec[kc].y + glane]; pa[kc] = Ax[rec[kc].y + glane]; }
+  }
+  for (int q = 0; q < S; ++q) {
+#pragma unroll
+    for (int kc = 0; kc < NKC; ++kc) {
+      {  // entries for the record requested one interval ago
+        constexpr int NKC_ = NKC;
+        const int kp = (kc + NKC_ - 1) % NKC_;
+        pc[kp] = 0; pa[kp] = 0.f;
+        if (rec[kp].y + glane < rec[kp].z) { pc[kp] = Ai[rec[kp].y + glane]; pa[kp] = Ax[rec[kp].y + glane]; }
+      }
+      int b, e;
+      range(q, kc, b, e);
+      if (b + cg < e) row(rec[kc], pc[kc], pa[kc]);
+      for (int x = b + cg + NG; x < e; x += NG) row_from_memory(x);  // more rows than lane groups
+      rec[kc] = load_rec(q + 1, kc);
+      lds_barrier();
+    }
+  }
+  // rows whose last column came with the last step
+  for (int x = sp[S] + cg; x < sp[S + 1]; x += NG) row_from_memory(x);
+}
+
 // ---------------------------------------------------------------------------------
 // Host-side launchers
 // ---------------------------------------------------------------------------------
@@ -931,12 +1345,36 @@ hipError_t launch_long_rows(const LongChunk *chunks, int n_chunks, const LongRow
 hipError_t launch_fused_gemm_spmm(const TileDesc *tiles, int n_tiles, const int *fused_ids,
                                   const float *B, const float *C, int K, int kc, const int *Ap,
                                   const int *Ai, const float *Ax, float *D, float *T, int N,
-                                  int lds_bytes, int accumulate, int compute_units, hipStream_t st) {
+                                  int lds_bytes, int accumulate, int compute_units, int regw,
+                                  hipStream_t st) {
   if (n_tiles <= 0) return hipSuccess;
   const int per = per_xcd_of(n_tiles);
   const int NB = N / 32;
   const int LPR = pick_shape(N).LPR;
   hipError_t err = hipSuccess;
+  if (regw) {
+    // W in registers: K <= 16*KS values of k per lane, CPW column blocks of 16 per wavefront
+    const int KS = K <= 64 ? 4 : K <= 128 ? 8 : 16;
+    const int CPW = N > 128 ? 2 : 1;
+    if (K > 256 || N > 256 || KS * CPW > 16) return hipErrorInvalidValue;
+#define CALL3(KS_, CPW_, L_)                                                                       \
+  err = allow_lds(fused_gemm_spmm_regw_kernel<KS_, CPW_, L_>, lds_bytes);                          \
+  if (err == hipSuccess)                                                                           \
+    hipLaunchKernelGGL((fused_gemm_spmm_regw_kernel<KS_, CPW_, L_>), dim3(grid_of(n_tiles)),       \
+                       dim3(kGemmBlock), lds_bytes, st, tiles, n_tiles, per, fused_ids, B, C, K, N, \
+                       Ap, Ai, Ax, D, T, accumulate)
+#define CALL2(KS_)                                                             \
+  do {                                                                         \
+    if (CPW == 2) { if constexpr (KS_ <= 8) { CALL3(KS_, 2, 64); } }           \
+    else if (LPR == 8) { CALL3(KS_, 1, 8); }                                   \
+    else if (LPR == 16) { CALL3(KS_, 1, 16); }                                 \
+    else { CALL3(KS_, 1, 32); }                                                \
+  } while (0)
+    if (KS == 4) CALL2(4); else if (KS == 8) CALL2(8); else CALL2(16);
+#undef CALL2
+#undef CALL3
+    return err != hipSuccess ? err : hipGetLastError();
+  }
   if (kc == K) {
     // W stays in LDS: persistent workgroups, one per compute unit (a multiple of 8 of them)
     const int n_virtual = grid_of(n_tiles);
@@ -971,6 +1409,38 @@ hipError_t launch_fused_gemm_spmm(const TileDesc *tiles, int n_tiles, const int 
   TF_DISPATCH_NB(NB, CALL);
 #undef CALL
 #undef CALL2
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+hipError_t launch_fused_gemm_spmm_stream(const TileDesc *tiles, int n_tiles, const int *step_begin,
+                                         const int *step_ptr, const int *fused_rec, const float *B,
+                                         const float *C, int K, int N, int ring_rows, const int *Ai,
+                                         const float *Ax, float *D, float *T, int lds_bytes, int accumulate,
+                                         hipStream_t st) {
+  if (n_tiles <= 0) return hipSuccess;
+  const int LPR = pick_shape(N).LPR;
+  const int KS = K <= 64 ? 4 : K <= 128 ? 8 : 16;
+  const int CPW = N > 128 ? 2 : 1;
+  if (K > 256 || N > 256 || KS * CPW > 16 || ring_rows < 256 || (ring_rows & (ring_rows - 1))) return hipErrorInvalidValue;
+  hipError_t err = hipSuccess;
+  const int4 *rec = reinterpret_cast<const int4 *>(fused_rec);
+  // eight consumer wavefronts when the producers' registers allow sixteen wavefronts, else four
+#define CALL3(KS_, CPW_, L_, NCW_)                                                                   \
+  err = allow_lds(fused_gemm_spmm_stream_kernel<KS_, CPW_, L_, NCW_>, lds_bytes);                    \
+  if (err == hipSuccess)                                                                             \
+    hipLaunchKernelGGL((fused_gemm_spmm_stream_kernel<KS_, CPW_, L_, NCW_>), dim3(n_tiles),          \
+                       dim3((kStreamProducers + NCW_) * 64), lds_bytes, st, tiles, step_begin, step_ptr, \
+                       rec, B, C, K, N, ring_rows, Ai, Ax, D, T, accumulate)
+#define CALL2(KS_, NCW_)                                                       \
+  do {                                                                         \
+    if (CPW == 2) { if constexpr (KS_ <= 8) { CALL3(KS_, 2, 64, 4); } }        \
+    else if (LPR == 8) { CALL3(KS_, 1, 8, NCW_); }                             \
+    else if (LPR == 16) { CALL3(KS_, 1, 16, NCW_); }                           \
+    else { CALL3(KS_, 1, 32, NCW_); }                                          \
+  } while (0)
+  if (KS == 4) CALL2(4, 8); else if (KS == 8) CALL2(8, 8); else CALL2(16, 4);
+#undef CALL2
+#undef CALL3
   return err != hipSuccess ? err : hipGetLastError();
 }
 
