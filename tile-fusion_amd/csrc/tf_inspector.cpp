@@ -232,6 +232,13 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       int own = std::max(user->tile_rows > 0 ? user->tile_rows : ceil_div(ceil_div(M, o.compute_units), 64) * 64, 64);
       own = std::min(own, 1000 * 64 - 2 * ring_rows);  // a run's step table holds 1024 steps
       const int qspan = ring_rows / 64 - 2;
+      // What the consumer wavefronts of the kernel take per step without falling behind, and
+      // the longest row a lane group holds in registers.
+      const int lpr = o.N <= 32 ? 8 : o.N <= 64 ? 16 : 32;
+      const int step_cap = ((o.K <= 128 ? 8 : 4) * 64 / lpr) * ((o.K <= 64 ? 4 : o.K <= 128 ? 8 : 16) / 2);
+      const int max_len = 32;
+      S->stream_step_cap = step_cap;
+      S->stream_max_len = max_len;
       while (s < M) {
         const int e = std::min(M, s + own);
         tf::TileDesc t{};
@@ -240,7 +247,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         t.wb_begin = t.wb_end = s;
         int hlo = INT_MAX, hhi = -1, useful = 0;
         auto candidate = [&](int i) {
-          return Ap[i + 1] > Ap[i] && hi[i] - lo[i] <= ring_rows - 64 && lo[i] >= s - ring_rows && hi[i] <= e + ring_rows;
+          return Ap[i + 1] > Ap[i] && Ap[i + 1] - Ap[i] <= max_len && hi[i] - lo[i] <= ring_rows - 64 &&
+                 lo[i] >= s - ring_rows && hi[i] <= e + ring_rows;
         };
         for (int i = s; i < e && i < L; ++i)
           if (candidate(i)) { hlo = std::min(hlo, lo[i]); hhi = std::max(hhi, hi[i]); }
@@ -256,9 +264,21 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
           if (4 * useful >= e - s && (float)(steps * 64) <= o.max_redundancy * (float)std::max(e - s, 64)) {
             t.prod_begin = pb; t.prod_end = pe;
             S->tile_step.push_back((int)S->step_ptr.size());
+            // A step takes at most step_cap rows; the rest wait for the next step if their first
+            // column is still in the ring then, and are left to the remainder otherwise.  The
+            // step after the last production step takes everything.
+            std::vector<int> carry, next;
             for (int q = 0; q <= steps; ++q) {
               S->step_ptr.push_back((int)S->fused_ids.size());
-              for (int i : by_step[q]) { S->fused_ids.push_back(i); fused[i] = 1; }
+              int taken = 0;
+              next.clear();
+              auto place = [&](int i) {
+                if (taken < step_cap || q == steps) { S->fused_ids.push_back(i); fused[i] = 1; ++taken; }
+                else if ((lo[i] - pb) / 64 >= q + 1 - ring_rows / 64 + 1) next.push_back(i);
+              };
+              for (int i : carry) place(i);
+              for (int i : by_step[q]) place(i);
+              carry.swap(next);
             }
             S->step_ptr.push_back((int)S->fused_ids.size());
             t.cons_end = (int)S->fused_ids.size();
@@ -525,9 +545,13 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
       for (int q = 0; q <= steps; ++q) {
         if (s->step_ptr[st + q + 1] < s->step_ptr[st + q])
           return tf::fail(TF_ESCHEDULE, "tile %zu: step table not monotone at step %d", ti, q);
+        if (q < steps && s->step_ptr[st + q + 1] - s->step_ptr[st + q] > s->stream_step_cap)
+          return tf::fail(TF_ESCHEDULE, "tile %zu: step %d has more rows than the consumers take", ti, q);
         for (int x = s->step_ptr[st + q]; x < s->step_ptr[st + q + 1]; ++x) {
           const int i = s->fused_ids[x];
           if (i < 0 || i >= L) return tf::fail(TF_ESCHEDULE, "tile %zu: fused row %d out of range", ti, i);
+          if (Ap[i + 1] - Ap[i] > s->stream_max_len || Ap[i + 1] == Ap[i])
+            return tf::fail(TF_ESCHEDULE, "tile %zu: fused row %d has %d entries", ti, i, Ap[i + 1] - Ap[i]);
           if (s->fused_rec[4 * (size_t)x] != i || s->fused_rec[4 * (size_t)x + 1] != Ap[i] || s->fused_rec[4 * (size_t)x + 2] != Ap[i + 1])
             return tf::fail(TF_ESCHEDULE, "tile %zu: record of fused row %d does not match the matrix", ti, i);
           for (int k = Ap[i]; k < Ap[i + 1]; ++k) {

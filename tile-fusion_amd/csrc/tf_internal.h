@@ -51,6 +51,8 @@ struct tf_schedule {
   int slab_ld = 0;            // floats between two slab rows of the general / GeMM-SpMM tile kernels
   bool gemm_stream = false;   // GeMM-SpMM tiles are long runs streamed through a ring of ring_rows slab rows
   int ring_rows = 0;
+  int stream_step_cap = 0;    // rows a step of a streamed run may hold (all but the last step)
+  int stream_max_len = 0;     // entries a fused row of a streamed run may have
   std::vector<int> tile_step;    // per tile: first entry of its steps in step_ptr (-1: fuses nothing)
   std::vector<int> launch_step;  // the same for launch_tiles
   std::vector<int> step_ptr;     // per streamed tile steps+2 offsets into fused_ids: rows of step q are

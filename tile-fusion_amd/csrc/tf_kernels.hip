@@ -219,6 +219,25 @@ __device__ __forceinline__ fvec<4> lds_row_dot(const int2 *__restrict__ ent, int
   return acc;
 }
 
+// The same with eight entries in flight: all entry reads of a batch are issued, then all
+// gathers, then the fmas -- two LDS round trips per eight entries.  For callers whose row is
+// alone on its lane group's critical path.
+__device__ __forceinline__ fvec<4> lds_row_dot8(const int2 *__restrict__ ent, int kb, int ke,
+                                                const char *base, fvec<4> acc) {
+  int k = kb;
+  for (; k + 8 <= ke; k += 8) {
+    int2 e[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) e[u] = ent[k + u];
+    fvec<4> x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) x[u] = *reinterpret_cast<const fvec<4> *>(base + e[u].x);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) vfma<4>(__int_as_float(e[u].y), x[u], acc);
+  }
+  return lds_row_dot(ent, k, ke, base, acc);
+}
+
 // One 16-byte unit of a strip of the window of C (unit u = row-in-window * LPR + quad).
 // Threads past the end re-read unit 0, which always exists; the value is not used.
 template <int LPR>
@@ -1003,26 +1022,27 @@ __global__ __launch_bounds__(kGemmBlock) void fused_gemm_spmm_regw_kernel(
 // twice inside a run.  Both kinds of wavefront meet at one barrier per 32 values of k
 // (the staging rhythm: KS/2 intervals per step, the ones past K empty); the consumers spread
 // a step's rows evenly over those intervals.
-// Nothing that is still in flight is ever moved between registers: the staging units
-// alternate between two registers by the parity of the interval, and a consumer lane group
+// Nothing that is still in flight is ever moved between registers: a producer thread keeps
+// one staging register per interval of a step (a whole step of X in flight), the barriers
+// wait for LDS traffic only, and a consumer lane group
 // keeps one register set per interval of a step -- the (row, first entry, end) record of the
-// row it will compute in the same interval of the next step is requested right after the
-// current row is done, its first LPR entries one interval later.  The entries are turned
+// row it will compute in the same interval of the next step is requested a step ahead, its
+// first LPR entries half a step ahead, both unconditionally (clamped to existing records).  The entries are turned
 // into (byte offset into the ring, value) pairs in a small per-group LDS area and walked in
 // CSR order with broadcast reads.
 constexpr int kStreamProducers = 8;   // wavefronts
 
-template <int KS, int CPW, int LPR, int NCW>
+template <int KS, int CPW, int LPR, int NCW, bool ACC>
 __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm_stream_kernel(
     const TileDesc *__restrict__ tiles, const int *__restrict__ step_begin, const int *__restrict__ step_ptr,
     const int4 *__restrict__ fused_rec, const float *__restrict__ B, const float *__restrict__ W, int K, int N,
     int ring_rows, const int *__restrict__ Ai, const float *__restrict__ Ax, float *__restrict__ D,
-    float *__restrict__ T, int accumulate) {
+    float *__restrict__ T) {
   extern __shared__ __align__(16) float lds[];
   const TileDesc t = tiles[blockIdx.x];
   constexpr int NW = kStreamProducers;
   constexpr int NKC = KS / 2;  // intervals per step
-  static_assert(NKC % 2 == 0, "the staging registers alternate by interval parity");
+  static_assert(NKC % 2 == 0, "the two LDS staging buffers alternate by interval parity");
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int ld = N + kSlabPad;
   const int P = t.prod_end - t.prod_begin;
@@ -1041,20 +1061,24 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
     const int cb0 = RG > 1 ? wave % (NW / RG) : wave;
     const int rg = RG > 1 ? wave / (NW / RG) : 0;
     const int sr = threadIdx.x / 8, sk = (threadIdx.x % 8) * 4;
-    const int nchunks = S * NKC;
+    // Always a load (of the last row / the last values of k when past the end, zeroed when it
+    // is stored to LDS): a load under a condition would have to land before the next barrier.
     auto chunk_unit = [&](int ch) -> fvec<4> {
-      const int q = ch / NKC, k = (ch % NKC) * kXChunk + sk;
+      const int q = min(ch / NKC, S - 1), k = min((ch % NKC) * kXChunk + sk, K - 4);
       const int row = t.prod_begin + min(q * kXRows + sr, P - 1);
-      return (ch < nchunks && k < K) ? *reinterpret_cast<const fvec<4> *>(B + (size_t)row * K + k) : vzero<4>();
+      return *reinterpret_cast<const fvec<4> *>(B + (size_t)row * K + k);
+    };
+    auto unit_or_zero = [&](const fvec<4> &x, int kc) -> fvec<4> {
+      return kc * kXChunk + sk < K ? x : vzero<4>();
     };
     float *const xdst = xbuf + sr * kXLd + sk;
     {
       const fvec<4> first = chunk_unit(0);
-      *reinterpret_cast<fvec<4> *>(xdst) = first;
+      *reinterpret_cast<fvec<4> *>(xdst) = unit_or_zero(first, 0);
     }
-    fvec<4> xs[2];  // xs[p]: the unit of the next interval of parity p
-    xs[1] = chunk_unit(1);
-    xs[0] = chunk_unit(2);
+    fvec<4> xs[NKC];  // xs[k]: the unit of the next interval k of a step that is not in LDS yet
+#pragma unroll
+    for (int k = 0; k < NKC; ++k) xs[(k + 1) % NKC] = chunk_unit(k + 1);
     float w[CPW][KS * 4];
 #pragma unroll
     for (int c = 0; c < CPW; ++c) {
@@ -1099,9 +1123,9 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
           }
         }
         // the unit of the next interval goes to the other buffer, its register takes the unit
-        // three intervals ahead
-        *reinterpret_cast<fvec<4> *>(xdst + ((kc + 1) & 1) * (kXRows * kXLd)) = xs[(kc + 1) & 1];
-        xs[(kc + 1) & 1] = chunk_unit(ch + 3);
+        // of the same interval of the next step
+        *reinterpret_cast<fvec<4> *>(xdst + ((kc + 1) & 1) * (kXRows * kXLd)) = unit_or_zero(xs[(kc + 1) % NKC], (kc + 1) % NKC);
+        xs[(kc + 1) % NKC] = chunk_unit(ch + 1 + NKC);
         if (kc == NKC - 1 && cb0 < CB) {
           // last interval of the step: the 64 new rows go into the ring (and to HBM where the
           // remainder reads them) before the barrier that lets the consumers at them
@@ -1140,6 +1164,8 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
   const bool ok = coff < N;
   int2 *scratch = reinterpret_cast<int2 *>(ring + ring_rows * ld) + cg * LPR;
   const char *rbase = reinterpret_cast<const char *>(ring) + (ok ? coff : 0) * 4;
+  lds_barrier();  // step table visible (the producers' first staging unit too)
+  const int sp_first = sp[0], sp_last = sp[S + 1];
   // rows of step q handled in its interval kc: an even share of [sp[q], sp[q+1])
   auto range = [&](int q, int kc, int &b, int &e) {
     if (q >= S) { b = 0; e = 0; return; }
@@ -1147,63 +1173,78 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
     b = c0 + len * kc / NKC;
     e = c0 + len * (kc + 1) / NKC;
   };
+  // The record is loaded whether or not the interval has a row for this lane group (the index
+  // is clamped into the run's records): a load under a condition would have to land before
+  // the next barrier, an unconditional one stays in flight.  The row is used only if it exists.
+  const int rec_first = sp_first, rec_last = sp_last - 1;
   auto load_rec = [&](int q, int kc) -> int4 {
     int b, e;
     range(q, kc, b, e);
-    const int x = b + cg;
-    return x < e ? fused_rec[x] : make_int4(0, 0, 0, 0);
+    return fused_rec[min(max(b + cg, rec_first), rec_last)];
   };
-  auto row = [&](const int4 rec, int c, float a) {
+  // A fused row of a streamed schedule has at most EPL * LPR entries (32, or 64 when N > 128
+  // -- the inspector sees to it) and a step has at most NG rows per interval: the steady
+  // state below has no loop and no conditional load, so the loads it issues ahead of time
+  // are waited for only when their registers are read.
+  constexpr int EPL = LPR >= 32 ? 1 : 32 / LPR;  // entries of a row per lane
+  auto row = [&](const int4 rec, const int (&c)[EPL], const float (&a)[EPL]) {
     fvec<4> acc = vzero<4>();
     float *dst = D + (size_t)rec.x * N + coff;
-    if (accumulate && ok) acc = *reinterpret_cast<const fvec<4> *>(dst);
-    for (int k0 = rec.y;;) {
-      scratch[glane] = make_int2(((c - t.prod_begin) & ring_mask) * (ld * 4), __float_as_int(a));
-      acc = lds_row_dot(scratch, 0, min(LPR, rec.z - k0), rbase, acc);
-      k0 += LPR;
-      if (k0 >= rec.z) break;
-      c = 0; a = 0.f;
-      if (k0 + glane < rec.z) { c = Ai[k0 + glane]; a = Ax[k0 + glane]; }
+    if constexpr (ACC) { if (ok) acc = *reinterpret_cast<const fvec<4> *>(dst); }
+#pragma unroll
+    for (int u = 0; u < EPL; ++u) {
+      const int cnt = min(LPR, rec.z - rec.y - u * LPR);
+      if (u == 0 || cnt > 0) {
+        scratch[glane] = make_int2(((c[u] - t.prod_begin) & ring_mask) * (ld * 4), __float_as_int(a[u]));
+        acc = lds_row_dot8(scratch, 0, cnt, rbase, acc);
+      }
     }
     if (ok) *reinterpret_cast<fvec<4> *>(dst) = acc;
   };
-  auto row_from_memory = [&](int x) {
-    const int4 rec = fused_rec[x];
-    int c = 0;
-    float a = 0.f;
-    if (rec.y + glane < rec.z) { c = Ai[rec.y + glane]; a = Ax[rec.y + glane]; }
-    row(rec, c, a);
+  // Entries glane, glane + LPR, .. of a row (lanes past the row's end re-read its last entry;
+  // the row's length decides what is used).
+  auto load_entries = [&](const int4 r, int (&c)[EPL], float (&a)[EPL]) {
+#pragma unroll
+    for (int u = 0; u < EPL; ++u) {
+      const int k = min(r.y + u * LPR + glane, r.z - 1);
+      c[u] = Ai[k];
+      a[u] = Ax[k];
+    }
   };
-  lds_barrier();  // step table visible (the producers' first staging unit too)
+  constexpr int AHEAD = NKC / 2;  // a record is requested NKC intervals ahead, its entries AHEAD
   int4 rec[NKC];
-  int pc[NKC];
-  float pa[NKC];
+  int pc[NKC][EPL];
+  float pa[NKC][EPL];
 #pragma unroll
   for (int kc = 0; kc < NKC; ++kc) rec[kc] = load_rec(0, kc);
 #pragma unroll
-  for (int kc = 0; kc + 1 < NKC; ++kc) {
-    pc[kc] = 0; pa[kc] = 0.f;
-    if (rec[kc].y + glane < rec[kc].z) { pc[kc] = Ai[rec[kc].y + glane]; pa[kc] = Ax[rec[kc].y + glane]; }
-  }
+  for (int kc = 0; kc < AHEAD; ++kc) load_entries(rec[kc], pc[kc], pa[kc]);
   for (int q = 0; q < S; ++q) {
 #pragma unroll
     for (int kc = 0; kc < NKC; ++kc) {
-      {  // entries for the record requested one interval ago
-        constexpr int NKC_ = NKC;
-        const int kp = (kc + NKC_ - 1) % NKC_;
-        pc[kp] = 0; pa[kp] = 0.f;
-        if (rec[kp].y + glane < rec[kp].z) { pc[kp] = Ai[rec[kp].y + glane]; pa[kp] = Ax[rec[kp].y + glane]; }
-      }
+      const int4 cur = rec[kc];
+      int c[EPL];
+      float a[EPL];
+#pragma unroll
+      for (int u = 0; u < EPL; ++u) { c[u] = pc[kc][u]; a[u] = pa[kc][u]; }
+      constexpr int NKC_ = NKC;
+      const int kp = (kc + AHEAD) % NKC_;
+      load_entries(rec[kp], pc[kp], pa[kp]);
+      rec[kc] = load_rec(q + 1, kc);
       int b, e;
       range(q, kc, b, e);
-      if (b + cg < e) row(rec[kc], pc[kc], pa[kc]);
-      for (int x = b + cg + NG; x < e; x += NG) row_from_memory(x);  // more rows than lane groups
-      rec[kc] = load_rec(q + 1, kc);
+      if (b + cg < e) row(cur, c, a);
       lds_barrier();
     }
   }
   // rows whose last column came with the last step
-  for (int x = sp[S] + cg; x < sp[S + 1]; x += NG) row_from_memory(x);
+  for (int x = sp[S] + cg; x < sp[S + 1]; x += NG) {
+    const int4 r = fused_rec[x];
+    int c[EPL];
+    float a[EPL];
+    load_entries(r, c, a);
+    row(r, c, a);
+  }
 }
 
 // ---------------------------------------------------------------------------------
@@ -1421,26 +1462,28 @@ hipError_t launch_fused_gemm_spmm_stream(const TileDesc *tiles, int n_tiles, con
   const int LPR = pick_shape(N).LPR;
   const int KS = K <= 64 ? 4 : K <= 128 ? 8 : 16;
   const int CPW = N > 128 ? 2 : 1;
-  if (K > 256 || N > 256 || KS * CPW > 16 || ring_rows < 256 || (ring_rows & (ring_rows - 1))) return hipErrorInvalidValue;
+  if (K > 256 || N > 128 || CPW != 1 || ring_rows < 256 || (ring_rows & (ring_rows - 1))) return hipErrorInvalidValue;
   hipError_t err = hipSuccess;
   const int4 *rec = reinterpret_cast<const int4 *>(fused_rec);
   // eight consumer wavefronts when the producers' registers allow sixteen wavefronts, else four
-#define CALL3(KS_, CPW_, L_, NCW_)                                                                   \
-  err = allow_lds(fused_gemm_spmm_stream_kernel<KS_, CPW_, L_, NCW_>, lds_bytes);                    \
+#define CALL4(KS_, L_, NCW_, ACC_)                                                                   \
+  err = allow_lds(fused_gemm_spmm_stream_kernel<KS_, 1, L_, NCW_, ACC_>, lds_bytes);                 \
   if (err == hipSuccess)                                                                             \
-    hipLaunchKernelGGL((fused_gemm_spmm_stream_kernel<KS_, CPW_, L_, NCW_>), dim3(n_tiles),          \
+    hipLaunchKernelGGL((fused_gemm_spmm_stream_kernel<KS_, 1, L_, NCW_, ACC_>), dim3(n_tiles),       \
                        dim3((kStreamProducers + NCW_) * 64), lds_bytes, st, tiles, step_begin, step_ptr, \
-                       rec, B, C, K, N, ring_rows, Ai, Ax, D, T, accumulate)
+                       rec, B, C, K, N, ring_rows, Ai, Ax, D, T)
+#define CALL3(KS_, L_, NCW_)                                                   \
+  do { if (accumulate) { CALL4(KS_, L_, NCW_, true); } else { CALL4(KS_, L_, NCW_, false); } } while (0)
 #define CALL2(KS_, NCW_)                                                       \
   do {                                                                         \
-    if (CPW == 2) { if constexpr (KS_ <= 8) { CALL3(KS_, 2, 64, 4); } }        \
-    else if (LPR == 8) { CALL3(KS_, 1, 8, NCW_); }                             \
-    else if (LPR == 16) { CALL3(KS_, 1, 16, NCW_); }                           \
-    else { CALL3(KS_, 1, 32, NCW_); }                                          \
+    if (LPR == 8) { CALL3(KS_, 8, NCW_); }                                     \
+    else if (LPR == 16) { CALL3(KS_, 16, NCW_); }                              \
+    else { CALL3(KS_, 32, NCW_); }                                             \
   } while (0)
   if (KS == 4) CALL2(4, 8); else if (KS == 8) CALL2(8, 8); else CALL2(16, 4);
 #undef CALL2
 #undef CALL3
+#undef CALL4
   return err != hipSuccess ? err : hipGetLastError();
 }
 
