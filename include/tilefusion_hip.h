@@ -186,6 +186,15 @@ typedef struct {
   const int *ptr1, *ptr2, *ker_begin, *id, *type;
   const int *tile_range;
   const int *writeback; /* [2*n_tiles] begin,end of intermediate rows a tile stores to HBM */
+  /* Streamed GeMM-SpMM schedules only (else null / 0): a tile is a long run produced 64 rows
+     a step; tile_step[t] = first entry of tile t in step_ptr, or -1 if it fuses nothing.  With
+     steps = ceil((producer_end - producer_begin) / 64), the fused rows computed while step q
+     is produced are fused ids [step_ptr[tile_step[t] + q], step_ptr[tile_step[t] + q + 1])
+     of the tile, q = 0..steps (step `steps` comes after the last production step); offsets
+     count from the tile's first fused id, i.e. from id[ker_begin[2t]]. */
+  const int *tile_step;
+  const int *step_ptr;
+  int n_step_ptr;
 } tf_schedule_view;
 
 tf_status tf_schedule_get_view(const tf_schedule *s, tf_schedule_view *view);

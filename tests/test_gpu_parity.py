@@ -298,6 +298,46 @@ def test_gemm_spmm_reductions_and_accumulate(gpu, tf, orc):
     assert orc.rel_err(acc, D0.astype(np.float64) + base) <= 1e-6
 
 
+@pytest.mark.parametrize("K,N", [(128, 128), (64, 128), (256, 128), (8, 96), (256, 64), (64, 64), (32, 32)])
+def test_gemm_spmm_streamed(gpu, tf, orc, K, N):
+    """Long matrices take the streamed kernel: every banded row fused out of the LDS ring; rows
+    with more than 32 entries or a far column go through the remainder and read the rows the
+    runs write back; D += is a separate instantiation."""
+    say(f"gemm_spmm streamed K={K} N={N}")
+    M = 36000
+    A0 = tf.workloads.banded_random(M, 32, 16, seed=70)
+    rng = np.random.default_rng(71 + K + N)
+    B = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    Cd = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    want, _ = orc.gemm_spmm(A0, B, Cd, orc.unfused_schedule(M), nthreads=8)
+    got, info = run_gemm_spmm(tf, A0, B, Cd, compute_units=256)
+    assert info["streamed"] == 1 and info["n_fused_rows"] == M and info["n_writeback_rows"] == 0
+    assert orc.rel_err(got, want) <= TOL
+    lil = A0.tolil()
+    for i in rng.choice(M, 40, replace=False):
+        lo = max(0, i - 30)
+        lil[i, lo:lo + 40] = 0.5
+    for i in rng.choice(M, 40, replace=False):
+        lil[i, (i + M // 3) % M] = -2.0
+    lil[M // 2] = 0  # an empty row
+    A = sp.csr_matrix(lil, dtype=np.float32)
+    A.eliminate_zeros()
+    want, _ = orc.gemm_spmm(A, B, Cd, orc.unfused_schedule(M), nthreads=8)
+    got, info = run_gemm_spmm(tf, A, B, Cd, compute_units=256)
+    assert info["streamed"] == 1 and 0 < info["n_remainder_rows"] <= 81 and info["n_writeback_rows"] > 0
+    assert orc.rel_err(got, want) <= TOL
+    D0 = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    acc, _ = run_gemm_spmm(tf, A, B, Cd, accumulate=True, D0=D0, compute_units=256)
+    assert orc.rel_err(acc, D0.astype(np.float64) + want) <= TOL
+    Bi = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    Ci = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    Ai = A0.copy()
+    Ai.data = rng.integers(-2, 3, Ai.nnz).astype(np.float32)
+    exact = (Ai.astype(np.int64) @ (Bi.astype(np.int64) @ Ci.astype(np.int64))).astype(np.float32)
+    got, _ = run_gemm_spmm(tf, Ai, Bi, Ci, compute_units=256)
+    assert np.array_equal(got, exact)  # integer operands: exact whatever the summation order
+
+
 def test_power_law_row_sums_full_size(gpu, tf):
     """2^21-node R-MAT, row-normalised: with all-ones B (M x 128) and C (128 x 128) the
     intermediate is 128 everywhere, so D is 128 on every non-empty row and 0 on empty ones."""

@@ -31,7 +31,23 @@ def validate(view, info, A, lds_budget):
         assert kb[2 * t + 1] == ptr2[t + 1]
         assert np.array_equal(own, np.arange(ob, oe))
         assert np.all(typ[ptr2[t]:kb[2 * t]] == 0) and np.all(typ[kb[2 * t]:kb[2 * t + 1]] == 1)
-        if len(fused):
+        if len(fused) and info["streamed"]:
+            # a streamed run is produced 64 rows a step into a ring of ring_rows rows: a row of
+            # step q is computed while rows pb + 64q .. are produced, so all its columns come from
+            # earlier steps and lie within the last ring_rows - 64 rows
+            ring = info["ring_rows"]
+            assert ring >= 256 and ring % 64 == 0 and ring * (info["N"] + 4) * 4 <= lds_budget
+            st = view["tile_step"][t]
+            steps = -(-(pe - pb) // 64)
+            sp_ = view["step_ptr"][st:st + steps + 2]
+            assert st >= 0 and sp_[0] == 0 and sp_[-1] == len(fused) and np.all(np.diff(sp_) >= 0)
+            for q in range(steps + 1):
+                for i in fused[sp_[q]:sp_[q + 1]]:
+                    cols = A.indices[A.indptr[i]:A.indptr[i + 1]]
+                    assert 0 < len(cols) <= 32
+                    qc = (cols - pb) // 64
+                    assert qc.max() <= q - 1 and qc.min() >= q - ring // 64 + 1, f"row {i} step {q}"
+        elif len(fused):
             assert (pe - pb) * info["N"] * 4 <= lds_budget
         for i in fused:
             cols = A.indices[A.indptr[i]:A.indptr[i + 1]]
@@ -203,3 +219,44 @@ def test_far_stencil_distance_sets_xcd_chunk(tf):
     assert tf.inspector(tf.CsrMatrix.from_scipy(A), 1, op=tf.OP_SPMM_SPMM, N=64).info()["xcd_chunk_rows"] == 512
     A = tf.workloads.erdos_renyi_gcn(20000, 10.0, seed=5)  # random graph: no dominant distance
     assert tf.inspector(tf.CsrMatrix.from_scipy(A), 1, op=tf.OP_SPMM_SPMM, N=64).info()["xcd_chunk_rows"] == 0
+
+
+def test_streamed_runs(tf):
+    """GeMM-SpMM on a long banded matrix: one run per compute unit, every row fused, rows listed
+    step by step at no more than 64 a step, no halo beyond the band; denser and far-reaching
+    rows are left to the remainder and their intermediate rows written back."""
+    M = 40000
+    A = tf.workloads.banded_random(M, 32, 16, seed=5)
+    S, view, info = inspect(tf, A, op=tf.OP_GEMM_SPMM, N=128, K=128, compute_units=256)
+    validate(view, info, A, 163840)
+    assert info["streamed"] == 1 and info["ring_rows"] == 256
+    assert info["n_fused_rows"] == M and info["n_writeback_rows"] == 0
+    tr = view["tile_range"]
+    assert len(tr) == M // 256 and np.all(tr[:, 2] - tr[:, 0] <= 16) and np.all(tr[:, 1] - tr[:, 3] <= 16)
+    for t in range(len(tr)):
+        st = view["tile_step"][t]
+        steps = -(-(tr[t][1] - tr[t][0]) // 64)
+        assert np.all(np.diff(view["step_ptr"][st:st + steps + 1]) <= 64)
+    # a matrix too short to give every compute unit a run keeps the tile kernel
+    S2, _, info2 = inspect(tf, tf.workloads.banded_random(4096, 32, 16, seed=5), op=tf.OP_GEMM_SPMM, N=128, K=128, compute_units=256)
+    assert info2["streamed"] == 0 and info2["n_fused_rows"] == 4096
+    # rows the stream cannot take: more than 32 entries, or a column far away
+    rng = np.random.default_rng(6)
+    B = A.tolil()
+    dense_rows = rng.choice(M, 50, replace=False)
+    for i in dense_rows:
+        lo = max(0, i - 30)
+        B[i, lo:lo + 40] = 1.0
+    far_rows = rng.choice(M, 50, replace=False)
+    for i in far_rows:
+        B[i, (i + M // 2) % M] = 2.0
+    B = sp.csr_matrix(B, dtype=np.float32)
+    S3, view3, info3 = inspect(tf, B, op=tf.OP_GEMM_SPMM, N=128, K=128, compute_units=256)
+    validate(view3, info3, B, 163840)
+    out = set(dense_rows.tolist()) | set(far_rows.tolist())
+    assert info3["streamed"] == 1 and info3["n_remainder_rows"] == len(out) and info3["n_writeback_rows"] > 0
+    # wider rows and narrower rings: N = 32 holds a ring of 1024 rows, and K = 256 halves the consumers
+    for N, K in ((32, 64), (64, 256), (96, 8)):
+        S4, view4, info4 = inspect(tf, A, op=tf.OP_GEMM_SPMM, N=N, K=K, compute_units=256)
+        validate(view4, info4, A, 163840)
+        assert info4["streamed"] == 1 and info4["n_fused_rows"] == M

@@ -54,7 +54,8 @@ class ScheduleView(C.Structure):
                 ("ptr1", C.POINTER(C.c_int)), ("ptr2", C.POINTER(C.c_int)),
                 ("ker_begin", C.POINTER(C.c_int)), ("id", C.POINTER(C.c_int)),
                 ("type", C.POINTER(C.c_int)), ("tile_range", C.POINTER(C.c_int)),
-                ("writeback", C.POINTER(C.c_int))]
+                ("writeback", C.POINTER(C.c_int)), ("tile_step", C.POINTER(C.c_int)),
+                ("step_ptr", C.POINTER(C.c_int)), ("n_step_ptr", C.c_int)]
 
 
 _PI = C.POINTER(C.c_int)
@@ -276,7 +277,9 @@ class FusedSchedule:
         return {"n1_": v.n1, "ptr1_": arr(v.ptr1, 3), "ptr2_": arr(v.ptr2, P + 1),
                 "ker_begin_": arr(v.ker_begin, 2 * P), "id_": arr(v.id, nid), "type_": arr(v.type, nid),
                 "tile_range": arr(v.tile_range, 4 * nt).reshape(nt, 4),
-                "writeback": arr(v.writeback, 2 * nt).reshape(nt, 2)}
+                "writeback": arr(v.writeback, 2 * nt).reshape(nt, 2),
+                "tile_step": arr(v.tile_step, nt) if v.n_step_ptr else None,
+                "step_ptr": arr(v.step_ptr, v.n_step_ptr) if v.n_step_ptr else None}
 
     def validate(self, A=None):
         A = A or self._A

@@ -65,14 +65,19 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     for (int c = 256; c <= 4096 && stream_fixed + (long long)c * (o.N + 4) * 4 <= budget; c *= 2) r = c;
     return r;
   };
-  const int ring_rows = gemm_regw ? ring_for(o.lds_budget_bytes > 0 ? o.lds_budget_bytes : kMaxLds) : 0;
+  // (a run needs a few hundred rows to pay for its start-up and halo: with fewer than 128 rows
+  // per compute unit the tile kernel, which spreads over all of them, is the faster one)
+  if (o.compute_units <= 0) o.compute_units = tf::default_compute_units();
+  const bool long_enough = user->tile_rows > 0 || M >= 128LL * o.compute_units;
+  const int ring_rows = gemm_regw && long_enough ? ring_for(o.lds_budget_bytes > 0 ? o.lds_budget_bytes : kMaxLds) : 0;
   const bool gemm_stream = ring_rows > 0;
   if (o.lds_budget_bytes <= 0)  // two workgroups per CU, except for the kernels that own a compute unit
     o.lds_budget_bytes = o.op == TF_OP_GEMM_SPMM ? (gemm_stream ? kMaxLds : gemm_regw ? 81920 : 131072)
                                                  : has_inner ? 81920 : 65536;
   if (o.lds_budget_bytes > kMaxLds)
     return tf::fail(TF_EINVAL, "tf_inspect: lds_budget_bytes %d exceeds %d", o.lds_budget_bytes, kMaxLds);
-  if (o.max_redundancy <= 0.f) o.max_redundancy = (o.op == TF_OP_GEMM_SPMM) ? 1.5f : 3.0f;
+  // (recomputed GEMM rows cost MFMA time, unless the matrix is too short to fill the device anyway)
+  if (o.max_redundancy <= 0.f) o.max_redundancy = (o.op == TF_OP_GEMM_SPMM && long_enough) ? 1.5f : 3.0f;
   if (o.max_redundancy < 1.f) o.max_redundancy = 1.f;
   if (o.long_row_nnz <= 0) o.long_row_nnz = 32;
   if (o.long_row_nnz > 2048) o.long_row_nnz = 2048;  // a row must fit one staging batch of the row kernel
@@ -229,18 +234,21 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     // one that produced its last column, and by then its first column must still be in the
     // ring: with q(c) = (c - prod_begin) / 64 that is q(last) - q(first) <= ring_rows/64 - 2.
     if (gemm_stream) {
-      int own = std::max(user->tile_rows > 0 ? user->tile_rows : ceil_div(ceil_div(M, o.compute_units), 64) * 64, 64);
+      int own = user->tile_rows > 0 ? std::max(user->tile_rows, 64)
+                                     : std::max(ceil_div(ceil_div(M, o.compute_units), 64) * 64, 256);  // short runs are mostly halo
       own = std::min(own, 1000 * 64 - 2 * ring_rows);  // a run's step table holds 1024 steps
       const int qspan = ring_rows / 64 - 2;
       // What the consumer wavefronts of the kernel take per step without falling behind, and
       // the longest row a lane group holds in registers.
       const int lpr = o.N <= 32 ? 8 : o.N <= 64 ? 16 : 32;
-      const int step_cap = ((o.K <= 128 ? 8 : 4) * 64 / lpr) * ((o.K <= 64 ? 4 : o.K <= 128 ? 8 : 16) / 2);
+      const int per_round = ((o.K <= 128 ? 8 : 4) * 64 / lpr) * ((o.K <= 64 ? 4 : o.K <= 128 ? 8 : 16) / 2);
+      const int step_cap = per_round * ceil_div(64, per_round);  // lane groups x intervals x rows per interval
       const int max_len = 32;
       S->stream_step_cap = step_cap;
       S->stream_max_len = max_len;
       while (s < M) {
-        const int e = std::min(M, s + own);
+        int e = std::min(M, s + own);
+        if (M - e < own / 2) e = M;  // a short last run would be mostly halo: the one before takes its rows
         tf::TileDesc t{};
         t.own_begin = s; t.own_end = e; t.prod_begin = s; t.prod_end = e;
         t.cons_begin = t.cons_end = (int)S->fused_ids.size();
@@ -285,7 +293,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
             slab_rows = std::max(slab_rows, pe - pb);
           }
         }
-        if (t.cons_end == t.cons_begin) S->tile_step.push_back(-1);
+        if ((int)S->tile_step.size() == (int)S->tiles.size()) S->tile_step.push_back(-1);  // nothing streamed here
         S->n_producer_rows += t.prod_end - t.prod_begin;
         S->tiles.push_back(t);
         s = e;
@@ -464,6 +472,15 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       S->ker_begin[2 * p + 1] = (int)S->id.size();
       S->ptr2[p + 1] = (int)S->id.size();
     }
+    if (gemm_stream) {  // step offsets relative to each tile's first fused id, for the view
+      S->view_step_ptr = S->step_ptr;
+      for (size_t ti = 0; ti < S->tiles.size(); ++ti) {
+        const int st = S->tile_step[ti];
+        if (st < 0) continue;
+        const int steps = (S->tiles[ti].prod_end - S->tiles[ti].prod_begin + 63) / 64;
+        for (int q = 0; q <= steps + 1; ++q) S->view_step_ptr[st + q] -= S->tiles[ti].cons_begin;
+      }
+    }
   } catch (const std::bad_alloc &) {
     delete S;
     return tf::fail(TF_ENOMEM, "tf_inspect: out of host memory");
@@ -514,6 +531,9 @@ extern "C" tf_status tf_schedule_get_view(const tf_schedule *s, tf_schedule_view
   v->ptr1 = s->ptr1.data(); v->ptr2 = s->ptr2.data(); v->ker_begin = s->ker_begin.data();
   v->id = s->id.data(); v->type = s->type.data();
   v->tile_range = s->tile_range.data(); v->writeback = s->writeback.data();
+  v->tile_step = s->gemm_stream ? s->tile_step.data() : nullptr;
+  v->step_ptr = s->gemm_stream ? s->view_step_ptr.data() : nullptr;
+  v->n_step_ptr = s->gemm_stream ? (int)s->view_step_ptr.size() : 0;
   return TF_OK;
 }
 

@@ -57,6 +57,7 @@ struct tf_schedule {
   std::vector<int> launch_step;  // the same for launch_tiles
   std::vector<int> step_ptr;     // per streamed tile steps+2 offsets into fused_ids: rows of step q are
                                  // [step_ptr[q], step_ptr[q+1]), computed while rows 64q.. are produced
+  std::vector<int> view_step_ptr;  // step_ptr with offsets counted from each tile's first fused id
   std::vector<int> fused_rec;    // (row, first entry, end, 0) per fused id of a streamed schedule
   std::vector<tf::TileDesc> tiles;
   std::vector<tf::TileDesc> launch_tiles;  // the tiles that fuse something: one workgroup each

@@ -1166,10 +1166,8 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
   const char *rbase = reinterpret_cast<const char *>(ring) + (ok ? coff : 0) * 4;
   lds_barrier();  // step table visible (the producers' first staging unit too)
   const int sp_first = sp[0], sp_last = sp[S + 1];
-  // rows of step q handled in its interval kc: an even share of [sp[q], sp[q+1])
-  auto range = [&](int q, int kc, int &b, int &e) {
-    if (q >= S) { b = 0; e = 0; return; }
-    const int c0 = sp[q], len = sp[q + 1] - c0;
+  // Rows of a step [c0, c0 + len) handled in its interval kc: an even share.
+  auto share = [&](int c0, int len, int kc, int &b, int &e) {
     b = c0 + len * kc / NKC;
     e = c0 + len * (kc + 1) / NKC;
   };
@@ -1177,10 +1175,10 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
   // is clamped into the run's records): a load under a condition would have to land before
   // the next barrier, an unconditional one stays in flight.  The row is used only if it exists.
   const int rec_first = sp_first, rec_last = sp_last - 1;
-  auto load_rec = [&](int q, int kc) -> int4 {
+  auto load_rec = [&](int c0, int len, int kc, int r) -> int4 {
     int b, e;
-    range(q, kc, b, e);
-    return fused_rec[min(max(b + cg, rec_first), rec_last)];
+    share(c0, len, kc, b, e);
+    return fused_rec[min(max(b + cg + NG * r, rec_first), rec_last)];
   };
   // A fused row of a streamed schedule has at most EPL * LPR entries (32, or 64 when N > 128
   // -- the inspector sees to it) and a step has at most NG rows per interval: the steady
@@ -1212,30 +1210,49 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
     }
   };
   constexpr int AHEAD = NKC / 2;  // a record is requested NKC intervals ahead, its entries AHEAD
-  int4 rec[NKC];
-  int pc[NKC][EPL];
-  float pa[NKC][EPL];
+  // rows a lane group computes per interval so that a step's 64 new rows are taken in one step
+  constexpr int RPI = (kXRows + NG * NKC - 1) / (NG * NKC);
+  int4 rec[NKC][RPI];
+  int pc[NKC][RPI][EPL];
+  float pa[NKC][RPI][EPL];
 #pragma unroll
-  for (int kc = 0; kc < NKC; ++kc) rec[kc] = load_rec(0, kc);
+  for (int kc = 0; kc < NKC; ++kc)
 #pragma unroll
-  for (int kc = 0; kc < AHEAD; ++kc) load_entries(rec[kc], pc[kc], pa[kc]);
+    for (int r = 0; r < RPI; ++r) rec[kc][r] = load_rec(sp_first, sp[1] - sp_first, kc, r);
+#pragma unroll
+  for (int kc = 0; kc < AHEAD; ++kc)
+#pragma unroll
+    for (int r = 0; r < RPI; ++r) load_entries(rec[kc][r], pc[kc][r], pa[kc][r]);
+  int s0 = sp_first, s1 = sp[1];  // rows of step q are [s0, s1)
   for (int q = 0; q < S; ++q) {
+    const int s2 = q + 1 < S ? sp[q + 2] : s1;  // rows of the next production step: [s1, s2)
 #pragma unroll
     for (int kc = 0; kc < NKC; ++kc) {
-      const int4 cur = rec[kc];
-      int c[EPL];
-      float a[EPL];
+      int4 cur[RPI];
+      int c[RPI][EPL];
+      float a[RPI][EPL];
 #pragma unroll
-      for (int u = 0; u < EPL; ++u) { c[u] = pc[kc][u]; a[u] = pa[kc][u]; }
+      for (int r = 0; r < RPI; ++r) {
+        cur[r] = rec[kc][r];
+#pragma unroll
+        for (int u = 0; u < EPL; ++u) { c[r][u] = pc[kc][r][u]; a[r][u] = pa[kc][r][u]; }
+      }
       constexpr int NKC_ = NKC;
       const int kp = (kc + AHEAD) % NKC_;
-      load_entries(rec[kp], pc[kp], pa[kp]);
-      rec[kc] = load_rec(q + 1, kc);
+#pragma unroll
+      for (int r = 0; r < RPI; ++r) {
+        load_entries(rec[kp][r], pc[kp][r], pa[kp][r]);
+        rec[kc][r] = load_rec(s1, s2 - s1, kc, r);
+      }
       int b, e;
-      range(q, kc, b, e);
-      if (b + cg < e) row(cur, c, a);
+      share(s0, s1 - s0, kc, b, e);
+#pragma unroll
+      for (int r = 0; r < RPI; ++r)
+        if (b + cg + NG * r < e) row(cur[r], c[r], a[r]);
       lds_barrier();
     }
+    s0 = s1;
+    s1 = s2;
   }
   // rows whose last column came with the last step
   for (int x = sp[S] + cg; x < sp[S + 1]; x += NG) {
