@@ -5,7 +5,7 @@ One "step" is one pass of the hot path, D = A*(B*C), over one synthetic workload
 operands are already resident in HBM.  Default workload: the banded SpMM-SpMM
 configuration (65,536 rows, bandwidth 32, N = 128).  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {1..5}]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {1..6}] [--unfused]
 """
 import argparse
 import importlib
@@ -95,7 +95,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5, 6])
     ap.add_argument("--lds", type=int, default=0, help="LDS budget per tile in bytes (0 = library default)")
     ap.add_argument("--tile-rows", type=int, default=0)
     ap.add_argument("--max-redundancy", type=float, default=0.0)
@@ -103,6 +103,8 @@ def main():
     ap.add_argument("--no-window", action="store_true", help="do not build windowed tiles")
     ap.add_argument("--xcd-chunk", type=int, default=0, help="rows per XCD turn of the row kernels (-1 contiguous)")
     ap.add_argument("--long-row", type=int, default=0, help="rows with more entries than this are chunked")
+    ap.add_argument("--unfused", action="store_true",
+                    help="GeMM-SpMM as two launches (tf_gemm, tf_spmm) with the intermediate in HBM, for comparison")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the result check")
     ap.add_argument("--calibrate", action="store_true",
@@ -140,6 +142,9 @@ def main():
     else:
         Bd = tf.DenseMatrix.from_numpy(cfg["B"])
         step = lambda st: tf.gemm_spmm(Ah, Bd, Cd, D, S, stream=st)  # noqa: E731
+        if args.unfused:  # the two products as separate launches, the intermediate through HBM
+            T = tf.DenseMatrix(A.shape[1], N)
+            step = lambda st: (tf.gemm(Bd, Cd, T, stream=st), tf.spmm(Ah, T, D, stream=st))  # noqa: E731
 
     st = tf.Stream()
     for _ in range(args.warmup):
@@ -182,7 +187,7 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": cfg["name"], "op": cfg["op"], "rows": int(A.shape[0]), "nnz": int(A.nnz), "N": N, "K": K,
-                   "lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
+                   "lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "streamed": bool(info["streamed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
                    "remainder_rows": info["n_remainder_rows"], "recomputed_rows": info["n_producer_rows"] - A.shape[1],
                    "writeback_rows": info["n_writeback_rows"], "kernels_per_step": n_kernels,
                    "inspector_s": round(inspect_s, 4), "rel_err_vs_f64": check, "device": dev["arch"]},
@@ -190,7 +195,8 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes": int(alg_bytes), "kernel_ms": round(dev_ms, 5),
                      "kernel": ("fused_spmm_spmm_window_kernel" if info["windowed"] else "fused_spmm_spmm_kernel")
-                     if op == tf.OP_SPMM_SPMM else "fused_gemm_spmm_kernel",
+                     if op == tf.OP_SPMM_SPMM else ("gemm_rows_kernel + spmm_rows_kernel" if args.unfused else
+                                                    "fused_gemm_spmm_stream_kernel" if info["streamed"] else "fused_gemm_spmm_kernel"),
                      "note": "kernel_ms = HIP-event time on the launch stream / steps (all kernels of a step)"},
     }
     try:  # measured HBM traffic of the dominant kernel, if a committed profile covers this schedule

@@ -87,12 +87,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   int gemm_kc = 0, staging = 0;
   if (gemm_regw) staging = 2 * 64 * 36 * 4;  // the two X staging buffers of the register-W tile kernel
   if (o.op == TF_OP_GEMM_SPMM && !gemm_regw) {
-    if ((long long)o.K * o.N * 4 <= o.lds_budget_bytes / 2) {
-      gemm_kc = o.K;  // W stays resident in LDS next to the slab
-    } else {
-      const int stage_cap = std::min(32768, o.lds_budget_bytes / 2);
-      gemm_kc = std::min(o.K, std::max(8, (stage_cap / (4 * o.N)) / 8 * 8));
-    }
+    const int stage_cap = std::min(32768, o.lds_budget_bytes / 2);
+    gemm_kc = std::min(o.K, std::max(8, (stage_cap / (4 * o.N)) / 8 * 8));
     staging = gemm_kc * o.N * 4;
   }
   // (the register-W tile kernel also keeps 16 bytes per fused row behind the slab)

@@ -593,59 +593,6 @@ __device__ __forceinline__ void stage_weights_interleaved(const float *__restric
   }
 }
 
-// acc += X[32 rows, :K] * W for one 32-row block: Xrow is this lane's A-operand row (+ 4h),
-// wl this lane's first operand in the interleaved W.  A operands are fetched 32 values of k
-// ahead, W operands one 8-wide step ahead of the MFMAs that use them.
-template <int NB>
-__device__ __forceinline__ void mfma_row_block(const float *__restrict__ Xrow, bool row_ok, int steps,
-                                               const wvec<NB> *wl, v16f (&acc)[NB]) {
-  fvec<4> c0 = vzero<4>(), c1 = c0, c2 = c0, c3 = c0;
-  if (row_ok) {
-    c0 = *reinterpret_cast<const fvec<4> *>(Xrow);
-    if (steps > 1) c1 = *reinterpret_cast<const fvec<4> *>(Xrow + 8);
-    if (steps > 2) c2 = *reinterpret_cast<const fvec<4> *>(Xrow + 16);
-    if (steps > 3) c3 = *reinterpret_cast<const fvec<4> *>(Xrow + 24);
-  }
-  wvec<NB> bw[4], bn[4];
-#pragma unroll
-  for (int t = 0; t < 4; ++t) bw[t] = wl[t * 32];
-  for (int s0 = 0; s0 < steps; s0 += 4) {
-    fvec<4> n0 = vzero<4>(), n1 = n0, n2 = n0, n3 = n0;
-    if (s0 + 4 < steps && row_ok) {
-      const float *nx = Xrow + (s0 + 4) * 8;
-      n0 = *reinterpret_cast<const fvec<4> *>(nx);
-      if (s0 + 5 < steps) n1 = *reinterpret_cast<const fvec<4> *>(nx + 8);
-      if (s0 + 6 < steps) n2 = *reinterpret_cast<const fvec<4> *>(nx + 16);
-      if (s0 + 7 < steps) n3 = *reinterpret_cast<const fvec<4> *>(nx + 24);
-    }
-    {
-      const int sn = min(s0 + 1, steps - 1);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) bn[t] = wl[(8 * sn + t) * 32];
-      mfma_step8<NB>(c0, bw, acc);
-    }
-    if (s0 + 1 < steps) {
-      const int sn = min(s0 + 2, steps - 1);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) bw[t] = wl[(8 * sn + t) * 32];
-      mfma_step8<NB>(c1, bn, acc);
-    }
-    if (s0 + 2 < steps) {
-      const int sn = min(s0 + 3, steps - 1);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) bn[t] = wl[(8 * sn + t) * 32];
-      mfma_step8<NB>(c2, bw, acc);
-    }
-    if (s0 + 3 < steps) {
-      const int sn = min(s0 + 4, steps - 1);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) bw[t] = wl[(8 * sn + t) * 32];
-      mfma_step8<NB>(c3, bn, acc);
-    }
-    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
-  }
-}
-
 template <int NB>
 __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__restrict__ X,
                                                                const float *__restrict__ W,
@@ -754,73 +701,6 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
     }
     Xrow = Xnext;
     row_ok = next_ok;
-  }
-}
-
-// Fused GeMM-SpMM tile kernel with W resident in LDS (K*N*4 <= half the LDS budget):
-// persistent workgroups walk the fused tiles; per tile the wavefronts compute the
-// intermediate rows 32 at a time on MFMA into the LDS slab (and to HBM for the rows the
-// remainder reads), then the lane groups compute the tile's fused rows out of the slab.
-template <int NB, int LPR>
-__global__ __launch_bounds__(kGemmBlock) void fused_gemm_spmm_resident_kernel(
-    const TileDesc *__restrict__ tiles, int n_tiles, int per_xcd, int n_virtual,
-    const int *__restrict__ fused_ids, const float *__restrict__ B, const float *__restrict__ W, int K,
-    const int *__restrict__ Ap, const int *__restrict__ Ai, const float *__restrict__ Ax,
-    float *__restrict__ D, float *__restrict__ T, int accumulate) {
-  extern __shared__ __align__(16) float lds[];
-  constexpr int N = NB * 32;
-  constexpr int V = 4;
-  constexpr int G = kGemmBlock / LPR;
-  constexpr int NW = kGemmBlock / 64;
-  float *wlds = lds;
-  float *slab = lds + K * N;
-  stage_weights_interleaved<NB>(W, K, wlds);
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  const int h = lane / 32, j = lane % 32;
-  const int steps = K / 8;
-  const wvec<NB> *wl = reinterpret_cast<const wvec<NB> *>(wlds) + (4 * h) * 32 + j;
-  const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
-  const int coff = glane * V;
-  const bool ok = coff < N;
-  for (int v = blockIdx.x; v < n_virtual; v += gridDim.x) {  // gridDim.x is a multiple of 8
-    const int tile = xcd_contiguous(v, per_xcd);
-    if (tile >= n_tiles) continue;  // uniform for the workgroup
-    __syncthreads();                // W staged; slab free again
-    const TileDesc t = tiles[tile];
-    const int P = t.prod_end - t.prod_begin;
-    const bool has_cons = t.cons_end > t.cons_begin;
-    for (int rb = wave; rb * 32 < P; rb += NW) {
-      const int row = t.prod_begin + rb * 32 + j;
-      const bool row_ok = row < t.prod_end;
-      v16f acc[NB];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
-      mfma_row_block<NB>(B + (size_t)(row_ok ? row : t.prod_begin) * K + 4 * h, row_ok, steps, wl, acc);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int orow = t.prod_begin + rb * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-        if (orow < t.prod_end) {
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) {
-            const float val = acc[nb][r];
-            if (has_cons) slab[(orow - t.prod_begin) * N + nb * 32 + j] = val;
-            if (orow >= t.wb_begin && orow < t.wb_end) T[(size_t)orow * N + nb * 32 + j] = val;
-          }
-        }
-      }
-    }
-    if (!has_cons) continue;
-    __syncthreads();
-    const LdsRows<V> tsrc{slab, N, ok ? coff : 0, t.prod_begin};
-    for (int q = t.cons_begin + group; q < t.cons_end; q += G) {
-      const int i = fused_ids[q];
-      fvec<V> acc = vzero<V>();
-      if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)i * N + coff);
-      row_dot<V, LPR>(Ai, Ax, Ap[i], Ap[i + 1], glane, ok, tsrc, acc);
-      if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)i * N + coff) = acc;
-    }
   }
 }
 
@@ -1431,26 +1311,6 @@ hipError_t launch_fused_gemm_spmm(const TileDesc *tiles, int n_tiles, const int 
     if (KS == 4) CALL2(4); else if (KS == 8) CALL2(8); else CALL2(16);
 #undef CALL2
 #undef CALL3
-    return err != hipSuccess ? err : hipGetLastError();
-  }
-  if (kc == K) {
-    // W stays in LDS: persistent workgroups, one per compute unit (a multiple of 8 of them)
-    const int n_virtual = grid_of(n_tiles);
-    const int grid = std::min(n_virtual, std::max(kXcds, compute_units / kXcds * kXcds));
-#define CALL2(NB_, L_)                                                                          \
-  err = allow_lds(fused_gemm_spmm_resident_kernel<NB_, L_>, lds_bytes);                         \
-  if (err == hipSuccess)                                                                        \
-    hipLaunchKernelGGL((fused_gemm_spmm_resident_kernel<NB_, L_>), dim3(grid), dim3(kGemmBlock), \
-                       lds_bytes, st, tiles, n_tiles, per, n_virtual, fused_ids, B, C, K, Ap, Ai, \
-                       Ax, D, T, accumulate)
-#define CALL(NB_)                                                         \
-  do {                                                                    \
-    if (LPR == 8) { CALL2(NB_, 8); } else if (LPR == 16) { CALL2(NB_, 16); } \
-    else if (LPR == 32) { CALL2(NB_, 32); } else { CALL2(NB_, 64); }      \
-  } while (0)
-    TF_DISPATCH_NB(NB, CALL);
-#undef CALL
-#undef CALL2
     return err != hipSuccess ? err : hipGetLastError();
   }
 #define CALL2(NB_, L_)                                                                      \

@@ -110,6 +110,9 @@ CONFIG_NAMES = {
     3: "cfg3 GeMM-SpMM GCN layer, Erdos-Renyi 200k nodes deg 10, K=256 N=128",
     4: "cfg4 GeMM-SpMM R-MAT 2^21 nodes, K=N=128",
     5: "cfg5 SpMM-SpMM 3D Laplacian 128^3, N=64",
+    # not one of the reference's configurations: the banded pattern of cfg2 under GeMM-SpMM, the
+    # workload on which the fused GeMM-SpMM kernel has rows to fuse at full size
+    6: "extra GeMM-SpMM banded bw32 262144 rows, K=N=128",
 }
 
 
@@ -139,6 +142,10 @@ def make_config(idx, scale=1.0):
         A = laplacian_3d(g)
         M = A.shape[0]
         return dict(op="spmm_spmm", A=A, B=A, C=uniform((M, 64), 11), K=0, N=64, name=CONFIG_NAMES[5])
+    if idx == 6:
+        M = max(256, int(262144 * scale))
+        A = banded_random(M, 32, 16, seed=3)
+        return dict(op="gemm_spmm", A=A, B=uniform((M, 128), 12), C=uniform((128, 128), 13), K=128, N=128, name=CONFIG_NAMES[6])
     raise ValueError(f"unknown config {idx}")
 
 
