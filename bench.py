@@ -103,6 +103,11 @@ def main():
     ap.add_argument("--no-window", action="store_true", help="do not build windowed tiles")
     ap.add_argument("--xcd-chunk", type=int, default=0, help="rows per XCD turn of the row kernels (-1 contiguous)")
     ap.add_argument("--long-row", type=int, default=0, help="rows with more entries than this are chunked")
+    ap.add_argument("--matrix", default=None, help="run on a .mtx / .smtx file instead of a synthetic configuration "
+                    "(square; symmetric files are expanded), with --op, --N and --K")
+    ap.add_argument("--op", default="spmm_spmm", choices=["spmm_spmm", "gemm_spmm"])
+    ap.add_argument("--N", type=int, default=64)
+    ap.add_argument("--K", type=int, default=64)
     ap.add_argument("--unfused", action="store_true",
                     help="GeMM-SpMM as two launches (tf_gemm, tf_spmm) with the intermediate in HBM, for comparison")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -121,7 +126,16 @@ def main():
     if args.calibrate:
         calibrate(tf)
         return
-    cfg = w.make_config(args.config)
+    if args.matrix:
+        Af = tf.read_matrix(args.matrix)
+        if Af.shape[0] != Af.shape[1]:
+            sys.exit("bench.py --matrix: the matrix must be square")
+        Mf = Af.shape[0]
+        gemm = args.op == "gemm_spmm"
+        cfg = dict(op=args.op, A=Af, B=w.uniform((Mf, args.K), 21) if gemm else Af, C=w.uniform((args.K if gemm else Mf, args.N), 22),
+                   K=args.K if gemm else 0, N=args.N, name=f"file {os.path.basename(args.matrix)} {args.op} N={args.N}" + (f" K={args.K}" if gemm else ""))
+    else:
+        cfg = w.make_config(args.config)
     A, N, K = cfg["A"], cfg["N"], cfg["K"]
     op = tf.OP_GEMM_SPMM if cfg["op"] == "gemm_spmm" else tf.OP_SPMM_SPMM
 

@@ -94,6 +94,23 @@ tf_status tf_dense_fill(tf_dense *d, float value, void *stream);
 float *tf_dense_device_ptr(const tf_dense *d);
 void tf_dense_free(tf_dense *d);
 
+/* ---- matrices from files -------------------------------------------------------- */
+
+/* Reads a sparse matrix into host CSR arrays (sorted columns, duplicates summed) that the
+ * caller releases with tf_host_free.  By file extension, as get_matrix_from_parameter does
+ * (fusion/src/Fusion_Utils.cpp:254-272):
+ *   .mtx   MatrixMarket coordinate or array, real / integer / pattern (pattern entries are 1);
+ *          symmetric and skew-symmetric files are expanded to the full matrix, which the
+ *          reference's drivers do with make_full before use (SpMM_SpMM_SP_Demo.cpp:24-32);
+ *   .smtx  DLMC: "rows, cols, nnz", the row pointers, the column indices; every value is 1
+ *          (readSparseMatrix, Fusion_Utils.cpp:205-250).
+ * Host-only; no GPU is needed. */
+tf_status tf_read_matrix(const char *path, int *M, int *N, int *nnz, int **Ap, int **Ai, float **Ax);
+/* The same file kinds as a dense row-major matrix (the feature matrices of the GCN drivers,
+ * read_mtx_array_real at Fusion_Utils.cpp:283). */
+tf_status tf_read_dense(const char *path, int *M, int *N, float **data);
+void tf_host_free(void *p);
+
 /* ---- inspector ---------------------------------------------------------------- */
 
 enum { TF_OP_SPMM_SPMM = 0, TF_OP_GEMM_SPMM = 1 };

@@ -86,6 +86,9 @@ SIGNATURES = {
     "tf_dense_fill": (C.c_int, [_VP, C.c_float, _VP]),
     "tf_dense_device_ptr": (_VP, [_VP]),
     "tf_dense_free": (None, [_VP]),
+    "tf_read_matrix": (C.c_int, [C.c_char_p, _PI, _PI, _PI, C.POINTER(_PI), C.POINTER(_PI), C.POINTER(_PF)]),
+    "tf_read_dense": (C.c_int, [C.c_char_p, _PI, _PI, C.POINTER(_PF)]),
+    "tf_host_free": (None, [_VP]),
     "tf_inspect": (C.c_int, [C.c_int, C.c_int, _PI, _PI, C.POINTER(InspectOpts), C.POINTER(_VP)]),
     "tf_schedule_free": (None, [_VP]),
     "tf_schedule_get_info": (C.c_int, [_VP, C.POINTER(ScheduleInfo)]),
@@ -329,3 +332,32 @@ def spmm(A, X, Y, *, accumulate=False, stream=None):
 
 def gemm(X, W, Y, *, stream=None):
     _check(lib().tf_gemm(X.h, W.h, Y.h, stream.h if stream else None))
+
+
+def read_matrix(path):
+    """A .mtx / .smtx file as a scipy CSR matrix (int32 indices, fp32 values), read by the
+    library's own reader -- the formats the reference's drivers take (Fusion_Utils.cpp:254-272)."""
+    import scipy.sparse as sp
+    M, N, nnz = C.c_int(), C.c_int(), C.c_int()
+    Ap, Ai, Ax = _PI(), _PI(), _PF()
+    _check(lib().tf_read_matrix(str(path).encode(), C.byref(M), C.byref(N), C.byref(nnz), C.byref(Ap), C.byref(Ai), C.byref(Ax)))
+    try:
+        p = np.ctypeslib.as_array(Ap, shape=(M.value + 1,)).copy()
+        i = np.ctypeslib.as_array(Ai, shape=(max(nnz.value, 1),))[:nnz.value].copy()
+        x = np.ctypeslib.as_array(Ax, shape=(max(nnz.value, 1),))[:nnz.value].copy()
+    finally:
+        for q in (Ap, Ai, Ax):
+            lib().tf_host_free(C.cast(q, _VP))
+    return sp.csr_matrix((x, i, p), shape=(M.value, N.value))
+
+
+def read_dense(path):
+    """A MatrixMarket file as a dense row-major fp32 array (Fusion_Utils.cpp:283)."""
+    M, N = C.c_int(), C.c_int()
+    d = _PF()
+    _check(lib().tf_read_dense(str(path).encode(), C.byref(M), C.byref(N), C.byref(d)))
+    try:
+        out = np.ctypeslib.as_array(d, shape=(max(M.value * N.value, 1),))[:M.value * N.value].copy()
+    finally:
+        lib().tf_host_free(C.cast(d, _VP))
+    return out.reshape(M.value, N.value)
