@@ -146,9 +146,10 @@ typedef struct {
   int inner_cols;
   int strip_cols;        /* windowed tiles work on this many columns of C/D at a time (32 or 64);
                             default 32                                                         */
-  int xcd_chunk_rows;    /* the row kernels deal rows to the 8 XCDs in chunks of this many rows;
-                            0 = choose (an eighth of a dominant far stencil distance, else one
-                            contiguous run per XCD), -1 = always contiguous                   */
+  int xcd_chunk_rows;    /* how the row kernels' workgroups are dealt to the 8 XCDs: 0 = round-robin
+                            (default), n > 0 = chunks of n rows per XCD turn (a 3D stencil with
+                            plane distance d keeps its halo in one L2 with n = d/8), -1 = one
+                            contiguous run of rows per XCD                                     */
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -180,7 +181,7 @@ typedef struct {
   int lds_bytes;         /* dynamic LDS of the fused-tile kernel                    */
   int windowed;          /* 1 when tiles stage their window of C in LDS             */
   int strip_cols;        /* columns per strip of the windowed kernel, else 0        */
-  int xcd_chunk_rows;    /* rows per XCD turn chosen for the row kernels (0: contiguous) */
+  int xcd_chunk_rows;    /* rows per XCD turn of the row kernels (0: round-robin, -1: contiguous) */
   int streamed;          /* 1 when GeMM-SpMM tiles are long runs streamed through an LDS ring */
   int ring_rows;         /* intermediate rows the ring holds, else 0                 */
   long long fused_nnz;   /* stored entries of A in fused rows (getFusedNnzNum)      */

@@ -140,17 +140,17 @@ def test_spmm_spmm_long_rows(gpu, tf, orc):
 
 
 def test_spmm_spmm_xcd_chunked_rows(gpu, tf, orc):
-    """3D stencil whose plane distance makes the inspector deal rows to the XCDs in chunks:
-    same bits as the contiguous mapping and as the oracle."""
-    say("spmm_spmm 3D Laplacian, chunked XCD mapping")
-    g, N = 52, 64  # planes 2704 rows apart -> chunks of 320 rows
+    """The row kernels under every workgroup-to-XCD mapping (round-robin, chunks of rows,
+    one run per XCD): same bits as the oracle."""
+    say("spmm_spmm 3D Laplacian, XCD mappings")
+    g, N = 52, 64
     A = tf.workloads.laplacian_3d(g)
     Cd = tf.workloads.uniform((g ** 3, N), 46)
     want = oracle_spmm_spmm(orc, A, A, Cd)
     got, info = run_spmm_spmm(tf, A, A, Cd)
-    assert info["xcd_chunk_rows"] == 320 and info["n_fused_rows"] == 0
+    assert info["xcd_chunk_rows"] == 0 and info["n_fused_rows"] == 0
     assert np.array_equal(got, want)
-    for chunk in (-1, 64, 4096):
+    for chunk in (-1, 64, 320, 4096):
         got, info = run_spmm_spmm(tf, A, A, Cd, xcd_chunk_rows=chunk)
         assert np.array_equal(got, want), chunk
 
@@ -374,6 +374,39 @@ def test_unfused_building_blocks(gpu, tf, orc):
     Z = tf.DenseMatrix(2000, 64)
     tf.gemm(tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W), Z)
     assert orc.rel_err(Z.to_numpy(), X.astype(np.float64) @ W.astype(np.float64)) <= 1e-6
+
+
+@pytest.mark.parametrize("N", [32, 64, 128, 256, 20, 320])
+def test_spmm_long_row_lists_bit_exact(gpu, tf, orc, N):
+    """Row lists of 4096 rows and more take the kernel that stages row pointers and entries ahead:
+    rows with 0, a few, exactly 16, and more than 16 entries, unsorted columns, accumulate."""
+    say(f"tf_spmm staged N={N}")
+    M = 9000
+    rng = np.random.default_rng(80 + N)
+    lens = rng.choice([0, 1, 3, 7, 8, 9, 15, 16, 17, 24, 31, 32], size=M)
+    lens[-1] = 5
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    indices = np.concatenate([rng.choice(M, l, replace=False) for l in lens]).astype(np.int32)
+    data = rng.uniform(-1, 1, indptr[-1]).astype(np.float32)
+    A = sp.csr_matrix((data, indices, indptr), shape=(M, M))
+    X = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    Y = tf.DenseMatrix(M, N)
+    Y.fill(float("nan"))
+    tf.spmm(Ah, tf.DenseMatrix.from_numpy(X), Y)
+    want = orc.spmm(A, X)
+    assert np.array_equal(Y.to_numpy(), want)
+    Y0 = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    Y = tf.DenseMatrix(M, N, Y0)
+    tf.spmm(Ah, tf.DenseMatrix.from_numpy(X), Y, accumulate=True)
+    got = Y.to_numpy()
+    ref = Y0.copy()
+    for i in range(0, M, 97):  # accumulate continues the fma chain from the old value
+        acc = Y0[i].copy()
+        for k in range(indptr[i], indptr[i + 1]):
+            acc = (np.float64(data[k]) * X[indices[k]].astype(np.float64) + acc).astype(np.float32)
+        ref[i] = acc
+    assert np.array_equal(got[::97], ref[::97])
 
 
 def test_cpp_readme_api(gpu):

@@ -212,13 +212,12 @@ def test_windowed_tiles(tf):
     assert tf.inspector(Rh, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Rh).info()["windowed"] == 0
 
 
-def test_far_stencil_distance_sets_xcd_chunk(tf):
-    A = tf.workloads.laplacian_3d(40)  # planes 1600 rows apart: below the 2048-row floor
-    assert tf.inspector(tf.CsrMatrix.from_scipy(A), 1, op=tf.OP_SPMM_SPMM, N=64).info()["xcd_chunk_rows"] == 0
-    A = tf.workloads.laplacian_3d(64)  # planes 4096 rows apart -> chunks of 512 rows
-    assert tf.inspector(tf.CsrMatrix.from_scipy(A), 1, op=tf.OP_SPMM_SPMM, N=64).info()["xcd_chunk_rows"] == 512
-    A = tf.workloads.erdos_renyi_gcn(20000, 10.0, seed=5)  # random graph: no dominant distance
-    assert tf.inspector(tf.CsrMatrix.from_scipy(A), 1, op=tf.OP_SPMM_SPMM, N=64).info()["xcd_chunk_rows"] == 0
+def test_xcd_chunk_is_the_callers_choice(tf):
+    A = tf.workloads.laplacian_3d(40)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64).info()["xcd_chunk_rows"] == 0
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, xcd_chunk_rows=512).info()["xcd_chunk_rows"] == 512
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, xcd_chunk_rows=-1).info()["xcd_chunk_rows"] == -1
 
 
 def test_streamed_runs(tf):

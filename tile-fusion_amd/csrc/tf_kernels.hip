@@ -92,7 +92,7 @@ __device__ __forceinline__ void row_dot_batch(int c, float a, int t, int cnt, bo
   if (col_ok) {
     fvec<V> x[B];
 #pragma unroll
-    for (int u = 0; u < B; ++u) x[u] = src.load(cc[u]);
+    for (int u = 0; u < B; ++u) x[u] = (t + u < cnt) ? src.load(cc[u]) : vzero<V>();
 #pragma unroll
     for (int u = 0; u < B; ++u) {
       fvec<V> next = acc;
@@ -123,6 +123,35 @@ __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float
     float a = 0.f;
     if (k < ke) { c = idx[k]; a = val[k]; }
     row_dot_loaded<V, LPR>(c, a, min(LPR, ke - k0), col_ok, src, acc);
+  }
+}
+
+// The same sum with every lane reading the row's (column, value) pairs itself: the lanes of a
+// group read the same address, which costs one request per group and no cross-lane traffic.
+// Eight pairs, then their eight gathers, then the fmas; slots past the row's end load nothing.
+template <int V, int LPR, class Src>
+__device__ __forceinline__ void row_dot_direct(const int *__restrict__ idx, const float *__restrict__ val,
+                                               int kb, int ke, bool col_ok, const Src &src, fvec<V> &acc) {
+  for (int k0 = kb; k0 < ke; k0 += 8) {
+    int cc[8];
+    float aa[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      cc[u] = 0;
+      aa[u] = 0.f;
+      if (k0 + u < ke) { cc[u] = idx[k0 + u]; aa[u] = val[k0 + u]; }
+    }
+    if (col_ok) {
+      fvec<V> x[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) x[u] = (k0 + u < ke) ? src.load(cc[u]) : vzero<V>();
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        fvec<V> next = acc;
+        vfma<V>(aa[u], x[u], next);
+        if (k0 + u < ke) acc = next;
+      }
+    }
   }
 }
 
@@ -351,7 +380,7 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
     const GlobalRows<V> src{X, ldx, ok ? coff : 0};
     fvec<V> acc = vzero<V>();
     if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
-    row_dot<V, LPR>(Ai, Ax, kb, ke, glane, ok, src, acc);
+    row_dot_direct<V, LPR>(Ai, Ax, kb, ke, ok, src, acc);
     if (ok) *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
   }
 }
@@ -1254,7 +1283,8 @@ hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const in
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
   const int n_blocks = (n_rows + G - 1) / G;
-  const int bpc = chunk_bpc(n_blocks, xcd_chunk_rows > 0 ? std::max(1, xcd_chunk_rows / G) : 0);
+  // 0: workgroup b takes block b; > 0: chunks of rows per XCD turn; < 0: one contiguous run per XCD
+  const int bpc = xcd_chunk_rows == 0 ? 0 : chunk_bpc(n_blocks, xcd_chunk_rows > 0 ? std::max(1, xcd_chunk_rows / G) : 0);
 #define CALL(V_, L_)                                                                                   \
   hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(grid_chunked(n_blocks, bpc)), dim3(kBlock), 0, st, \
                      rows, n_rows, n_blocks, bpc, Ap, Ai, Ax, X, N, Y, N, accumulate)
