@@ -73,21 +73,22 @@ def cpu_baseline(cfg, budget_s=20.0):
 
 
 def calibrate(tf, rows=1 << 20, N=128, reps=5):
-    """A plain copy of known size: Y = I * X through tf_spmm reads X (rows*N*4 bytes) plus the
-    CSR of the identity (12 bytes a row + 4) and writes Y (rows*N*4 bytes), with no reuse.
-    Run under `rocprofv3 --pmc FETCH_SIZE` (then WRITE_SIZE): the ratio of the counter to
-    these byte counts is the factor the counter has to be scaled by."""
-    import scipy.sparse as sp
-    eye = sp.identity(rows, dtype=np.float32, format="csr")
-    A = tf.CsrMatrix.from_scipy(eye).to_device()
+    """A plain copy of known size: Y = X, device to device (tf_dense_copy; the runtime's copy
+    kernel), reads rows*N*4 bytes and writes as many, with no reuse.  Run under
+    `rocprofv3 --pmc FETCH_SIZE` (then WRITE_SIZE): the ratio of the counter to these byte
+    counts is the factor the counter has to be scaled by."""
     X = tf.DenseMatrix(rows, N)
     X.fill(1.0)
     Y = tf.DenseMatrix(rows, N)
-    for _ in range(reps):
-        tf.spmm(A, X, Y)
     tf.device_synchronize()
-    print(json.dumps({"calibration_kernel": "spmm_rows_kernel", "launches": reps,
-                      "read_bytes_per_launch": rows * N * 4 + 12 * rows + 4, "write_bytes_per_launch": rows * N * 4}))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        Y.copy_from(X)
+    tf.device_synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    print(json.dumps({"calibration_kernel": "device-to-device copy (tf_dense_copy)", "launches": reps,
+                      "read_bytes_per_launch": rows * N * 4, "write_bytes_per_launch": rows * N * 4,
+                      "copy_GBps_read_plus_write": round(2 * rows * N * 4 / dt / 1e9, 1)}))
 
 
 def main():
@@ -208,8 +209,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes": int(alg_bytes), "kernel_ms": round(dev_ms, 5),
-                     "kernel": ("fused_spmm_spmm_window_kernel" if info["windowed"] else "fused_spmm_spmm_kernel")
-                     if op == tf.OP_SPMM_SPMM else ("gemm_rows_kernel + spmm_rows_kernel" if args.unfused else
+                     "kernel": ("fused_spmm_spmm_window_kernel" if info["windowed"] else
+                                "fused_spmm_spmm_kernel" if info["n_fused_rows"] else "spmm_rows_kernel (twice)")
+                     if op == tf.OP_SPMM_SPMM else ("gemm_rows_kernel + spmm_rows_kernel" if args.unfused or info["n_fused_rows"] == 0 else
                                                     "fused_gemm_spmm_stream_kernel" if info["streamed"] else "fused_gemm_spmm_kernel"),
                      "note": "kernel_ms = HIP-event time on the launch stream / steps (all kernels of a step)"},
     }

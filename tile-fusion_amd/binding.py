@@ -84,6 +84,7 @@ SIGNATURES = {
     "tf_dense_wrap_device": (C.c_int, [C.c_int, C.c_int, _VP, C.POINTER(_VP)]),
     "tf_dense_download": (C.c_int, [_VP, _PF]),
     "tf_dense_fill": (C.c_int, [_VP, C.c_float, _VP]),
+    "tf_dense_copy": (C.c_int, [_VP, _VP, _VP]),
     "tf_dense_device_ptr": (_VP, [_VP]),
     "tf_dense_free": (None, [_VP]),
     "tf_read_matrix": (C.c_int, [C.c_char_p, _PI, _PI, _PI, C.POINTER(_PI), C.POINTER(_PI), C.POINTER(_PF)]),
@@ -239,6 +240,9 @@ class DenseMatrix:
         self.h = _VP()
         _check(lib().tf_dense_wrap_device(self.M, self.N, _VP(device_ptr), C.byref(self.h)))
         return self
+
+    def copy_from(self, src, stream=None):
+        _check(lib().tf_dense_copy(self.h, src.h, stream.h if stream else None))
 
     def fill(self, value, stream=None):
         _check(lib().tf_dense_fill(self.h, float(value), stream.h if stream else None))

@@ -341,6 +341,15 @@ extern "C" tf_status tf_dense_fill(tf_dense *d, float value, void *stream) {
   return TF_OK;
 }
 
+extern "C" tf_status tf_dense_copy(tf_dense *dst, const tf_dense *src, void *stream) {
+  if (!dst || !src) return fail(TF_EINVAL, "tf_dense_copy: null argument");
+  if (dst->M != src->M || dst->N != src->N)
+    return fail(TF_EINVAL, "tf_dense_copy: shapes differ (%d x %d and %d x %d)", dst->M, dst->N, src->M, src->N);
+  TF_HIP(hipMemcpyAsync(dst->d, src->d, (size_t)src->M * src->N * sizeof(float), hipMemcpyDeviceToDevice,
+                        static_cast<hipStream_t>(stream)));
+  return TF_OK;
+}
+
 extern "C" float *tf_dense_device_ptr(const tf_dense *d) { return d ? d->d : nullptr; }
 
 extern "C" void tf_dense_free(tf_dense *d) {
