@@ -111,6 +111,9 @@ def main():
     ap.add_argument("--K", type=int, default=64)
     ap.add_argument("--unfused", action="store_true",
                     help="GeMM-SpMM as two launches (tf_gemm, tf_spmm) with the intermediate in HBM, for comparison")
+    ap.add_argument("--host-buffers", action="store_true",
+                    help="also time the step as the README API runs it on un-pinned operands: upload A, B/C and D, "
+                         "execute, download D (reported as host_buffer_ms_per_step; never part of value)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the result check")
     ap.add_argument("--calibrate", action="store_true",
@@ -226,6 +229,19 @@ def main():
     if op == tf.OP_GEMM_SPMM:
         gemm_flops = 2.0 * A.shape[1] * K * N
         out["roofline"]["mfma_frac_if_gemm_only"] = round(gemm_flops / (dev_ms * 1e-3) / 1e12 / MFMA_FP32_PEAK_TF, 4)
+    if args.host_buffers:  # PCIe-inclusive: every operand crosses the bus each step
+        reps = 5
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            Ah2 = tf.CsrMatrix.from_scipy(A).to_device()
+            Cd2 = tf.DenseMatrix.from_numpy(cfg["C"])
+            D2 = tf.DenseMatrix(A.shape[0], N, np.zeros((A.shape[0], N), np.float32))
+            if op == tf.OP_SPMM_SPMM:
+                tf.spmm_spmm(Ah2, Ah2 if cfg["B"] is A else tf.CsrMatrix.from_scipy(cfg["B"]).to_device(), Cd2, D2, S, accumulate=True)
+            else:
+                tf.gemm_spmm(Ah2, tf.DenseMatrix.from_numpy(cfg["B"]), Cd2, D2, S, accumulate=True)
+            D2.to_numpy()
+        out["host_buffer_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / reps, 3)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(out))
