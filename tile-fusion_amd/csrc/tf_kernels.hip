@@ -622,7 +622,9 @@ __device__ __forceinline__ void stage_weights_interleaved(const float *__restric
   }
 }
 
-template <int NB>
+constexpr int kGemmSeg = 16;  // row blocks whose row numbers a wavefront keeps in LDS at a time
+
+template <int NB, bool LIST>
 __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__restrict__ X,
                                                                const float *__restrict__ W,
                                                                float *__restrict__ Y,
@@ -637,99 +639,95 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
   const int total_waves = gridDim.x * (kGemmBlock / 64);
   const int nrb = (n_rows + 31) / 32;
   const int steps = K / 8;  // 8-wide k steps; this lane's rows of W in step s are 8s + 4h + t
+  const int G4 = (steps + 3) / 4;  // groups of four steps (32 values of k): the unit the A operand is fetched in
   const wvec<NB> *wl = reinterpret_cast<const wvec<NB> *>(wlds) + (4 * h) * 32 + j;
+  // this wavefront's slice of LDS behind W: the row numbers of the blocks it is working on (row
+  // lists only).  Reading them from LDS keeps the row list out of the chain of global loads, so
+  // the A operands requested ahead are never waited for early.
+  int *ridx = reinterpret_cast<int *>(wlds + K * N) + wave * (kGemmSeg * 32);
   // every wavefront walks one contiguous run of row blocks; run lengths differ by at most one
   // and the longer runs are spread evenly over the compute units
   const int gw = blockIdx.x * (kGemmBlock / 64) + wave;
-  const int rb0 = (int)((long long)gw * nrb / total_waves);
-  const int rb_end = (int)((long long)(gw + 1) * nrb / total_waves);
-  // A operand: four 8-wide steps (32 values of k) in registers, the next four in flight --
-  // across row blocks too: the first four steps of the next block are requested before the
-  // current block's results are stored.
-  fvec<4> c0 = vzero<4>(), c1 = c0, c2 = c0, c3 = c0;
-  const float *Xrow = X;
-  bool row_ok = false;
-  if (rb0 < rb_end) {
-    const int q = rb0 * 32 + j;  // list position whose row this lane feeds as the A operand
-    row_ok = q < n_rows;
-    Xrow = X + (size_t)(row_ok ? (rows ? rows[q] : q) : 0) * K + 4 * h;
-    if (row_ok) {
-      c0 = *reinterpret_cast<const fvec<4> *>(Xrow);
-      if (steps > 1) c1 = *reinterpret_cast<const fvec<4> *>(Xrow + 8);
-      if (steps > 2) c2 = *reinterpret_cast<const fvec<4> *>(Xrow + 16);
-      if (steps > 3) c3 = *reinterpret_cast<const fvec<4> *>(Xrow + 24);
+  const int run0 = (int)((long long)gw * nrb / total_waves);
+  const int run_end = (int)((long long)(gw + 1) * nrb / total_waves);
+  for (int rb0 = run0; rb0 < run_end; rb0 += kGemmSeg) {
+    const int rb_end = min(run_end, rb0 + kGemmSeg);
+    if constexpr (LIST) {
+      for (int x = lane; x < (rb_end - rb0) * 32; x += 64) ridx[x] = rows[min(rb0 * 32 + x, n_rows - 1)];
     }
-  }
-  for (int rb = rb0; rb < rb_end; ++rb) {
+    const int total_groups = (rb_end - rb0) * G4;
+    // row (of X and Y) behind position x of this segment
+    auto row_at = [&](int x) { return LIST ? ridx[x] : min(rb0 * 32 + x, n_rows - 1); };
+    // A operand of group gi (block rb0 + gi / G4, steps 4 (gi % G4) ..): four 16-byte loads per lane,
+    // always issued (block and k clamped to existing ones, the surplus is never used) so that the
+    // loads of later groups stay in flight while earlier ones are consumed.
+    auto load_group = [&](int gi, fvec<4> (&c)[4]) {
+      const int g = min(gi, total_groups - 1);
+      const int s0 = (g % G4) * 4;
+      const float *p = X + (size_t)row_at((g / G4) * 32 + j) * K + s0 * 8 + 4 * h;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) c[u] = *reinterpret_cast<const fvec<4> *>(p + 8 * min(u, steps - 1 - s0));
+    };
+    // three register sets, used in turn: a group's operands are requested two groups ahead
+    fvec<4> set0[4], set1[4], set2[4];
+    load_group(0, set0);
+    load_group(1, set1);
     v16f acc[NB];
+    auto run_group = [&](int gi, const fvec<4> (&c)[4]) {
+      const int g = gi % G4, blk = gi / G4, s0 = 4 * g;
+      if (g == 0) {
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
+        for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
-    // the row this lane will feed in the wave's next block
-    const int rbn = rb + 1;
-    const int qn = rbn * 32 + j;
-    const bool next_ok = rbn < rb_end && qn < n_rows;
-    const float *Xnext = X + (size_t)(next_ok ? (rows ? rows[qn] : qn) : 0) * K + 4 * h;
-    wvec<NB> bw[4], bn[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) bw[t] = wl[t * 32];
-    for (int s0 = 0; s0 < steps; s0 += 4) {
-      fvec<4> n0 = vzero<4>(), n1 = n0, n2 = n0, n3 = n0;
-      if (s0 + 4 < steps) {
-        if (row_ok) {
-          const float *nx = Xrow + (s0 + 4) * 8;
-          n0 = *reinterpret_cast<const fvec<4> *>(nx);
-          if (s0 + 5 < steps) n1 = *reinterpret_cast<const fvec<4> *>(nx + 8);
-          if (s0 + 6 < steps) n2 = *reinterpret_cast<const fvec<4> *>(nx + 16);
-          if (s0 + 7 < steps) n3 = *reinterpret_cast<const fvec<4> *>(nx + 24);
-        }
-      } else if (next_ok) {  // last group of this block: fetch the next block's first group
-        n0 = *reinterpret_cast<const fvec<4> *>(Xnext);
-        if (steps > 1) n1 = *reinterpret_cast<const fvec<4> *>(Xnext + 8);
-        if (steps > 2) n2 = *reinterpret_cast<const fvec<4> *>(Xnext + 16);
-        if (steps > 3) n3 = *reinterpret_cast<const fvec<4> *>(Xnext + 24);
+          for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
       }
-      // step s0
+      wvec<NB> bw[4], bn[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) bw[t] = wl[(8 * s0 + t) * 32];
       {
         const int sn = min(s0 + 1, steps - 1);
 #pragma unroll
         for (int t = 0; t < 4; ++t) bn[t] = wl[(8 * sn + t) * 32];
-        mfma_step8<NB>(c0, bw, acc);
+        mfma_step8<NB>(c[0], bw, acc);
       }
       if (s0 + 1 < steps) {
         const int sn = min(s0 + 2, steps - 1);
 #pragma unroll
         for (int t = 0; t < 4; ++t) bw[t] = wl[(8 * sn + t) * 32];
-        mfma_step8<NB>(c1, bn, acc);
+        mfma_step8<NB>(c[1], bn, acc);
       }
       if (s0 + 2 < steps) {
         const int sn = min(s0 + 3, steps - 1);
 #pragma unroll
         for (int t = 0; t < 4; ++t) bn[t] = wl[(8 * sn + t) * 32];
-        mfma_step8<NB>(c2, bw, acc);
+        mfma_step8<NB>(c[2], bw, acc);
       }
-      if (s0 + 3 < steps) {
-        const int sn = min(s0 + 4, steps - 1);
+      if (s0 + 3 < steps) mfma_step8<NB>(c[3], bn, acc);
+      if (g == G4 - 1) {
+        // accumulator register r of lane (h, j) holds output row 8*(r/4) + 4*h + r%4, column j
 #pragma unroll
-        for (int t = 0; t < 4; ++t) bw[t] = wl[(8 * sn + t) * 32];
-        mfma_step8<NB>(c3, bn, acc);
+        for (int r = 0; r < 16; ++r) {
+          const int x = blk * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+          if (rb0 * 32 + x < n_rows) {
+            float *dst = Y + (size_t)row_at(x) * N + j;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) dst[nb * 32] = acc[nb][r];
+          }
+        }
       }
-      c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    };
+    for (int gi = 0; gi < total_groups; gi += 3) {
+      load_group(gi + 2, set2);
+      run_group(gi, set0);
+      if (gi + 1 < total_groups) {
+        load_group(gi + 3, set0);
+        run_group(gi + 1, set1);
+      }
+      if (gi + 2 < total_groups) {
+        load_group(gi + 4, set1);
+        run_group(gi + 2, set2);
+      }
     }
-    // accumulator register r of lane (h, j) holds output row 8*(r/4) + 4*h + r%4, column j
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int oq = rb * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-      if (oq < n_rows) {
-        const int orow = rows ? rows[oq] : oq;
-        float *dst = Y + (size_t)orow * N + j;
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) dst[nb * 32] = acc[nb][r];
-      }
-    }
-    Xrow = Xnext;
-    row_ok = next_ok;
   }
 }
 
@@ -1405,13 +1403,16 @@ hipError_t launch_gemm(const float *X, const float *W, float *Y, const int *rows
     const int per_cu = 1;  // register use (accumulators + both operand pipelines) allows one 8-wave workgroup
     const int nrb = (n_rows + 31) / 32;
     const int grid = std::max(1, std::min(compute_units * per_cu, (nrb + kGemmBlock / 64 - 1) / (kGemmBlock / 64)));
-#define CALL(NB_)                                                                               \
-  err = allow_lds(gemm_rows_kernel<NB_>, w_bytes);                                              \
-  if (err == hipSuccess)                                                                        \
-    hipLaunchKernelGGL((gemm_rows_kernel<NB_>), dim3(grid), dim3(kGemmBlock), w_bytes, st, X, W, Y, \
+    const int lds = w_bytes + (rows ? (kGemmBlock / 64) * kGemmSeg * 32 * 4 : 0);  // + the wavefronts' row numbers
+#define CALL2(NB_, LIST_)                                                                           \
+  err = allow_lds(gemm_rows_kernel<NB_, LIST_>, lds);                                               \
+  if (err == hipSuccess)                                                                            \
+    hipLaunchKernelGGL((gemm_rows_kernel<NB_, LIST_>), dim3(grid), dim3(kGemmBlock), lds, st, X, W, Y, \
                        rows, n_rows, K)
+#define CALL(NB_) do { if (rows) { CALL2(NB_, true); } else { CALL2(NB_, false); } } while (0)
     TF_DISPATCH_NB(NB, CALL);
 #undef CALL
+#undef CALL2
     return err != hipSuccess ? err : hipGetLastError();
   }
   if (rows) return hipErrorInvalidValue;  // the streamed-W kernel takes contiguous rows only
