@@ -91,7 +91,9 @@ tf_status tf_dense_alloc(int M, int N, tf_dense **out); /* contents undefined */
 tf_status tf_dense_wrap_device(int M, int N, float *dptr, tf_dense **out);
 tf_status tf_dense_download(const tf_dense *d, float *host);
 tf_status tf_dense_fill(tf_dense *d, float value, void *stream);
-/* dst = src (same shape), device to device on the given stream. */
+/* dst = src (same shape), device to device on the given stream.  No counterpart in the reference
+ * (its operands never leave host memory); used to keep results on the device and by the
+ * benchmark's counter calibration. */
 tf_status tf_dense_copy(tf_dense *dst, const tf_dense *src, void *stream);
 float *tf_dense_device_ptr(const tf_dense *d);
 void tf_dense_free(tf_dense *d);
