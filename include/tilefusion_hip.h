@@ -123,7 +123,10 @@ enum { TF_OP_SPMM_SPMM = 0, TF_OP_GEMM_SPMM = 1 };
 typedef struct {
   int op;                /* TF_OP_SPMM_SPMM or TF_OP_GEMM_SPMM                               */
   int N;                 /* columns of C and D (reference: bCols / EmbedDim)                 */
-  int K;                 /* GeMM-SpMM: columns of dense B = rows of C (FeatureDim); else 0   */
+  int K;                 /* GeMM-SpMM: columns of dense B = rows of C (FeatureDim); else 0.
+                            Any K > 0: the kernels step k by 8, so for other K the executor
+                            copies B and C, zero-padded to the next multiple of 8, into the
+                            schedule's workspace on every call (counted in workspace_bytes) */
   int lds_budget_bytes;  /* LDS one fused tile may take; plays the role of the cache budget
                             ScheduleParameters::TileM of the reference's variable-tile
                             inspector.  Default 65536 (81920 when an inner pattern is
@@ -256,7 +259,8 @@ tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf
 /* Unfused building blocks, the reference's in-process baselines:
  * Y = A * X   (swiftware::sparse::spmmCsrParallel<float>, fusion/src/SpMM_SpMM.cpp:37-55) */
 tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, unsigned flags, void *stream);
-/* Y = X * W   (the cblas_sgemm call at fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:1144) */
+/* Y = X * W   (the cblas_sgemm call at fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:1144).
+ * Needs K % 8 == 0, N % 32 == 0 and N <= 256 (TF_EUNSUPPORTED otherwise): it has no workspace to pad into. */
 tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, void *stream);
 
 #ifdef __cplusplus

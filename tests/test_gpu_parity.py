@@ -267,6 +267,28 @@ def test_gemm_spmm_shapes(gpu, tf, orc, K, N):
     assert np.array_equal(got, exact)  # integer operands: exact whatever the summation order
 
 
+@pytest.mark.parametrize("M,K,N", [(1296, 1, 32), (1296, 20, 64), (1296, 30, 128), (1296, 129, 64), (36000, 20, 64),
+                                   (36000, 100, 128)])
+def test_gemm_spmm_any_k(gpu, tf, orc, M, K, N):
+    """The reference's executor takes any K (fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:218-291 hands
+    K straight to cblas_sgemm); here a K that is not a multiple of 8 is zero-padded into the
+    schedule's workspace on every call, for tiles and for streamed runs alike."""
+    say(f"gemm_spmm any K M={M} K={K} N={N}")
+    A = tf.workloads.banded_random(M, 32, 16, seed=80)
+    rng = np.random.default_rng(81 + K)
+    B = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    Cd = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    want, _ = orc.gemm_spmm(A, B, Cd, orc.unfused_schedule(M), nthreads=8)
+    got, info = run_gemm_spmm(tf, A, B, Cd, compute_units=256)
+    assert info["K"] == K and info["workspace_bytes"] >= (M + N) * ((K + 7) // 8 * 8) * 4
+    assert info["streamed"] == (1 if M >= 32768 else 0)
+    assert orc.rel_err(got, want) <= TOL
+    B2 = rng.uniform(-1, 1, (M, K)).astype(np.float32)  # second call: the padding is redone, not cached
+    want2, _ = orc.gemm_spmm(A, B2, Cd, orc.unfused_schedule(M), nthreads=8)
+    got2, _ = run_gemm_spmm(tf, A, B2, Cd, compute_units=256)
+    assert orc.rel_err(got2, want2) <= TOL
+
+
 @pytest.mark.parametrize("idx,scale", [(1, 1.0), (3, 0.02), (4, 2.0 ** -6)])
 def test_gemm_spmm_configs(gpu, tf, orc, idx, scale):
     cfg = tf.workloads.make_config(idx, scale)

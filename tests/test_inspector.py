@@ -174,6 +174,8 @@ def test_rectangular_and_bad_arguments(tf):
     with pytest.raises(tf.TileFusionError) as e:
         tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=48, K=64)
     assert e.value.status == -5
+    Sq = tf.inspector(tf.CsrMatrix.from_scipy(A2[:, :200]), 1, op=tf.OP_GEMM_SPMM, N=64, K=20)  # any K: padded to 24
+    assert Sq.info()["K"] == 20 and Sq.info()["workspace_bytes"] >= (200 + 64) * 24 * 4
     bad = tf.CsrMatrix(4, 4, [0, 1, 2, 3, 4], [0, 1, 9, 3], [1, 1, 1, 1])
     with pytest.raises(tf.TileFusionError):
         tf.inspector(bad, 1, op=tf.OP_SPMM_SPMM, N=8)

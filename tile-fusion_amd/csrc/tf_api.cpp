@@ -41,6 +41,8 @@ struct DeviceSchedule {
   LongRow *long_rows = nullptr;
   float *inter = nullptr;    // M x N intermediate, only if some tile writes back
   float *partial = nullptr;  // n_long_chunks x N
+  float *Bpad = nullptr;     // M x K' and K' x N copies of B and C, zero-padded, when K is not a multiple of 8
+  float *Cpad = nullptr;
 };
 
 // launchers in tf_kernels.hip
@@ -62,6 +64,7 @@ hipError_t launch_fused_gemm_spmm_stream(const TileDesc *, int, const int *, con
                                          const float *, float *, float *, int, int, hipStream_t);
 hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t);
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
+hipError_t launch_pad(const float *, int, int, float *, int, int, hipStream_t);
 
 static thread_local char g_err[512] = "";
 
@@ -97,7 +100,7 @@ void release_device_schedule(DeviceSchedule *d) {
   (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows); (void)hipFree(d->plain_rows);
   (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows);
   (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
-  (void)hipFree(d->inter); (void)hipFree(d->partial);
+  (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad);
   delete d;
 }
 
@@ -136,6 +139,11 @@ static tf_status ensure_device(tf_schedule *s) {
   if (!rc && s->n_writeback_rows > 0) {
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->inter), (size_t)s->M * s->opts.N * sizeof(float));
     if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(intermediate)");
+  }
+  if (!rc && s->opts.op == TF_OP_GEMM_SPMM && s->user_K != s->opts.K) {
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->Bpad), (size_t)s->M * s->opts.K * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&d->Cpad), (size_t)s->opts.K * s->opts.N * sizeof(float));
+    if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(padded operands)");
   }
   if (!rc && !s->long_chunks.empty()) {
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->partial), s->long_chunks.size() * (size_t)s->opts.N * sizeof(float));
@@ -417,24 +425,31 @@ extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_d
   if (rc) return rc;
   if (!B) return fail(TF_EINVAL, "tf_gemm_spmm: B is null");
   if (B->M != A->N) return fail(TF_EINVAL, "tf_gemm_spmm: B has %d rows, A has %d columns", B->M, A->N);
-  if (B->N != s->opts.K || C->M != s->opts.K)
-    return fail(TF_ESCHEDULE, "tf_gemm_spmm: schedule was built for K = %d, B has %d columns and C has %d rows", s->opts.K, B->N, C->M);
+  if (B->N != s->user_K || C->M != s->user_K)
+    return fail(TF_ESCHEDULE, "tf_gemm_spmm: schedule was built for K = %d, B has %d columns and C has %d rows", s->user_K, B->N, C->M);
   rc = tf::ensure_device(s);
   if (rc) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
   const tf::DeviceSchedule *d = s->dev;
+  const float *Bd = B->d, *Cd = C->d;
+  if (s->user_K != s->opts.K) {  // zero-padded copies with K rounded up to 8 (the kernels' k step)
+    TF_HIP(tf::launch_pad(B->d, B->M, B->N, d->Bpad, B->M, s->opts.K, st));
+    TF_HIP(tf::launch_pad(C->d, C->M, C->N, d->Cpad, s->opts.K, C->N, st));
+    Bd = d->Bpad;
+    Cd = d->Cpad;
+  }
   if (s->gemm_stream)
     TF_HIP(tf::launch_fused_gemm_spmm_stream(d->tiles, (int)s->launch_tiles.size(), d->step_begin, d->step_ptr,
-                                             d->fused_rec, B->d, C->d, s->opts.K, s->opts.N, s->ring_rows,
+                                             d->fused_rec, Bd, Cd, s->opts.K, s->opts.N, s->ring_rows,
                                              A->i, A->x, D->d, d->inter, s->lds_bytes, acc, st));
   else
-  TF_HIP(tf::launch_fused_gemm_spmm(d->tiles, (int)s->launch_tiles.size(), d->fused_ids, B->d, C->d,
-                                    s->opts.K, s->gemm_kc, A->p, A->i, A->x, D->d, d->inter,
-                                    s->opts.N, s->lds_bytes, acc, s->opts.compute_units, s->gemm_regw ? 1 : 0, st));
+    TF_HIP(tf::launch_fused_gemm_spmm(d->tiles, (int)s->launch_tiles.size(), d->fused_ids, Bd, Cd,
+                                      s->opts.K, s->gemm_kc, A->p, A->i, A->x, D->d, d->inter,
+                                      s->opts.N, s->lds_bytes, acc, s->opts.compute_units, s->gemm_regw ? 1 : 0, st));
   if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
     const bool all = (int)s->plain_rows.size() == s->M;
-    TF_HIP(tf::launch_gemm(B->d, C->d, d->inter, all ? nullptr : d->plain_rows, (int)s->plain_rows.size(),
+    TF_HIP(tf::launch_gemm(Bd, Cd, d->inter, all ? nullptr : d->plain_rows, (int)s->plain_rows.size(),
                            s->opts.K, s->opts.N, s->opts.compute_units, st));
   }
   return tf::run_remainder(A, D, s, acc, st);

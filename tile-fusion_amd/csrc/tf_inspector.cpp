@@ -43,14 +43,16 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     return tf::fail(TF_EUNSUPPORTED, "tf_inspect: rows*N exceeds int32 indexing");
   if (o.op == TF_OP_GEMM_SPMM) {
     if (o.K <= 0) return tf::fail(TF_EINVAL, "tf_inspect: GeMM-SpMM needs K > 0");
-    if (o.K % 8 != 0 || o.N % 32 != 0)
-      return tf::fail(TF_EUNSUPPORTED,
-                      "tf_inspect: the MFMA tile GEMM needs K %% 8 == 0 and N %% 32 == 0 (K=%d N=%d)",
-                      o.K, o.N);
+    if (o.N % 32 != 0)
+      return tf::fail(TF_EUNSUPPORTED, "tf_inspect: the MFMA tile GEMM needs N %% 32 == 0 (N=%d)", o.N);
     if (o.N > 256) return tf::fail(TF_EUNSUPPORTED, "tf_inspect: GeMM-SpMM supports N <= 256");
   } else {
     o.K = 0;
   }
+  // The MFMA kernels walk k in steps of 8: a K that is not a multiple of 8 is rounded up here and
+  // the executor pads B's columns and C's rows with zeros into its workspace on every call.
+  const int user_K = o.K;
+  o.K = (o.K + 7) / 8 * 8;
   const bool has_inner = o.op == TF_OP_SPMM_SPMM && o.inner_Ap != nullptr;
   // GeMM-SpMM tiles keep C in registers when a wavefront's K x 16 slice (two slices when
   // N > 128) fits 64 registers per lane; LDS then holds only the slab, rows padded by 4 floats.
@@ -118,6 +120,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     S->M = M;
     S->nnz = nnz;
     S->gemm_kc = gemm_kc;
+    S->user_K = user_K;
     S->gemm_regw = gemm_regw;
     S->gemm_stream = gemm_stream;
     S->ring_rows = ring_rows;
@@ -469,7 +472,7 @@ extern "C" void tf_schedule_free(tf_schedule *s) {
 extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info *info) {
   if (!s || !info) return tf::fail(TF_EINVAL, "tf_schedule_get_info: null argument");
   std::memset(info, 0, sizeof(*info));
-  info->op = s->opts.op; info->N = s->opts.N; info->K = s->opts.K;
+  info->op = s->opts.op; info->N = s->opts.N; info->K = s->user_K;
   info->rows = s->L; info->inter_rows = s->M;
   info->n_tiles = (int)s->tiles.size();
   info->n_fused_rows = (int)s->fused_ids.size();
@@ -489,6 +492,7 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   long long ws = 0;
   if (s->n_writeback_rows > 0) ws += (long long)s->M * s->opts.N * 4;
   ws += (long long)s->long_chunks.size() * s->opts.N * 4;
+  if (s->user_K != s->opts.K) ws += ((long long)s->M + s->opts.N) * s->opts.K * 4;  // padded copies of B and C
   info->workspace_bytes = ws;
   return TF_OK;
 }

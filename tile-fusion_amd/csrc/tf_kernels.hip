@@ -276,12 +276,11 @@ __device__ __forceinline__ fvec<4> window_unit(const float *__restrict__ C, int 
   return *reinterpret_cast<const fvec<4> *>(C + (size_t)(first_row + uu / LPR) * N + c0 + (uu % LPR) * 4);
 }
 
-template <int SW, int BLOCK>
+template <int SW, int BLOCK, bool ACC>
 __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
     const TileDesc *__restrict__ tiles, const int2 *__restrict__ win, int n_tiles, int per_xcd,
     const int *__restrict__ fused_ids, const int *__restrict__ Bp, const int *__restrict__ Bi,
-    const float *__restrict__ Bx, const float *__restrict__ C, float *__restrict__ D, int N,
-    int accumulate) {
+    const float *__restrict__ Bx, const float *__restrict__ C, float *__restrict__ D, int N) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int LPR = SW / 4;           // lanes per row
   constexpr int G = BLOCK / LPR;        // rows in flight per workgroup
@@ -348,7 +347,9 @@ __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
       const int r = cons[q];
       float *dst = D + (size_t)(t.prod_begin + r) * N + c0 + glane * 4;
       fvec<4> acc = vzero<4>();
-      if (accumulate) acc = *reinterpret_cast<const fvec<4> *>(dst);
+      // (a compile-time switch: a load under a run-time condition would make every store of
+      // this loop wait for the one before it)
+      if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
       acc = lds_row_dot(ent, rp[r], rp[r + 1] - kWinPad, tbase, acc);
       *reinterpret_cast<fvec<4> *>(dst) = acc;
     }
@@ -426,6 +427,16 @@ __global__ __launch_bounds__(kBlock) void long_row_reduce_kernel(const LongRow *
     float s = accumulate ? Y[(size_t)lr.row * N + c] : 0.f;
     for (int p = 0; p < lr.count; ++p) s += partial[(size_t)(lr.first + p) * N + c];
     Y[(size_t)lr.row * N + c] = s;
+  }
+}
+
+// dst (rows x ld_dst) = src (src_rows x ld_src) in its top left corner, zeros elsewhere.
+__global__ void pad_kernel(const float *__restrict__ src, int src_rows, int ld_src, float *__restrict__ dst, int rows,
+                           int ld_dst) {
+  const size_t n = (size_t)rows * ld_dst;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const int r = (int)(i / ld_dst), c = (int)(i % ld_dst);
+    dst[i] = (r < src_rows && c < ld_src) ? src[(size_t)r * ld_src + c] : 0.f;
   }
 }
 
@@ -1260,17 +1271,17 @@ hipError_t launch_fused_spmm_spmm_window(const TileDesc *tiles, const int *win, 
   const int per = per_xcd_of(n_tiles);
   const int2 *w2 = reinterpret_cast<const int2 *>(win);
   hipError_t err;
+#define CALLW(SW_, ACC_)                                                                               \
+  err = allow_lds(fused_spmm_spmm_window_kernel<SW_, BLOCK, ACC_>, lds_bytes);                         \
+  if (err == hipSuccess)                                                                               \
+    hipLaunchKernelGGL((fused_spmm_spmm_window_kernel<SW_, BLOCK, ACC_>), dim3(grid_of(n_tiles)), dim3(BLOCK), \
+                       lds_bytes, st, tiles, w2, n_tiles, per, fused_ids, Bp, Bi, Bx, C, D, N)
   if (strip == 32) {
-    err = allow_lds(fused_spmm_spmm_window_kernel<32, BLOCK>, lds_bytes);
-    if (err == hipSuccess)
-      hipLaunchKernelGGL((fused_spmm_spmm_window_kernel<32, BLOCK>), dim3(grid_of(n_tiles)), dim3(BLOCK), lds_bytes,
-                         st, tiles, w2, n_tiles, per, fused_ids, Bp, Bi, Bx, C, D, N, accumulate);
+    if (accumulate) { CALLW(32, true); } else { CALLW(32, false); }
   } else {
-    err = allow_lds(fused_spmm_spmm_window_kernel<64, BLOCK>, lds_bytes);
-    if (err == hipSuccess)
-      hipLaunchKernelGGL((fused_spmm_spmm_window_kernel<64, BLOCK>), dim3(grid_of(n_tiles)), dim3(BLOCK), lds_bytes,
-                         st, tiles, w2, n_tiles, per, fused_ids, Bp, Bi, Bx, C, D, N, accumulate);
+    if (accumulate) { CALLW(64, true); } else { CALLW(64, false); }
   }
+#undef CALLW
   return err != hipSuccess ? err : hipGetLastError();
 }
 
@@ -1428,6 +1439,14 @@ hipError_t launch_gemm(const float *X, const float *W, float *Y, const int *rows
   TF_DISPATCH_NB(NB, CALL);
 #undef CALL
   return err != hipSuccess ? err : hipGetLastError();
+}
+
+hipError_t launch_pad(const float *src, int src_rows, int ld_src, float *dst, int rows, int ld_dst, hipStream_t st) {
+  const size_t n = (size_t)rows * ld_dst;
+  if (n == 0) return hipSuccess;
+  const int blocks = (int)std::min<size_t>((n + kBlock - 1) / kBlock, 65536);
+  hipLaunchKernelGGL(pad_kernel, dim3(blocks), dim3(kBlock), 0, st, src, src_rows, ld_src, dst, rows, ld_dst);
+  return hipGetLastError();
 }
 
 hipError_t launch_fill(float *p, size_t n, float v, hipStream_t st) {

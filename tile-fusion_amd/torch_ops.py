@@ -23,7 +23,8 @@ Differences from the reference, all forced by where the data lives:
     adjacency and a pair of widths is built once and cached, so any schedule tensors that were
     made for the same adjacency select the same kernels.  MTileSize, CacheSize, NumThreads and
     MaxTileSize are accepted and ignored (tiles are sized by the LDS, not by a CPU cache).
-  * Widths that the MFMA tile GEMM does not take (K % 8, N % 32) are zero-padded on the fly.
+  * Output widths that the MFMA tile GEMM does not take (N % 32, N > 256) are zero-padded or split here;
+    the library itself takes any K.
   * The backward pass uses the transpose of the adjacency (the reference multiplies by the
     adjacency itself, Functions.cpp:840-852, which is only right for a symmetric matrix).
 """
@@ -163,10 +164,6 @@ def _gemm_spmm(ctx, X, Wkn):
         raise RuntimeError(f"sw_gcn: shapes do not chain: Adj {ctx.shape}, Feature {tuple(X.shape)}, weight {tuple(Wkn.shape)}")
     X = X.to(torch.float32)
     Wkn = Wkn.to(torch.float32)
-    Kp = _pad_to(K, 8)
-    if Kp != K:
-        X = torch.nn.functional.pad(X, (0, Kp - K))
-        Wkn = torch.nn.functional.pad(Wkn, (0, 0, 0, Kp - K))
     X = X.contiguous()
     out = torch.empty((ctx.shape[0], N), dtype=torch.float32, device=X.device)
     for n0 in range(0, N, _MAX_N):  # the library schedules at most 256 columns per call
@@ -178,7 +175,7 @@ def _gemm_spmm(ctx, X, Wkn):
         Wc = Wc.contiguous()
         whole = (n0 == 0 and n1 == N and Np == N)
         dst = out if whole else torch.empty((ctx.shape[0], Np), dtype=torch.float32, device=X.device)
-        S = ctx.schedule(Kp, Np)
+        S = ctx.schedule(K, Np)
         with _Dense(X) as xb, _Dense(Wc) as wc, _Dense(dst) as db:
             _b._check(_b.lib().tf_gemm_spmm(ctx.h, xb, wc, db, S.h, 0, _stream()))
         if not whole:
