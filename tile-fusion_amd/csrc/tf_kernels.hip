@@ -267,6 +267,51 @@ __device__ __forceinline__ fvec<4> lds_row_dot8(const int2 *__restrict__ ent, in
   return lds_row_dot(ent, k, ke, base, acc);
 }
 
+// The value lane G of the caller's quad holds (a DPP quad_perm broadcast, folded into the
+// consuming instruction: no LDS traffic and no instruction of its own).
+template <int G> __device__ __forceinline__ int quad_bcast(int v) {
+  return __builtin_amdgcn_mov_dpp(v, G * 0x55, 0xf, 0xf, true);
+}
+
+// Eight staged entries, held four to a lane by lanes GA and GB of the quad: gathers first, then the fmas in order.
+template <int GA, int GB, bool CHECK>
+__device__ __forceinline__ void quad_dot8(const int2 (&e)[4], const char *base, int left, fvec<4> &acc) {
+  fvec<4> x[8];
+  int val[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    val[j] = quad_bcast<GA>(e[j].y);
+    val[4 + j] = quad_bcast<GB>(e[j].y);
+    if (!CHECK || 4 * GA + j < left) x[j] = *reinterpret_cast<const fvec<4> *>(base + quad_bcast<GA>(e[j].x));
+    if (!CHECK || 4 * GB + j < left) x[4 + j] = *reinterpret_cast<const fvec<4> *>(base + quad_bcast<GB>(e[j].x));
+  }
+#pragma unroll
+  for (int u = 0; u < 8; ++u)
+    if (!CHECK || (u < 4 ? 4 * GA + u : 4 * GB + u - 4) < left) vfma<4>(__int_as_float(val[u]), x[u], acc);
+}
+
+// acc += sum_k val[k] * row(off[k]) over staged entries [kb, ke), in order, for a lane group
+// that is a whole number of quads.  A lane reads only every fourth run of four entries
+// (q = its position in its quad says which); the other twelve of each sixteen come from its
+// quad's lanes through DPP.  Against lds_row_dot this trades one LDS read of 8 bytes per lane
+// and entry for one of 32 bytes per lane and sixteen entries.
+__device__ __forceinline__ fvec<4> lds_row_dot_quad(const int2 *__restrict__ ent, int kb, int ke, const char *base,
+                                                    int q, fvec<4> acc) {
+  for (int c = kb; c < ke; c += 16) {
+    const int2 *p = ent + c + 4 * q;  // (may run past the row's end: those entries are not used)
+    const int2 e[4] = {p[0], p[1], p[2], p[3]};
+    const int left = ke - c;
+    if (left >= 16) {
+      quad_dot8<0, 1, false>(e, base, left, acc);
+      quad_dot8<2, 3, false>(e, base, left, acc);
+    } else {
+      quad_dot8<0, 1, true>(e, base, left, acc);
+      if (left > 8) quad_dot8<2, 3, true>(e, base, left, acc);
+    }
+  }
+  return acc;
+}
+
 // One 16-byte unit of a strip of the window of C (unit u = row-in-window * LPR + quad).
 // Threads past the end re-read unit 0, which always exists; the value is not used.
 template <int LPR>
@@ -339,7 +384,7 @@ __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
     }
     __syncthreads();
     for (int r = group; r < P; r += G) {
-      const fvec<4> acc = lds_row_dot(ent, rp[r], rp[r + 1] - kWinPad, cbase, vzero<4>());
+      const fvec<4> acc = lds_row_dot_quad(ent, rp[r], rp[r + 1] - kWinPad, cbase, glane & 3, vzero<4>());
       *reinterpret_cast<fvec<4> *>(Tbuf + r * SW + glane * 4) = acc;
     }
     __syncthreads();
@@ -350,7 +395,7 @@ __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
       // (a compile-time switch: a load under a run-time condition would make every store of
       // this loop wait for the one before it)
       if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
-      acc = lds_row_dot(ent, rp[r], rp[r + 1] - kWinPad, tbase, acc);
+      acc = lds_row_dot_quad(ent, rp[r], rp[r + 1] - kWinPad, tbase, glane & 3, acc);
       *reinterpret_cast<fvec<4> *>(dst) = acc;
     }
   }
