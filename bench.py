@@ -102,6 +102,8 @@ def main():
     ap.add_argument("--max-redundancy", type=float, default=0.0)
     ap.add_argument("--strip", type=int, default=0, help="columns per strip of windowed tiles (32 or 64)")
     ap.add_argument("--no-window", action="store_true", help="do not build windowed tiles")
+    ap.add_argument("--wide", type=int, default=0, choices=[-1, 0, 1],
+                    help="windowed tiles: 1 = the 64-column, 1024-thread kernel, -1 = the lane-group kernel, 0 = library's choice")
     ap.add_argument("--xcd-chunk", type=int, default=0, help="rows per XCD turn of the row kernels (-1 contiguous)")
     ap.add_argument("--long-row", type=int, default=0, help="rows with more entries than this are chunked")
     ap.add_argument("--matrix", default=None, help="run on a .mtx / .smtx file instead of a synthetic configuration "
@@ -147,7 +149,7 @@ def main():
     t0 = time.perf_counter()
     inner = Ah if (op == tf.OP_SPMM_SPMM and cfg["B"] is A and not args.no_window) else None
     S = tf.inspector(Ah, 1, op=op, N=N, K=K, lds_budget_bytes=args.lds, tile_rows=args.tile_rows,
-                     max_redundancy=args.max_redundancy, inner=inner, strip_cols=args.strip,
+                     max_redundancy=args.max_redundancy, inner=inner, strip_cols=args.strip, wide_strips=args.wide,
                      long_row_nnz=args.long_row, xcd_chunk_rows=args.xcd_chunk)
     inspect_s = time.perf_counter() - t0
     S.validate()
@@ -205,14 +207,15 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": cfg["name"], "op": cfg["op"], "rows": int(A.shape[0]), "nnz": int(A.nnz), "N": N, "K": K,
-                   "lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "streamed": bool(info["streamed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
+                   "lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "wide_strips": bool(info["wide_strips"]), "streamed": bool(info["streamed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
                    "remainder_rows": info["n_remainder_rows"], "recomputed_rows": info["n_producer_rows"] - A.shape[1],
                    "writeback_rows": info["n_writeback_rows"], "kernels_per_step": n_kernels,
                    "inspector_s": round(inspect_s, 4), "rel_err_vs_f64": check, "device": dev["arch"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes": int(alg_bytes), "kernel_ms": round(dev_ms, 5),
-                     "kernel": ("fused_spmm_spmm_window_kernel" if info["windowed"] else
+                     "kernel": ("fused_spmm_spmm_window64_kernel" if info["wide_strips"] else
+                                "fused_spmm_spmm_window_kernel" if info["windowed"] else
                                 "fused_spmm_spmm_kernel" if info["n_fused_rows"] else "spmm_rows_kernel (twice)")
                      if op == tf.OP_SPMM_SPMM else ("gemm_rows_kernel + spmm_rows_kernel" if args.unfused or info["n_fused_rows"] == 0 else
                                                     "fused_gemm_spmm_stream_kernel" if info["streamed"] else "fused_gemm_spmm_kernel"),

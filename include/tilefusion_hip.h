@@ -157,6 +157,14 @@ typedef struct {
                             (default), n > 0 = chunks of n rows per XCD turn (a 3D stencil with
                             plane distance d keeps its halo in one L2 with n = d/8), -1 = one
                             contiguous run of rows per XCD                                     */
+  int wide_strips;       /* which kernel runs windowed tiles: 1 = strips of 64 columns (N % 64 == 0),
+                            one workgroup of 1024 threads and up to 160 KB of LDS per tile, the
+                            entries read from the CSR arrays in place (LDS rows of 256 bytes are
+                            read without bank conflicts), tile_rows defaults to rows / compute
+                            units; -1 = strips of strip_cols columns, the tile's entries staged in
+                            LDS, two workgroups per compute unit; 0 = the first for matrices of
+                            128 rows per compute unit or more when strip_cols, tile_rows and
+                            lds_budget_bytes are left at 0, else the second                    */
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -191,6 +199,7 @@ typedef struct {
   int xcd_chunk_rows;    /* rows per XCD turn of the row kernels (0: round-robin, -1: contiguous) */
   int streamed;          /* 1 when GeMM-SpMM tiles are long runs streamed through an LDS ring */
   int ring_rows;         /* intermediate rows the ring holds, else 0                 */
+  int wide_strips;       /* 1 when windowed tiles run on the 64-column, 1024-thread kernel */
   long long fused_nnz;   /* stored entries of A in fused rows (getFusedNnzNum)      */
   long long workspace_bytes; /* device memory the executor keeps (intermediate + partials) */
 } tf_schedule_info;

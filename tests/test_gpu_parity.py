@@ -224,6 +224,61 @@ def test_spmm_spmm_windowed_bit_exact(gpu, tf, orc, N, strip):
         assert orc.rel_err(D.to_numpy(), D0.astype(np.float64) + want) <= 1e-6
 
 
+def ragged_band(M, reach, max_len, seed):
+    """Rows of 0 .. max_len entries at random columns within `reach` of the diagonal; the last
+    row's length is not a multiple of four."""
+    rng = np.random.default_rng(seed)
+    rows, cols = [], []
+    for i in range(M):
+        lo, hi = max(0, i - reach), min(M, i + reach + 1)
+        n = int(rng.integers(0, min(max_len, hi - lo) + 1))
+        if i == M - 1:
+            n = 7
+        if i % 97 == 5:
+            n = 0
+        c = rng.choice(np.arange(lo, hi), n, replace=False)
+        rows += [i] * n
+        cols += list(c)
+    vals = rng.uniform(-1, 1, len(rows)).astype(np.float32)
+    return sp.csr_matrix((vals, (rows, cols)), shape=(M, M), dtype=np.float32)
+
+
+@pytest.mark.parametrize("N", [128, 64, 192, 256])
+def test_spmm_spmm_wide_strips_bit_exact(gpu, tf, orc, N):
+    """Long matrices get one windowed tile per compute unit, worked on in 64-column strips by
+    1024 threads with the entries read from the CSR arrays in place (a lane loads four of
+    every sixteen, the rest come through its quad).  Rows of 0 to 40 entries, a last row that
+    ends the arrays at an odd length, D +=, and the same schedule with another B."""
+    say(f"spmm_spmm wide strips N={N}")
+    for A, kw in ((tf.workloads.banded_random(5000, 32, 16, seed=41), dict(compute_units=16)),
+                  (ragged_band(4100, 24, 40, seed=42), dict(compute_units=16)),
+                  (ragged_band(3000, 10, 13, seed=43), dict(wide_strips=1, tile_rows=100)),
+                  (tf.workloads.laplacian_2d(40, 70), dict(wide_strips=1))):
+        M = A.shape[0]
+        Cd = tf.workloads.uniform((M, N), 44)
+        want = oracle_spmm_spmm(orc, A, A, Cd)
+        Ah = tf.CsrMatrix.from_scipy(A)
+        S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N, inner=Ah, **kw)
+        S.validate()
+        info = S.info()
+        assert info["windowed"] == 1 and info["wide_strips"] == 1 and info["strip_cols"] == 64
+        assert info["n_fused_rows"] == M and info["n_writeback_rows"] == 0 and info["lds_bytes"] <= 163840
+        D = tf.DenseMatrix(M, N)
+        D.fill(float("nan"))
+        tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(Cd), D, S)
+        tf.device_synchronize()
+        assert np.array_equal(D.to_numpy(), want), (N, kw)
+        D0 = tf.workloads.uniform((M, N), 45)
+        D = tf.DenseMatrix.from_numpy(D0)
+        tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(Cd), D, S, accumulate=True)
+        assert orc.rel_err(D.to_numpy(), D0.astype(np.float64) + want) <= 1e-6
+        B2 = A.copy()
+        B2.data = tf.workloads.uniform((A.nnz,), 46)
+        D = tf.DenseMatrix(M, N)
+        tf.spmm_spmm(Ah, tf.CsrMatrix.from_scipy(B2), tf.DenseMatrix.from_numpy(Cd), D, S)
+        assert np.array_equal(D.to_numpy(), oracle_spmm_spmm(orc, A, B2, Cd))
+
+
 def test_spmm_spmm_windowed_schedule_with_other_inner_matrix(gpu, tf, orc):
     """A windowed schedule used with B != A falls back to the kernel that gathers C from
     HBM (same tiles), and refuses an inner matrix of another size."""

@@ -214,6 +214,28 @@ def test_windowed_tiles(tf):
     assert tf.inspector(Rh, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Rh).info()["windowed"] == 0
 
 
+def test_wide_strip_tiles(tf):
+    """A matrix with 128 rows per compute unit or more gets one windowed tile per compute unit
+    for the 64-column kernel: LDS holds row pointers, window and slab (no entries), up to
+    160 KB; any explicit strip, tile or LDS choice keeps the lane-group kernel's tiles."""
+    A = tf.workloads.banded_random(4096, 32, 16, seed=3)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128, inner=Ah, compute_units=16)
+    S.validate()
+    info, view = S.info(), S.view()
+    assert info["windowed"] == 1 and info["wide_strips"] == 1 and info["strip_cols"] == 64 and info["n_tiles"] == 16
+    assert info["n_fused_rows"] == 4096 and info["n_writeback_rows"] == 0
+    tr = view["tile_range"].reshape(-1, 4)
+    P = int((tr[:, 1] - tr[:, 0]).max())  # producer rows of the largest tile: window and slab each hold at least as many
+    assert 4 * 64 * 2 * P <= info["lds_bytes"] <= 163840
+    validate(view, info, A, 163840)
+    for kw in (dict(compute_units=64), dict(compute_units=16, strip_cols=32), dict(compute_units=16, tile_rows=128),
+               dict(compute_units=16, lds_budget_bytes=65536), dict(compute_units=16, wide_strips=-1)):
+        assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128, inner=Ah, **kw).info()["wide_strips"] == 0, kw
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=96, inner=Ah, compute_units=16).info()["wide_strips"] == 0
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah, compute_units=64, wide_strips=1).info()["wide_strips"] == 1
+
+
 def test_xcd_chunk_is_the_callers_choice(tf):
     A = tf.workloads.laplacian_3d(40)
     Ah = tf.CsrMatrix.from_scipy(A)

@@ -52,6 +52,9 @@ hipError_t launch_fused_spmm_spmm(const TileDesc *, int, const int *, const int 
 hipError_t launch_fused_spmm_spmm_window(const TileDesc *, const int *, int, const int *, const int *,
                                          const int *, const float *, const float *, float *, int, int,
                                          int, int, hipStream_t);
+hipError_t launch_fused_spmm_spmm_window64(const TileDesc *, const int *, int, const int *, const int *,
+                                           const float *, int, const float *, const int *, const int *,
+                                           const float *, int, float *, int, int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
                             float *, int, int, int, hipStream_t);
 hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const int *, const float *,
@@ -399,6 +402,12 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
                   s->inner_nnz, s->opts.inner_cols, B->nnz, B->N);
     // The windowed kernel walks one staged CSR chunk for both products: B must be A.
     const bool same = (B == A) || (B->p == A->p && B->i == A->i && B->x == A->x);
+    if (s->win_wide && A->nnz >= 4) {  // reads B's entries for the first product and A's for the second, in place
+      TF_HIP(tf::launch_fused_spmm_spmm_window64(d->tiles, d->win, (int)s->launch_tiles.size(), B->p, B->i, B->x,
+                                                 B->nnz, C->d, A->p, A->i, A->x, A->nnz, D->d, s->opts.N,
+                                                 s->lds_bytes, acc, st));
+      return TF_OK;
+    }
     if (same) {
       TF_HIP(tf::launch_fused_spmm_spmm_window(d->tiles, d->win, (int)s->launch_tiles.size(), d->fused_ids, A->p,
                                                A->i, A->x, C->d, D->d, s->opts.N, s->opts.strip_cols,

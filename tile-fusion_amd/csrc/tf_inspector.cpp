@@ -102,8 +102,13 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   if (o.strip_cols <= 0) o.strip_cols = 32;
   if (o.strip_cols != 32 && o.strip_cols != 64)
     return tf::fail(TF_EINVAL, "tf_inspect: strip_cols must be 32 or 64");
-  const bool want_window = o.op == TF_OP_SPMM_SPMM && o.inner_Ap && (o.inner_Ai || o.inner_Ap[M] == 0) &&
-                           o.inner_cols > 0 && o.N % o.strip_cols == 0;
+  const bool have_inner = o.op == TF_OP_SPMM_SPMM && o.inner_Ap && (o.inner_Ai || o.inner_Ap[M] == 0) && o.inner_cols > 0;
+  const bool want_window = have_inner && o.N % o.strip_cols == 0 && o.wide_strips <= 0;
+  // (one tile per compute unit: a matrix with fewer than 128 rows per compute unit is better
+  // served by more and smaller tiles)
+  const bool want_wide = have_inner && o.N % 64 == 0 && o.inner_Ap[M] >= 4 && nnz >= 4 &&
+                         (o.wide_strips > 0 || (o.wide_strips == 0 && user->strip_cols <= 0 && user->lds_budget_bytes <= 0 &&
+                                              user->tile_rows <= 0 && M >= 128LL * o.compute_units));
   int r_cap = o.tile_rows > 0 ? o.tile_rows : ceil_div(M, 2 * o.compute_units);
   if (o.op == TF_OP_GEMM_SPMM) r_cap = ceil_div(r_cap, 32) * 32;
   r_cap = std::max(r_cap, o.tile_rows > 0 ? 1 : 64);  // smaller tiles spend most of their work on halo rows
@@ -148,10 +153,17 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     // ---- windowed tiles (SpMM-SpMM with a known inner pattern) -------------------------
     // Every row must fuse, and the rows of C that a tile's producer rows read must form a
     // window small enough to sit in LDS next to the slab, one strip of columns at a time.
-    bool windowed = false;
-    if (want_window) {
+    // Two kernels run such tiles.  Wide strips: 64 columns at a time, LDS holds the window,
+    // the slab and the row pointers, the entries are read from the CSR arrays in place, and
+    // one workgroup of 1024 threads owns a compute unit and all of its LDS (a tile per compute
+    // unit: long matrices).  Narrow strips: 32 or 64 columns, the tile's entries staged in LDS
+    // as well, two workgroups per compute unit.
+    bool windowed = false, win_wide = false;
+    auto build_window = [&](bool wide) {
       const int *Bp = o.inner_Ap, *Bi = o.inner_Ai;
-      const int SW = o.strip_cols;
+      const int SW = wide ? 64 : o.strip_cols;
+      const int budget = wide ? (user->lds_budget_bytes > 0 ? user->lds_budget_bytes : kMaxLds) : o.lds_budget_bytes;
+      const int cap = wide ? (user->tile_rows > 0 ? user->tile_rows : std::max(64, ceil_div(M, o.compute_units))) : r_cap;
       std::vector<int> blo(M), bhi(M);
       bool ok = (Bp[0] == 0);
       for (int r = 0; r < M && ok; ++r) {
@@ -168,6 +180,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       }
       auto a16 = [](long long x) { return (x + 15) / 16 * 16; };
       auto lds_of = [&](int P, int R, long long nz, int Wc) {
+        if (wide) return a16(4LL * (P + 1)) + a16(4LL * (R + 1)) + 4LL * SW * ((long long)Wc + P);
         return a16(4LL * (P + 1)) + a16(4LL * R) + a16(8LL * (nz + 2LL * P)) + 4LL * SW * ((long long)Wc + P);  // 2 = pad slots per staged row
       };
       std::vector<tf::TileDesc> tiles;
@@ -177,18 +190,18 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       int s = 0;
       while (ok && s < M) {
         int wlo = s, whi = s, clo = INT_MAX, chi = 0, e = s;
-        while (e < M && e - s < r_cap) {
+        while (e < M && e - s < cap) {
           int nlo = std::min(wlo, e), nhi = std::max(whi, e + 1);
           if (e < L) { nlo = std::min(nlo, lo[e]); nhi = std::max(nhi, hi[e]); }
           int nclo = clo, nchi = chi;
           for (int r = nlo; r < wlo; ++r) { nclo = std::min(nclo, blo[r]); nchi = std::max(nchi, bhi[r]); }
           for (int r = std::max(whi, nlo); r < nhi; ++r) { nclo = std::min(nclo, blo[r]); nchi = std::max(nchi, bhi[r]); }
           const int Wc = nchi > nclo ? nchi - nclo : 0;
-          if (lds_of(nhi - nlo, e + 1 - s, (long long)Bp[nhi] - Bp[nlo], Wc) > o.lds_budget_bytes) break;
+          if (lds_of(nhi - nlo, e + 1 - s, (long long)Bp[nhi] - Bp[nlo], Wc) > budget) break;
           wlo = nlo; whi = nhi; clo = nclo; chi = nchi; ++e;
         }
         // (the last tile of the matrix may be short, and then has relatively more halo: 1.5x the limit)
-        if (e == s || (e != M && e - s < std::min(r_cap, 16)) ||
+        if (e == s || (e != M && e - s < std::min(cap, 16)) ||
             (float)(whi - wlo) > (e == M ? 1.5f : 1.0f) * o.max_redundancy * (float)(e - s)) { ok = false; break; }
         tf::TileDesc t{};
         t.own_begin = s; t.own_end = e; t.prod_begin = wlo; t.prod_end = whi;
@@ -204,18 +217,22 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         tiles.push_back(t);
         s = e;
       }
-      if (ok && L <= M) {
-        windowed = true;
-        S->inner_nnz = Bp[M];
-        S->tiles.swap(tiles);
-        S->fused_ids.swap(ids);
-        S->win.swap(win);
-        S->n_producer_rows = prod_rows;
-        S->slab_rows = slab;
-        S->lds_bytes = lds_max;
-        std::fill(fused.begin(), fused.end(), 1);
-      }
-    }
+      if (!(ok && L <= M)) return false;
+      S->inner_nnz = Bp[M];
+      S->tiles.swap(tiles);
+      S->fused_ids.swap(ids);
+      S->win.swap(win);
+      S->n_producer_rows = prod_rows;
+      S->slab_rows = slab;
+      S->lds_bytes = lds_max;
+      S->opts.strip_cols = SW;
+      S->opts.tile_rows = cap;
+      std::fill(fused.begin(), fused.end(), 1);
+      return true;
+    };
+    if (want_wide) windowed = win_wide = build_window(true);
+    if (!windowed && want_window) windowed = build_window(false);
+    S->win_wide = win_wide;
     S->windowed = windowed;
     if (!windowed) S->opts.strip_cols = 0;
 
@@ -484,6 +501,7 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   info->max_tile_producer_rows = s->slab_rows;
   info->lds_bytes = s->lds_bytes;
   info->windowed = s->windowed ? 1 : 0;
+  info->wide_strips = s->win_wide ? 1 : 0;
   info->streamed = s->gemm_stream ? 1 : 0;
   info->ring_rows = s->ring_rows;
   info->strip_cols = s->windowed ? s->opts.strip_cols : 0;

@@ -43,6 +43,7 @@ struct tf_schedule {
   int lds_bytes = 0;          // dynamic LDS of the fused kernel: intermediate slab (+ GEMM staging)
   int lds_bytes_general = 0;  // the same for the kernel that gathers C from HBM (fallback of windowed tiles)
   bool windowed = false;      // tiles stage their window of C in LDS (win holds the windows)
+  bool win_wide = false;      // ... in 64-column strips on the 1024-thread kernel (entries read in place)
   long long inner_nnz = 0;    // stored entries of the inner pattern the windows were built from
   std::vector<int> win;       // [2*n_tiles] first,last+1 row of C read by the tile's producer rows
   int slab_rows = 0;          // max producer rows of any tile

@@ -9,6 +9,7 @@
 // group, so the per-element sequence is acc = fma(value, x[column], acc) exactly as in
 // the reference's AVX2 kernels (fusion/src/SpMM_SpMM_vectorized.cpp:892-936).
 #include <hip/hip_runtime.h>
+#include <type_traits>
 
 #include "tf_internal.h"
 
@@ -273,21 +274,36 @@ template <int G> __device__ __forceinline__ int quad_bcast(int v) {
   return __builtin_amdgcn_mov_dpp(v, G * 0x55, 0xf, 0xf, true);
 }
 
+// acc += (val as held by lane G of the quad) * x: four v_fmac_f32 with the DPP broadcast on the
+// value operand.  (Written out because the compiler folds a broadcast into its consumer only
+// when there is a single one.  The value register is filled by a load; the two idle cycles
+// cover the case of a register copy placed right in front, which a DPP read must not follow
+// directly.)
+template <int G> __device__ __forceinline__ void quad_fma(int val, const fvec<4> &x, fvec<4> &acc) {
+  asm("s_nop 1\n\t"
+      "v_fmac_f32_dpp %0, %4, %5 quad_perm:[%9,%9,%9,%9] row_mask:0xf bank_mask:0xf bound_ctrl:0\n\t"
+      "v_fmac_f32_dpp %1, %4, %6 quad_perm:[%9,%9,%9,%9] row_mask:0xf bank_mask:0xf bound_ctrl:0\n\t"
+      "v_fmac_f32_dpp %2, %4, %7 quad_perm:[%9,%9,%9,%9] row_mask:0xf bank_mask:0xf bound_ctrl:0\n\t"
+      "v_fmac_f32_dpp %3, %4, %8 quad_perm:[%9,%9,%9,%9] row_mask:0xf bank_mask:0xf bound_ctrl:0"
+      : "+v"(acc.v[0]), "+v"(acc.v[1]), "+v"(acc.v[2]), "+v"(acc.v[3])
+      : "v"(val), "v"(x.v[0]), "v"(x.v[1]), "v"(x.v[2]), "v"(x.v[3]), "n"(G));
+}
+
 // Eight staged entries, held four to a lane by lanes GA and GB of the quad: gathers first, then the fmas in order.
 template <int GA, int GB, bool CHECK>
 __device__ __forceinline__ void quad_dot8(const int2 (&e)[4], const char *base, int left, fvec<4> &acc) {
   fvec<4> x[8];
-  int val[8];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    val[j] = quad_bcast<GA>(e[j].y);
-    val[4 + j] = quad_bcast<GB>(e[j].y);
     if (!CHECK || 4 * GA + j < left) x[j] = *reinterpret_cast<const fvec<4> *>(base + quad_bcast<GA>(e[j].x));
     if (!CHECK || 4 * GB + j < left) x[4 + j] = *reinterpret_cast<const fvec<4> *>(base + quad_bcast<GB>(e[j].x));
   }
 #pragma unroll
-  for (int u = 0; u < 8; ++u)
-    if (!CHECK || (u < 4 ? 4 * GA + u : 4 * GB + u - 4) < left) vfma<4>(__int_as_float(val[u]), x[u], acc);
+  for (int j = 0; j < 4; ++j)
+    if (!CHECK || 4 * GA + j < left) quad_fma<GA>(e[j].y, x[j], acc);
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    if (!CHECK || 4 * GB + j < left) quad_fma<GB>(e[j].y, x[4 + j], acc);
 }
 
 // acc += sum_k val[k] * row(off[k]) over staged entries [kb, ke), in order, for a lane group
@@ -398,6 +414,180 @@ __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
       acc = lds_row_dot_quad(ent, rp[r], rp[r + 1] - kWinPad, tbase, glane & 3, acc);
       *reinterpret_cast<fvec<4> *>(dst) = acc;
     }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Windowed fused SpMM-SpMM tile kernel for long matrices: strips of 64 columns, one
+// workgroup of 1024 threads (and up to the whole LDS) per compute unit.  The LDS of this GPU
+// reads 256 bytes a clock when the 16 lanes it serves together touch 64 different banks; a
+// 256-byte strip row read by a 16-lane group does, two 128-byte rows read by two 8-lane groups
+// collide whenever the rows sit on the same half of the banks (every second pair of rows).
+// The price is a row twice as large, so the tile's entries are not staged in LDS: a lane
+// loads its four of every sixteen from the CSR arrays (the rest reach it through its quad),
+// one row ahead of the row it works on.  Same fma sequence per element as the kernels above.
+// ---------------------------------------------------------------------------------
+constexpr int kW64Strip = 64, kW64Block = 1024, kW64Units = 6;
+typedef int int4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+
+struct QuadEntries {  // entries [k, k + 4) of a row as (byte offset into the window, value bits)
+  int2 e[4];
+};
+
+// Entries k .. k+3 of the CSR arrays as (byte offset into the window, value bits); off0 is
+// minus the window's first column times the row size.  EXACT: the caller may be within four
+// entries of the end of the arrays (the last tile of the matrix), so a lane that would read
+// past them loads one entry at a time; elsewhere the four come as one load each.
+template <bool EXACT>
+__device__ __forceinline__ QuadEntries load_quad_entries(const int *__restrict__ ci, const float *__restrict__ cv, int k,
+                                                         int end_k, int nnz, int off0) {
+  QuadEntries r;
+  const int kk = EXACT ? min(k, nnz - 4) : k;  // (nnz >= 4: checked on the host)
+  const int4u c = *reinterpret_cast<const int4u *>(ci + kk);
+  const float4u v = *reinterpret_cast<const float4u *>(cv + kk);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) r.e[j] = make_int2((c[j] << 8) + off0, __float_as_int(v[j]));
+  if constexpr (EXACT) {
+    if (kk != k && k < end_k) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int kj = min(k + j, nnz - 1);
+        r.e[j] = make_int2((ci[kj] << 8) + off0, __float_as_int(cv[kj]));
+      }
+    }
+  }
+  return r;
+}
+static_assert(kW64Strip * 4 == 1 << 8, "row size of the 64-column strip");
+
+// acc += the row's entries [kb, ke) times their window rows; `first` holds this lane's four of
+// the first sixteen.
+template <bool EXACT>
+__device__ __forceinline__ fvec<4> row_dot_quad_regs(const QuadEntries &first, const int *__restrict__ ci,
+                                                     const float *__restrict__ cv, int kb, int ke, int nnz,
+                                                     int off0, const char *base, int q, fvec<4> acc) {
+  const int n = ke - kb;
+  if (n >= 16) {
+    quad_dot8<0, 1, false>(first.e, base, n, acc);
+    quad_dot8<2, 3, false>(first.e, base, n, acc);
+  } else {
+    quad_dot8<0, 1, true>(first.e, base, n, acc);
+    if (n > 8) quad_dot8<2, 3, true>(first.e, base, n, acc);
+  }
+  for (int c = kb + 16; c < ke; c += 16) {
+    const QuadEntries cur = load_quad_entries<EXACT>(ci, cv, c + 4 * q, ke, nnz, off0);
+    const int left = ke - c;
+    if (left >= 16) {
+      quad_dot8<0, 1, false>(cur.e, base, left, acc);
+      quad_dot8<2, 3, false>(cur.e, base, left, acc);
+    } else {
+      quad_dot8<0, 1, true>(cur.e, base, left, acc);
+      if (left > 8) quad_dot8<2, 3, true>(cur.e, base, left, acc);
+    }
+  }
+  return acc;
+}
+
+__device__ __forceinline__ fvec<4> window64_unit(const float *__restrict__ C, int first_row, int N, int c0, int n4,
+                                                 int u) {
+  const int uu = u < n4 ? u : 0;
+  return *reinterpret_cast<const fvec<4> *>(C + (size_t)(first_row + uu / 16) * N + c0 + (uu % 16) * 4);
+}
+
+template <bool ACC>
+__global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
+    const TileDesc *__restrict__ tiles, const int2 *__restrict__ win, int n_tiles, int per_xcd,
+    const int *__restrict__ Bp, const int *__restrict__ Bi, const float *__restrict__ Bx, int nnzB,
+    const float *__restrict__ C, const int *__restrict__ Ap, const int *__restrict__ Ai,
+    const float *__restrict__ Ax, int nnzA, float *__restrict__ D, int N) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int SW = kW64Strip, LPR = SW / 4, G = kW64Block / LPR, ROWB = SW * 4;
+  const int tile = xcd_contiguous(blockIdx.x, per_xcd);
+  if (tile >= n_tiles) return;
+  const TileDesc t = tiles[tile];
+  const int2 w = win[tile];
+  // (a windowed tile's fused rows are its own rows, in order)
+  const int P = t.prod_end - t.prod_begin, R = t.cons_end - t.cons_begin, Wc = w.y - w.x;
+  int *rpB = reinterpret_cast<int *>(smem);                        // row pointers of the producer rows (B)
+  int *rpA = reinterpret_cast<int *>(smem + align16i(4 * (P + 1)));  // ... and of the fused rows (A)
+  float *Cbuf = reinterpret_cast<float *>(reinterpret_cast<unsigned char *>(rpA) + align16i(4 * (R + 1)));
+  float *Tbuf = Cbuf + Wc * SW;
+  const int tid = threadIdx.x, group = tid / LPR, glane = tid % LPR, q = glane & 3;
+  const int n4 = Wc * LPR;
+  fvec<4> pre[kW64Units];
+#pragma unroll
+  for (int j = 0; j < kW64Units; ++j) pre[j] = window64_unit(C, w.x, N, 0, n4, tid + j * kW64Block);
+  for (int i = tid; i <= P; i += kW64Block) rpB[i] = Bp[t.prod_begin + i];
+  for (int i = tid; i <= R; i += kW64Block) rpA[i] = Ap[t.own_begin + i];
+  // column c of B is row c - w.x of the window, column c of A row c - prod_begin of the slab
+  const char *cbase = reinterpret_cast<const char *>(Cbuf) + glane * 16;
+  const char *tbase = reinterpret_cast<const char *>(Tbuf) + glane * 16;
+  const int offB = -w.x * ROWB, offA = -t.prod_begin * ROWB;
+  // (only the last tile of the matrix can come within a load of the end of the arrays)
+  const bool near_end = Bp[t.prod_end] + 16 > nnzB || Ap[t.own_begin + R] + 16 > nnzA;
+  auto products = [&](auto exact_tag, int c0) {
+    constexpr bool EXACT = decltype(exact_tag)::value;
+    QuadEntries ea, eb;
+    auto fetchB = [&](int r) {
+      const int rr = min(r, P - 1);
+      return load_quad_entries<EXACT>(Bi, Bx, rpB[rr] + 4 * q, rpB[rr + 1], nnzB, offB);
+    };
+    auto fetchA = [&](int r) {
+      const int rr = min(r, R - 1);
+      return load_quad_entries<EXACT>(Ai, Ax, rpA[rr] + 4 * q, rpA[rr + 1], nnzA, offA);
+    };
+    lds_barrier();
+    // first product: slab rows 0 .. P-1, a lane group per row, the next row's entries on their way
+    ea = fetchB(group);
+    for (int r = group; r < P; r += 2 * G) {
+      eb = fetchB(r + G);
+      *reinterpret_cast<fvec<4> *>(Tbuf + r * SW + glane * 4) =
+          row_dot_quad_regs<EXACT>(ea, Bi, Bx, rpB[r], rpB[r + 1], nnzB, offB, cbase, q, vzero<4>());
+      if (r + G >= P) break;
+      ea = fetchB(r + 2 * G);
+      *reinterpret_cast<fvec<4> *>(Tbuf + (r + G) * SW + glane * 4) =
+          row_dot_quad_regs<EXACT>(eb, Bi, Bx, rpB[r + G], rpB[r + G + 1], nnzB, offB, cbase, q, vzero<4>());
+    }
+    lds_barrier();
+    // then the fused rows out of the slab
+    if (R > 0) ea = fetchA(group);
+    for (int i = group; i < R; i += 2 * G) {
+      eb = fetchA(i + G);
+      {
+        float *dst = D + (size_t)(t.own_begin + i) * N + c0 + glane * 4;
+        fvec<4> acc = vzero<4>();
+        if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
+        *reinterpret_cast<fvec<4> *>(dst) =
+            row_dot_quad_regs<EXACT>(ea, Ai, Ax, rpA[i], rpA[i + 1], nnzA, offA, tbase, q, acc);
+      }
+      if (i + G >= R) break;
+      ea = fetchA(i + 2 * G);
+      {
+        float *dst = D + (size_t)(t.own_begin + i + G) * N + c0 + glane * 4;
+        fvec<4> acc = vzero<4>();
+        if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
+        *reinterpret_cast<fvec<4> *>(dst) =
+            row_dot_quad_regs<EXACT>(eb, Ai, Ax, rpA[i + G], rpA[i + G + 1], nnzA, offA, tbase, q, acc);
+      }
+    }
+  };
+  for (int c0 = 0; c0 < N; c0 += SW) {
+    lds_barrier();  // previous strip fully consumed (and, first time, row pointers visible)
+    {
+      fvec<4> *cb = reinterpret_cast<fvec<4> *>(Cbuf);
+#pragma unroll
+      for (int j = 0; j < kW64Units; ++j)
+        if (tid + j * kW64Block < n4) cb[tid + j * kW64Block] = pre[j];
+      for (int u = tid + kW64Units * kW64Block; u < n4; u += kW64Block)  // windows beyond the prefetch capacity
+        cb[u] = window64_unit(C, w.x, N, c0, n4, u);
+    }
+    if (c0 + SW < N) {
+#pragma unroll
+      for (int j = 0; j < kW64Units; ++j) pre[j] = window64_unit(C, w.x, N, c0 + SW, n4, tid + j * kW64Block);
+    }
+    if (near_end) products(std::true_type{}, c0);
+    else products(std::false_type{}, c0);
   }
 }
 
@@ -1327,6 +1517,25 @@ hipError_t launch_fused_spmm_spmm_window(const TileDesc *tiles, const int *win, 
     if (accumulate) { CALLW(64, true); } else { CALLW(64, false); }
   }
 #undef CALLW
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+hipError_t launch_fused_spmm_spmm_window64(const TileDesc *tiles, const int *win, int n_tiles, const int *Bp,
+                                           const int *Bi, const float *Bx, int nnzB, const float *C, const int *Ap,
+                                           const int *Ai, const float *Ax, int nnzA, float *D, int N, int lds_bytes,
+                                           int accumulate, hipStream_t st) {
+  if (n_tiles <= 0) return hipSuccess;
+  if (N % kW64Strip != 0 || nnzA < 4 || nnzB < 4) return hipErrorInvalidValue;
+  const int per = per_xcd_of(n_tiles);
+  const int2 *w2 = reinterpret_cast<const int2 *>(win);
+  hipError_t err;
+#define CALL64(ACC_)                                                                                    \
+  err = allow_lds(fused_spmm_spmm_window64_kernel<ACC_>, lds_bytes);                                    \
+  if (err == hipSuccess)                                                                                \
+    hipLaunchKernelGGL((fused_spmm_spmm_window64_kernel<ACC_>), dim3(grid_of(n_tiles)), dim3(kW64Block), \
+                       lds_bytes, st, tiles, w2, n_tiles, per, Bp, Bi, Bx, nnzB, C, Ap, Ai, Ax, nnzA, D, N)
+  if (accumulate) { CALL64(true); } else { CALL64(false); }
+#undef CALL64
   return err != hipSuccess ? err : hipGetLastError();
 }
 
