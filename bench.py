@@ -111,6 +111,10 @@ def main():
     ap.add_argument("--op", default="spmm_spmm", choices=["spmm_spmm", "gemm_spmm"])
     ap.add_argument("--N", type=int, default=64)
     ap.add_argument("--K", type=int, default=64)
+    ap.add_argument("--scramble", action="store_true",
+                    help="permute the rows and columns of the (square) matrix at random first")
+    ap.add_argument("--rcm", action="store_true",
+                    help="reorder the matrix with tf_reorder_rcm / tf_permute_csr before inspecting it (after --scramble)")
     ap.add_argument("--unfused", action="store_true",
                     help="GeMM-SpMM as two launches (tf_gemm, tf_spmm) with the intermediate in HBM, for comparison")
     ap.add_argument("--host-buffers", action="store_true",
@@ -142,6 +146,31 @@ def main():
                    K=args.K if gemm else 0, N=args.N, name=f"file {os.path.basename(args.matrix)} {args.op} N={args.N}" + (f" K={args.K}" if gemm else ""))
     else:
         cfg = w.make_config(args.config)
+    reorder_s = None
+    if args.scramble or args.rcm:  # same product on a renumbered graph: A' = A[p,:][:,p], dense row operands follow
+        A0 = cfg["A"]
+        if A0.shape[0] != A0.shape[1]:
+            sys.exit("bench.py --scramble/--rcm: the matrix must be square")
+        same_b = cfg["B"] is A0
+        rows_follow = ["B"] if cfg["op"] == "gemm_spmm" else ["C"]
+        if args.scramble:
+            import numpy as np
+            p = np.random.default_rng(5).permutation(A0.shape[0]).astype("int32")
+            A0 = tf.permute_csr(A0, p)
+            for k in rows_follow:
+                cfg[k] = cfg[k][p]
+            cfg["name"] += ", scrambled"
+        if args.rcm:
+            t0 = time.perf_counter()
+            p = tf.reorder_rcm(A0)
+            A0 = tf.permute_csr(A0, p)
+            reorder_s = time.perf_counter() - t0
+            for k in rows_follow:
+                cfg[k] = cfg[k][p]
+            cfg["name"] += ", RCM"
+        cfg["A"] = A0
+        if same_b:
+            cfg["B"] = A0
     A, N, K = cfg["A"], cfg["N"], cfg["K"]
     op = tf.OP_GEMM_SPMM if cfg["op"] == "gemm_spmm" else tf.OP_SPMM_SPMM
 
@@ -210,7 +239,7 @@ def main():
                    "lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "wide_strips": bool(info["wide_strips"]), "streamed": bool(info["streamed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
                    "remainder_rows": info["n_remainder_rows"], "recomputed_rows": info["n_producer_rows"] - A.shape[1],
                    "writeback_rows": info["n_writeback_rows"], "kernels_per_step": n_kernels,
-                   "inspector_s": round(inspect_s, 4), "rel_err_vs_f64": check, "device": dev["arch"]},
+                   "inspector_s": round(inspect_s, 4), **({"reorder_s": round(reorder_s, 4)} if reorder_s is not None else {}), "rel_err_vs_f64": check, "device": dev["arch"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes": int(alg_bytes), "kernel_ms": round(dev_ms, 5),

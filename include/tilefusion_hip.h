@@ -115,6 +115,20 @@ tf_status tf_read_matrix(const char *path, int *M, int *N, int *nnz, int **Ap, i
 tf_status tf_read_dense(const char *path, int *M, int *N, float **data);
 void tf_host_free(void *p);
 
+/* ---- reordering ------------------------------------------------------------------ */
+
+/* Reverse Cuthill-McKee ordering of a square matrix' pattern, symmetrised (A + A^T): rows
+ * that depend on each other end up close together, so that tiles can fuse them.  The
+ * reference reorders its inputs offline with scipy's reverse_cuthill_mckee
+ * (fusion/scripts/reorder_graphs.py:3,21).  perm[new index] = old index, M entries.  Every
+ * component starts from a pseudo-peripheral node; components are taken in order of their
+ * smallest-degree node.  Host-only. */
+tf_status tf_reorder_rcm(int M, const int *Ap, const int *Ai, int *perm);
+/* B = A[perm,:][:,perm] (reorder_graphs.py:22), columns sorted; the arrays are released with
+ * tf_host_free.  With C' = C[perm,:], D' = B (B C') is D[perm,:] of D = A (A C). */
+tf_status tf_permute_csr(int M, const int *Ap, const int *Ai, const float *Ax, const int *perm, int **Bp, int **Bi,
+                         float **Bx);
+
 /* ---- inspector ---------------------------------------------------------------- */
 
 enum { TF_OP_SPMM_SPMM = 0, TF_OP_GEMM_SPMM = 1 };

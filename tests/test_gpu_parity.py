@@ -299,6 +299,38 @@ def test_spmm_spmm_windowed_schedule_with_other_inner_matrix(gpu, tf, orc):
     assert e.value.status == -4
 
 
+def test_spmm_spmm_after_rcm_reordering(gpu, tf, orc):
+    """A band whose rows arrive in random order fuses nothing; after tf_reorder_rcm /
+    tf_permute_csr (the reference's offline step, scripts/reorder_graphs.py:21-22) every row
+    fuses, and D'[new] = D[perm[new]].  Reordering changes the order of a row's entries, so
+    the comparison with the oracle on the original matrix is to 1e-5, not bit for bit."""
+    say("spmm_spmm after RCM")
+    M, N = 40000, 64
+    A = tf.workloads.banded_random(M, 32, 16, seed=47)
+    p0 = np.random.default_rng(48).permutation(M)
+    S = sp.csr_matrix(A[p0, :][:, p0])
+    Cd = tf.workloads.uniform((M, N), 49)
+    want = oracle_spmm_spmm(orc, S, S, Cd)
+    Sh = tf.CsrMatrix.from_scipy(S)
+    sched = tf.inspector(Sh, 1, op=tf.OP_SPMM_SPMM, N=N, inner=Sh)
+    assert sched.info()["n_fused_rows"] < 0.05 * M
+    D = tf.DenseMatrix(M, N)
+    tf.spmm_spmm(Sh, Sh, tf.DenseMatrix.from_numpy(Cd), D, sched)
+    assert np.array_equal(D.to_numpy(), want)  # unfused, CSR order: still the reference's bits
+    perm = tf.reorder_rcm(S)
+    R = tf.permute_csr(S, perm)
+    Rh = tf.CsrMatrix.from_scipy(R)
+    sched = tf.inspector(Rh, 1, op=tf.OP_SPMM_SPMM, N=N, inner=Rh, compute_units=256)
+    sched.validate()
+    info = sched.info()
+    assert info["n_fused_rows"] == M and info["windowed"] == 1
+    D = tf.DenseMatrix(M, N)
+    tf.spmm_spmm(Rh, Rh, tf.DenseMatrix.from_numpy(np.ascontiguousarray(Cd[perm])), D, sched)
+    got = np.empty((M, N), np.float32)
+    got[perm] = D.to_numpy()
+    assert orc.rel_err(got, want) <= 1e-5
+
+
 # ---- GeMM-SpMM ----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("K,N", [(64, 64), (128, 128), (256, 128), (8, 32), (72, 96), (40, 256), (512, 64)])

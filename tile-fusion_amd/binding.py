@@ -90,6 +90,8 @@ SIGNATURES = {
     "tf_read_matrix": (C.c_int, [C.c_char_p, _PI, _PI, _PI, C.POINTER(_PI), C.POINTER(_PI), C.POINTER(_PF)]),
     "tf_read_dense": (C.c_int, [C.c_char_p, _PI, _PI, C.POINTER(_PF)]),
     "tf_host_free": (None, [_VP]),
+    "tf_reorder_rcm": (C.c_int, [C.c_int, _PI, _PI, _PI]),
+    "tf_permute_csr": (C.c_int, [C.c_int, _PI, _PI, _PF, _PI, C.POINTER(_PI), C.POINTER(_PI), C.POINTER(_PF)]),
     "tf_inspect": (C.c_int, [C.c_int, C.c_int, _PI, _PI, C.POINTER(InspectOpts), C.POINTER(_VP)]),
     "tf_schedule_free": (None, [_VP]),
     "tf_schedule_get_info": (C.c_int, [_VP, C.POINTER(ScheduleInfo)]),
@@ -365,3 +367,45 @@ def read_dense(path):
     finally:
         lib().tf_host_free(C.cast(d, _VP))
     return out.reshape(M.value, N.value)
+
+
+def _as_i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def reorder_rcm(A):
+    """Reverse Cuthill-McKee permutation of a square scipy CSR matrix (perm[new] = old), the
+    library's counterpart of scipy's reverse_cuthill_mckee in the reference's
+    scripts/reorder_graphs.py:21."""
+    import scipy.sparse as sp
+    A = sp.csr_matrix(A)
+    if A.shape[0] != A.shape[1]:
+        raise ValueError("reorder_rcm: the matrix must be square")
+    M = A.shape[0]
+    ap, ai = _as_i32(A.indptr), _as_i32(A.indices)
+    perm = np.empty(M, np.int32)
+    _check(lib().tf_reorder_rcm(M, ap.ctypes.data_as(_PI), ai.ctypes.data_as(_PI), perm.ctypes.data_as(_PI)))
+    return perm
+
+
+def permute_csr(A, perm):
+    """A[perm,:][:,perm] (reorder_graphs.py:22) as a scipy CSR matrix with sorted columns."""
+    import scipy.sparse as sp
+    A = sp.csr_matrix(A)
+    M = A.shape[0]
+    ap, ai, ax = _as_i32(A.indptr), _as_i32(A.indices), np.ascontiguousarray(A.data, dtype=np.float32)
+    pm = _as_i32(perm)
+    if pm.shape != (M,) or A.shape[0] != A.shape[1]:
+        raise ValueError("permute_csr: a square matrix and one index per row are needed")
+    bp, bi, bx = _PI(), _PI(), _PF()
+    _check(lib().tf_permute_csr(M, ap.ctypes.data_as(_PI), ai.ctypes.data_as(_PI), ax.ctypes.data_as(_PF),
+                                pm.ctypes.data_as(_PI), C.byref(bp), C.byref(bi), C.byref(bx)))
+    try:
+        indptr = np.ctypeslib.as_array(bp, shape=(M + 1,)).copy()
+        n = int(indptr[M])
+        indices = np.ctypeslib.as_array(bi, shape=(max(n, 1),))[:n].copy()
+        data = np.ctypeslib.as_array(bx, shape=(max(n, 1),))[:n].copy()
+    finally:
+        for q in (bp, bi, bx):
+            lib().tf_host_free(C.cast(q, _VP))
+    return sp.csr_matrix((data, indices, indptr), shape=A.shape)
