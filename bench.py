@@ -154,7 +154,6 @@ def main():
         same_b = cfg["B"] is A0
         rows_follow = ["B"] if cfg["op"] == "gemm_spmm" else ["C"]
         if args.scramble:
-            import numpy as np
             p = np.random.default_rng(5).permutation(A0.shape[0]).astype("int32")
             A0 = tf.permute_csr(A0, p)
             for k in rows_follow:

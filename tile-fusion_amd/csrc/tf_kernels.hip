@@ -433,6 +433,7 @@ typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
 
 struct QuadEntries {  // entries [k, k + 4) of a row as (byte offset into the window, value bits)
   int2 e[4];
+  int kb, ke;  // the row's entry range (kept by the row loops next to the entries fetched ahead)
 };
 
 // Entries k .. k+3 of the CSR arrays as (byte offset into the window, value bits); off0 is
@@ -444,8 +445,9 @@ __device__ __forceinline__ QuadEntries load_quad_entries(const int *__restrict__
                                                          int end_k, int nnz, int off0) {
   QuadEntries r;
   const int kk = EXACT ? min(k, nnz - 4) : k;  // (nnz >= 4: checked on the host)
-  const int4u c = *reinterpret_cast<const int4u *>(ci + kk);
-  const float4u v = *reinterpret_cast<const float4u *>(cv + kk);
+  const unsigned byte = (unsigned)kk * 4u;    // (one 32-bit offset from both array bases)
+  const int4u c = *reinterpret_cast<const int4u *>(reinterpret_cast<const char *>(ci) + byte);
+  const float4u v = *reinterpret_cast<const float4u *>(reinterpret_cast<const char *>(cv) + byte);
 #pragma unroll
   for (int j = 0; j < 4; ++j) r.e[j] = make_int2((c[j] << 8) + off0, __float_as_int(v[j]));
   if constexpr (EXACT) {
@@ -531,11 +533,17 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
     QuadEntries ea, eb;
     auto fetchB = [&](int r) {
       const int rr = min(r, P - 1);
-      return load_quad_entries<EXACT>(Bi, Bx, rpB[rr] + 4 * q, rpB[rr + 1], nnzB, offB);
+      const int kb = rpB[rr], ke = rpB[rr + 1];
+      QuadEntries e = load_quad_entries<EXACT>(Bi, Bx, kb + 4 * q, ke, nnzB, offB);
+      e.kb = kb; e.ke = ke;
+      return e;
     };
     auto fetchA = [&](int r) {
       const int rr = min(r, R - 1);
-      return load_quad_entries<EXACT>(Ai, Ax, rpA[rr] + 4 * q, rpA[rr + 1], nnzA, offA);
+      const int kb = rpA[rr], ke = rpA[rr + 1];
+      QuadEntries e = load_quad_entries<EXACT>(Ai, Ax, kb + 4 * q, ke, nnzA, offA);
+      e.kb = kb; e.ke = ke;
+      return e;
     };
     lds_barrier();
     // first product: slab rows 0 .. P-1, a lane group per row, the next row's entries on their way
@@ -543,32 +551,34 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
     for (int r = group; r < P; r += 2 * G) {
       eb = fetchB(r + G);
       *reinterpret_cast<fvec<4> *>(Tbuf + r * SW + glane * 4) =
-          row_dot_quad_regs<EXACT>(ea, Bi, Bx, rpB[r], rpB[r + 1], nnzB, offB, cbase, q, vzero<4>());
+          row_dot_quad_regs<EXACT>(ea, Bi, Bx, ea.kb, ea.ke, nnzB, offB, cbase, q, vzero<4>());
       if (r + G >= P) break;
       ea = fetchB(r + 2 * G);
       *reinterpret_cast<fvec<4> *>(Tbuf + (r + G) * SW + glane * 4) =
-          row_dot_quad_regs<EXACT>(eb, Bi, Bx, rpB[r + G], rpB[r + G + 1], nnzB, offB, cbase, q, vzero<4>());
+          row_dot_quad_regs<EXACT>(eb, Bi, Bx, eb.kb, eb.ke, nnzB, offB, cbase, q, vzero<4>());
     }
     lds_barrier();
     // then the fused rows out of the slab
     if (R > 0) ea = fetchA(group);
+    float *dst = D + (size_t)(t.own_begin + group) * N + c0 + glane * 4;
+    const size_t round_stride = (size_t)G * N;
     for (int i = group; i < R; i += 2 * G) {
       eb = fetchA(i + G);
       {
-        float *dst = D + (size_t)(t.own_begin + i) * N + c0 + glane * 4;
         fvec<4> acc = vzero<4>();
         if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
         *reinterpret_cast<fvec<4> *>(dst) =
-            row_dot_quad_regs<EXACT>(ea, Ai, Ax, rpA[i], rpA[i + 1], nnzA, offA, tbase, q, acc);
+            row_dot_quad_regs<EXACT>(ea, Ai, Ax, ea.kb, ea.ke, nnzA, offA, tbase, q, acc);
+        dst += round_stride;
       }
       if (i + G >= R) break;
       ea = fetchA(i + 2 * G);
       {
-        float *dst = D + (size_t)(t.own_begin + i + G) * N + c0 + glane * 4;
         fvec<4> acc = vzero<4>();
         if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
         *reinterpret_cast<fvec<4> *>(dst) =
-            row_dot_quad_regs<EXACT>(eb, Ai, Ax, rpA[i + G], rpA[i + G + 1], nnzA, offA, tbase, q, acc);
+            row_dot_quad_regs<EXACT>(eb, Ai, Ax, eb.kb, eb.ke, nnzA, offA, tbase, q, acc);
+        dst += round_stride;
       }
     }
   };
