@@ -127,7 +127,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-              "(the path shards by row blocks of A, see DESIGN.md)", file=sys.stderr)
+              "(more GPUs would each take a block of rows of A and D; no such path is built)", file=sys.stderr)
         sys.exit(2)
 
     tf = importlib.import_module("tile-fusion_amd")
