@@ -106,7 +106,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   const bool want_window = have_inner && o.N % o.strip_cols == 0 && o.wide_strips <= 0;
   // (one tile per compute unit: a matrix with fewer than 128 rows per compute unit is better
   // served by more and smaller tiles)
-  const bool want_wide = have_inner && o.N % 64 == 0 && o.inner_Ap[M] >= 4 && nnz >= 4 &&
+  // (the kernel addresses the CSR arrays with 32-bit byte offsets and loads four entries at a time)
+  const bool want_wide = have_inner && o.N % 64 == 0 && o.inner_Ap[M] >= 4 && nnz >= 4 && o.inner_Ap[M] < (1 << 30) && nnz < (1 << 30) &&
                          (o.wide_strips > 0 || (o.wide_strips == 0 && user->strip_cols <= 0 && user->lds_budget_bytes <= 0 &&
                                               user->tile_rows <= 0 && M >= 128LL * o.compute_units));
   int r_cap = o.tile_rows > 0 ? o.tile_rows : ceil_div(M, 2 * o.compute_units);

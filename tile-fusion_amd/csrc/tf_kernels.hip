@@ -1535,7 +1535,7 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *tiles, const int *win
                                            const int *Ai, const float *Ax, int nnzA, float *D, int N, int lds_bytes,
                                            int accumulate, hipStream_t st) {
   if (n_tiles <= 0) return hipSuccess;
-  if (N % kW64Strip != 0 || nnzA < 4 || nnzB < 4) return hipErrorInvalidValue;
+  if (N % kW64Strip != 0 || nnzA < 4 || nnzB < 4 || nnzA >= (1 << 30) || nnzB >= (1 << 30)) return hipErrorInvalidValue;
   const int per = per_xcd_of(n_tiles);
   const int2 *w2 = reinterpret_cast<const int2 *>(win);
   hipError_t err;
