@@ -106,6 +106,8 @@ def main():
                     help="windowed tiles: 1 = the 64-column, 1024-thread kernel, -1 = the lane-group kernel, 0 = library's choice")
     ap.add_argument("--xcd-chunk", type=int, default=0, help="rows per XCD turn of the row kernels (-1 contiguous)")
     ap.add_argument("--long-row", type=int, default=0, help="rows with more entries than this are chunked")
+    ap.add_argument("--long-part", type=int, default=0, choices=[-1, 0, 1],
+                    help="long rows: 1 = regrouped by the XCD partition of their columns, -1 = chunks of consecutive entries, 0 = library's choice")
     ap.add_argument("--matrix", default=None, help="run on a .mtx / .smtx file instead of a synthetic configuration "
                     "(square; symmetric files are expanded), with --op, --N and --K")
     ap.add_argument("--op", default="spmm_spmm", choices=["spmm_spmm", "gemm_spmm"])
@@ -178,7 +180,7 @@ def main():
     inner = Ah if (op == tf.OP_SPMM_SPMM and cfg["B"] is A and not args.no_window) else None
     S = tf.inspector(Ah, 1, op=op, N=N, K=K, lds_budget_bytes=args.lds, tile_rows=args.tile_rows,
                      max_redundancy=args.max_redundancy, inner=inner, strip_cols=args.strip, wide_strips=args.wide,
-                     long_row_nnz=args.long_row, xcd_chunk_rows=args.xcd_chunk)
+                     long_row_nnz=args.long_row, xcd_chunk_rows=args.xcd_chunk, long_row_partition=args.long_part)
     inspect_s = time.perf_counter() - t0
     S.validate()
     info = S.info()

@@ -179,6 +179,11 @@ typedef struct {
                             LDS, two workgroups per compute unit; 0 = the first for matrices of
                             128 rows per compute unit or more when strip_cols, tile_rows and
                             lds_budget_bytes are left at 0, else the second                    */
+  int long_row_partition; /* long remainder rows (more than long_row_nnz entries): 1 = regroup their entries
+                            by column so that each XCD gathers from its own part of the most-read
+                            intermediate rows, which then stays in its L2 (power-law graphs); -1 = cut
+                            them into chunks of consecutive entries; 0 = the first when the long rows
+                            hold a million entries or more and the intermediate exceeds 64 MB      */
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -203,7 +208,7 @@ typedef struct {
   int n_fused_rows;      /* second-op rows served from LDS                          */
   int n_remainder_rows;  /* second-op rows served from the intermediate in HBM      */
   int n_long_rows;       /* of those, rows split into chunks                        */
-  int n_long_chunks;
+  int n_long_chunks;     /* chunks of consecutive entries, or column-partitioned segments */
   int n_producer_rows;   /* sum over tiles of rows computed (>= M with recomputation) */
   int n_writeback_rows;  /* intermediate rows that are written to HBM               */
   int max_tile_producer_rows;
@@ -214,6 +219,7 @@ typedef struct {
   int streamed;          /* 1 when GeMM-SpMM tiles are long runs streamed through an LDS ring */
   int ring_rows;         /* intermediate rows the ring holds, else 0                 */
   int wide_strips;       /* 1 when windowed tiles run on the 64-column, 1024-thread kernel */
+  int long_row_hot_cols; /* intermediate rows kept in the XCDs' L2 partitions for the long rows, else 0 */
   long long fused_nnz;   /* stored entries of A in fused rows (getFusedNnzNum)      */
   long long workspace_bytes; /* device memory the executor keeps (intermediate + partials) */
 } tf_schedule_info;

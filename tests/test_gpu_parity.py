@@ -388,6 +388,38 @@ def test_gemm_spmm_configs(gpu, tf, orc, idx, scale):
         assert info["n_long_rows"] >= 1
 
 
+@pytest.mark.parametrize("N", [128, 64, 32])
+def test_long_rows_by_column_partition(gpu, tf, orc, N):
+    """Power-law graph, long rows regrouped by column partition (each XCD gathers from its own
+    part of the most-read intermediate rows): GeMM-SpMM and SpMM-SpMM against the oracle, and
+    D +=.  A long row's segments are added in a fixed order that is not CSR order: 1e-4."""
+    say(f"long rows by column partition N={N}")
+    cfg = tf.workloads.make_config(4, 2.0 ** -6)
+    A = cfg["A"]
+    M = A.shape[0]
+    rng = np.random.default_rng(90 + N)
+    B = rng.uniform(-1, 1, (M, 64)).astype(np.float32)
+    Cd = rng.uniform(-1, 1, (64, N)).astype(np.float32)
+    want, _ = orc.gemm_spmm(A, B, Cd, orc.unfused_schedule(M), nthreads=8)
+    got, info = run_gemm_spmm(tf, A, B, Cd, long_row_partition=1)
+    assert info["long_row_hot_cols"] > 0 and info["n_long_rows"] > 0
+    assert orc.rel_err(got, want) <= TOL
+    again, _ = run_gemm_spmm(tf, A, B, Cd, long_row_partition=1)
+    assert np.array_equal(got, again)  # fixed summation order
+    D0 = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    acc, _ = run_gemm_spmm(tf, A, B, Cd, accumulate=True, D0=D0, long_row_partition=1)
+    assert orc.rel_err(acc, D0.astype(np.float64) + want) <= TOL
+    C2 = rng.uniform(-1, 1, (M, N)).astype(np.float32)
+    want2 = oracle_spmm_spmm(orc, A, A, C2)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N, long_row_partition=1)
+    S.validate()
+    D = tf.DenseMatrix(M, N)
+    D.fill(float("nan"))
+    tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(C2), D, S)
+    assert orc.rel_err(D.to_numpy(), want2) <= TOL
+
+
 def test_gemm_spmm_reductions_and_accumulate(gpu, tf, orc):
     say("gemm_spmm reductions")
     M, K, N = 1000, 64, 64

@@ -236,6 +236,33 @@ def test_wide_strip_tiles(tf):
     assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah, compute_units=64, wide_strips=1).info()["wide_strips"] == 1
 
 
+def test_long_rows_by_column_partition(tf):
+    """long_row_partition: the long rows' entries regrouped by the XCD partition of their column
+    (the most-read intermediate rows, an L2's worth per XCD) into segments of at most 64;
+    every entry once, CSR order inside a segment, a column read through one partition only --
+    checked by the library's validator and recounted here from the info."""
+    cfg = tf.workloads.make_config(4, 2.0 ** -5)
+    A = cfg["A"]
+    Ah = tf.CsrMatrix.from_scipy(A)
+    base = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128)
+    assert base.info()["long_row_hot_cols"] == 0 and base.info()["n_long_rows"] > 0
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1)
+    S.validate()
+    info = S.info()
+    assert info["n_long_rows"] == base.info()["n_long_rows"]
+    rl = np.diff(A.indptr)
+    long_nnz = int(rl[rl > 32].sum())
+    assert 0 < info["long_row_hot_cols"] <= 8 * (4 << 20) // (128 * 4)
+    # at least one segment per 64 entries, and the eight hot lists are padded to whole workgroups
+    assert info["n_long_chunks"] >= long_nnz // 64 and info["n_long_chunks"] % 1 == 0
+    assert info["workspace_bytes"] >= info["n_long_chunks"] * 128 * 4 + long_nnz * 4
+    assert tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=-1).info()["long_row_hot_cols"] == 0
+    # SpMM-SpMM takes the same remainder path
+    S2 = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, long_row_partition=1)
+    S2.validate()
+    assert S2.info()["long_row_hot_cols"] > 0
+
+
 def test_xcd_chunk_is_the_callers_choice(tf):
     A = tf.workloads.laplacian_3d(40)
     Ah = tf.CsrMatrix.from_scipy(A)

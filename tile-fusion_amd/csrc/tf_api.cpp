@@ -39,8 +39,11 @@ struct DeviceSchedule {
   int *fused_rec = nullptr;
   LongChunk *long_chunks = nullptr;
   LongRow *long_rows = nullptr;
+  LongRow *seg_groups = nullptr;
   float *inter = nullptr;    // M x N intermediate, only if some tile writes back
-  float *partial = nullptr;  // n_long_chunks x N
+  float *partial = nullptr;  // n_long_chunks (or segments) x N
+  int *seg_ptr = nullptr, *ent_src = nullptr, *ent_pos = nullptr, *seg_col = nullptr, *lrow_seg = nullptr;  // column-partitioned long rows
+  float *seg_val = nullptr;  // A's values in the order of the regrouped entries
   float *Bpad = nullptr;     // M x K' and K' x N copies of B and C, zero-padded, when K is not a multiple of 8
   float *Cpad = nullptr;
 };
@@ -57,6 +60,9 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *, const int *, int, c
                                            const float *, int, float *, int, int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
                             float *, int, int, int, hipStream_t);
+hipError_t launch_long_rows_partitioned(const int *, const int *, const int *, const int *, float *, int, int, int, const LongRow *, int, const LongRow *, int,
+                                        const int *, const float *, const float *, float *, float *, int, int,
+                                        hipStream_t);
 hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const int *, const float *,
                             const float *, float *, float *, int, int, hipStream_t);
 hipError_t launch_fused_gemm_spmm(const TileDesc *, int, const int *, const float *, const float *,
@@ -101,7 +107,8 @@ int default_compute_units() {
 void release_device_schedule(DeviceSchedule *d) {
   if (!d) return;
   (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows); (void)hipFree(d->plain_rows);
-  (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows);
+  (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows); (void)hipFree(d->seg_groups);
+  (void)hipFree(d->seg_ptr); (void)hipFree(d->ent_src); (void)hipFree(d->ent_pos); (void)hipFree(d->seg_col); (void)hipFree(d->lrow_seg); (void)hipFree(d->seg_val);
   (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
   (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad);
   delete d;
@@ -139,6 +146,20 @@ static tf_status ensure_device(tf_schedule *s) {
   if (!rc) rc = upload_vec(s->fused_rec, &d->fused_rec);
   if (!rc) rc = upload_vec(s->long_chunks, &d->long_chunks);
   if (!rc) rc = upload_vec(s->long_rows, &d->long_rows);
+  if (!rc && s->long_part) {
+    rc = upload_vec(s->seg_ptr, &d->seg_ptr);
+    if (!rc) rc = upload_vec(s->ent_src, &d->ent_src);
+    if (!rc) rc = upload_vec(s->ent_pos, &d->ent_pos);
+    if (!rc) rc = upload_vec(s->seg_col, &d->seg_col);
+    if (!rc) rc = upload_vec(s->lrow_seg, &d->lrow_seg);
+    if (!rc) rc = upload_vec(s->seg_groups, &d->seg_groups);
+    if (!rc) {
+      hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->seg_val), std::max<size_t>(s->seg_src.size(), 1) * sizeof(float));
+      if (e == hipSuccess)
+        e = hipMalloc(reinterpret_cast<void **>(&d->partial), (s->seg_ptr.size() - 1 + s->seg_groups.size()) * (size_t)s->opts.N * sizeof(float));
+      if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(long-row segments)");
+    }
+  }
   if (!rc && s->n_writeback_rows > 0) {
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->inter), (size_t)s->M * s->opts.N * sizeof(float));
     if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(intermediate)");
@@ -168,6 +189,11 @@ static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int
     TF_HIP(launch_spmm_rows(s->rem_identity ? nullptr : d->rem_rows, (int)s->rem_rows.size(), A->p, A->i,
                             A->x, d->inter, D->d, N, accumulate, s->xcd_chunk_rows, st));
   }
+  if (s->long_part)
+    TF_HIP(launch_long_rows_partitioned(d->seg_ptr, d->seg_col, d->ent_src, d->ent_pos, d->seg_val, (int)s->seg_src.size(),
+                                        8 * s->seg_per_xcd, (int)s->seg_ptr.size() - 1, d->seg_groups, (int)s->seg_groups.size(), d->long_rows,
+                                        (int)s->long_rows.size(), d->lrow_seg, A->x, d->inter, d->partial, D->d, N,
+                                        accumulate, st));
   if (!s->long_chunks.empty())
     TF_HIP(launch_long_rows(d->long_chunks, (int)s->long_chunks.size(), d->long_rows,
                             (int)s->long_rows.size(), A->i, A->x, d->inter, d->partial, D->d, N,

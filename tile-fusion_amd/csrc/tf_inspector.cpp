@@ -10,6 +10,7 @@
 // so that boundary rows still fuse, and the remainder is cut into wavefront-sized
 // row groups plus chunks of very long rows.
 #include <algorithm>
+#include <numeric>
 #include <climits>
 #include <cstdio>
 #include <cstring>
@@ -384,6 +385,121 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         S->rem_rows.push_back(i);
       }
     }
+    // Long rows by column.  On a power-law graph a few intermediate rows take most of the reads
+    // of the long rows, but not few enough to survive in an L2 next to the stream of all the
+    // others.  Each of the 8 XCDs has its own L2: the most-read rows are dealt to 8 partitions
+    // that fit one L2 each, every long row's entries are regrouped by partition (CSR order kept
+    // inside a group), and a group is worked on, like a short row, by the XCD of its partition;
+    // entries outside all partitions ("cold") go to all XCDs as before.  Groups are cut into
+    // segments of at most 64 entries; a row's segments are added up in a fixed order.
+    {
+      long long long_nnz = 0;
+      for (const auto &lr : S->long_rows) long_nnz += Ap[lr.row + 1] - Ap[lr.row];
+      const bool want = o.long_row_partition > 0 ||
+                        (o.long_row_partition == 0 && long_nnz >= (1 << 20) && (long long)M * o.N * 4 > (64LL << 20));
+      const int part_rows = std::max(64, (4 << 20) / (o.N * 4));  // an L2's 4 MB (measured: a gather set of that size still stays resident)
+      if (want && !S->long_rows.empty() && long_nnz < INT_MAX) {
+        constexpr int kParts = 8, kSegMax = 64, kPad = 256, kMinGroup = 4;
+        std::vector<int> reads(M, 0);
+        for (const auto &lr : S->long_rows)
+          for (int k = Ap[lr.row]; k < Ap[lr.row + 1]; ++k) ++reads[Ai[k]];
+        std::vector<int> hot;
+        for (int c = 0; c < M; ++c)
+          if (reads[c] >= 2) hot.push_back(c);
+        const size_t n_hot = std::min(hot.size(), (size_t)kParts * part_rows);
+        std::partial_sort(hot.begin(), hot.begin() + n_hot, hot.end(),
+                          [&](int a, int b) { return reads[a] != reads[b] ? reads[a] > reads[b] : a < b; });
+        hot.resize(n_hot);
+        std::vector<signed char> part(M, -1);
+        for (size_t h = 0; h < n_hot; ++h) {  // dealt in turn, snake-wise, so that the partitions' read counts match
+          const int lap = (int)(h / kParts), pos = (int)(h % kParts);
+          part[hot[h]] = (signed char)((lap & 1) ? kParts - 1 - pos : pos);
+        }
+        // segments per class (0..7 hot, 8 cold), in row order
+        std::vector<std::vector<int>> cls_ptr(kParts + 1), cls_src(kParts + 1);
+        std::vector<std::vector<std::pair<int, int>>> row_segs(S->long_rows.size());  // (class, index in class)
+        for (auto &v : cls_ptr) v.push_back(0);
+        std::vector<int> bucket[kParts + 1];
+        for (size_t r = 0; r < S->long_rows.size(); ++r) {
+          const int i = S->long_rows[r].row;
+          for (auto &b : bucket) b.clear();
+          for (int k = Ap[i]; k < Ap[i + 1]; ++k) bucket[part[Ai[k]] < 0 ? kParts : part[Ai[k]]].push_back(k);
+          // a handful of entries does not pay for a partial sum of its own: such groups join the cold one
+          bool moved = false;
+          for (int c = 0; c < kParts; ++c)
+            if (!bucket[c].empty() && (int)bucket[c].size() < kMinGroup) {
+              bucket[kParts].insert(bucket[kParts].end(), bucket[c].begin(), bucket[c].end());
+              bucket[c].clear();
+              moved = true;
+            }
+          if (moved) std::sort(bucket[kParts].begin(), bucket[kParts].end());
+          for (int c = 0; c <= kParts; ++c)
+            for (size_t b0 = 0; b0 < bucket[c].size(); b0 += kSegMax) {
+              const size_t b1 = std::min(bucket[c].size(), b0 + kSegMax);
+              cls_src[c].insert(cls_src[c].end(), bucket[c].begin() + b0, bucket[c].begin() + b1);
+              row_segs[r].emplace_back(c, (int)cls_ptr[c].size() - 1);
+              cls_ptr[c].push_back((int)cls_src[c].size());
+            }
+        }
+        size_t per = 0;
+        for (int c = 0; c < kParts; ++c) per = std::max(per, cls_ptr[c].size() - 1);
+        per = (per + kPad - 1) / kPad * kPad;  // whole workgroups of the row kernel, whatever its rows per workgroup
+        const size_t n_cold = cls_ptr[kParts].size() - 1;
+        if ((long long)kParts * per + n_cold < INT_MAX / 2) {
+          S->long_part = true;
+          S->seg_per_xcd = (int)per;
+          S->hot_cols = (int)n_hot;
+          S->long_chunks.clear();
+          S->seg_ptr.assign(1, 0);
+          std::vector<int> cls_base(kParts + 1);
+          for (int c = 0; c <= kParts; ++c) {
+            cls_base[c] = (int)S->seg_ptr.size() - 1;
+            const int base = (int)S->seg_src.size();
+            S->seg_src.insert(S->seg_src.end(), cls_src[c].begin(), cls_src[c].end());
+            for (size_t q = 1; q < cls_ptr[c].size(); ++q) S->seg_ptr.push_back(base + cls_ptr[c][q]);
+            if (c < kParts)
+              for (size_t q = cls_ptr[c].size() - 1; q < per; ++q) S->seg_ptr.push_back(S->seg_ptr.back());  // empty pads
+          }
+          S->seg_col.resize(S->seg_src.size());
+          for (size_t k = 0; k < S->seg_src.size(); ++k) S->seg_col[k] = Ai[S->seg_src[k]];
+          // the executor copies A's values into this order walking A's array once: pairs sorted by source
+          {
+            std::vector<int> pos_of((size_t)nnz);
+            for (size_t e = 0; e < S->seg_src.size(); ++e) pos_of[S->seg_src[e]] = (int)e;
+            S->ent_src.reserve(S->seg_src.size());
+            S->ent_pos.reserve(S->seg_src.size());
+            std::vector<int> lrows;
+            for (const auto &lr : S->long_rows) lrows.push_back(lr.row);
+            std::sort(lrows.begin(), lrows.end());
+            for (const int i : lrows)
+              for (int k = Ap[i]; k < Ap[i + 1]; ++k) { S->ent_src.push_back(k); S->ent_pos.push_back(pos_of[k]); }
+          }
+          // A row adds up its segments' sums in a fixed order; a hub row has thousands of them, so
+          // groups of up to 32 segments are summed first (into slots behind the segments').
+          const int n_seg = (int)S->seg_ptr.size() - 1;
+          constexpr int kGroup = 32;
+          std::vector<int> slots;
+          for (size_t r = 0; r < S->long_rows.size(); ++r) {
+            slots.clear();
+            for (const auto &cs : row_segs[r]) slots.push_back(cls_base[cs.first] + cs.second);
+            if ((int)slots.size() > kGroup) {
+              std::vector<int> groups;
+              for (size_t b0 = 0; b0 < slots.size(); b0 += kGroup) {
+                const size_t b1 = std::min(slots.size(), b0 + kGroup);
+                tf::LongRow g{n_seg + (int)S->seg_groups.size(), (int)S->lrow_seg.size(), (int)(b1 - b0), 0};
+                S->lrow_seg.insert(S->lrow_seg.end(), slots.begin() + b0, slots.begin() + b1);
+                groups.push_back(g.row);
+                S->seg_groups.push_back(g);
+              }
+              slots.swap(groups);
+            }
+            S->long_rows[r].first = (int)S->lrow_seg.size();
+            S->long_rows[r].count = (int)slots.size();
+            S->lrow_seg.insert(S->lrow_seg.end(), slots.begin(), slots.end());
+          }
+        }
+      }
+    }
     // Remainder rows of similar length go together: a lane group walks a row alone, so a
     // workgroup is as slow as its longest row.  Order is kept inside a length class, and a
     // matrix whose rows all fall in one class keeps its order entirely.
@@ -496,7 +612,8 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   info->n_fused_rows = (int)s->fused_ids.size();
   info->n_remainder_rows = (int)(s->rem_rows.size() + s->long_rows.size());
   info->n_long_rows = (int)s->long_rows.size();
-  info->n_long_chunks = (int)s->long_chunks.size();
+  info->n_long_chunks = s->long_part ? (int)s->seg_ptr.size() - 1 : (int)s->long_chunks.size();
+  info->long_row_hot_cols = s->long_part ? s->hot_cols : 0;
   info->n_producer_rows = (int)std::min<long long>(s->n_producer_rows, INT_MAX);
   info->n_writeback_rows = s->n_writeback_rows;
   info->max_tile_producer_rows = s->slab_rows;
@@ -511,6 +628,7 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   long long ws = 0;
   if (s->n_writeback_rows > 0) ws += (long long)s->M * s->opts.N * 4;
   ws += (long long)s->long_chunks.size() * s->opts.N * 4;
+  if (s->long_part) ws += ((long long)s->seg_ptr.size() - 1 + (long long)s->seg_groups.size()) * s->opts.N * 4 + (long long)s->seg_src.size() * 4;  // partial sums, regrouped values
   if (s->user_K != s->opts.K) ws += ((long long)s->M + s->opts.N) * s->opts.K * 4;  // padded copies of B and C
   info->workspace_bytes = ws;
   return TF_OK;
@@ -609,7 +727,59 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
       return tf::fail(TF_ESCHEDULE, "remainder row %d is long but not chunked", i);
     if (tf_status rc = check_rem(i)) return rc;
   }
+  if (s->long_part) {
+    const int n_seg = (int)s->seg_ptr.size() - 1, n_hot_seg = 8 * s->seg_per_xcd;
+    if (n_seg < n_hot_seg || s->seg_ptr.empty() || s->seg_ptr[0] != 0 || s->seg_ptr[n_seg] != (int)s->seg_src.size() ||
+        s->seg_col.size() != s->seg_src.size())
+      return tf::fail(TF_ESCHEDULE, "long-row segments: bad tables");
+    std::vector<signed char> reader(M, -1);  // partition through which an intermediate row is read
+    std::vector<char> seen(s->nnz > 0 ? (size_t)s->nnz : 1, 0);
+    std::vector<char> seg_used(n_seg, 0);
+    for (const auto &lr : s->long_rows) {
+      if (tf_status rc = check_rem(lr.row)) return rc;
+      if (done[lr.row]++) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled twice", lr.row);
+      if (lr.first < 0 || lr.count < 0 || lr.first + lr.count > (int)s->lrow_seg.size())
+        return tf::fail(TF_ESCHEDULE, "long row %d: bad segment range", lr.row);
+      long long covered = 0;
+      std::vector<int> segs;  // the row's segments, groups expanded
+      for (int q = lr.first; q < lr.first + lr.count; ++q) {
+        const int slot = s->lrow_seg[q];
+        if (slot >= n_seg) {
+          if (slot - n_seg >= (int)s->seg_groups.size()) return tf::fail(TF_ESCHEDULE, "long row %d: unknown group slot %d", lr.row, slot);
+          const auto &g = s->seg_groups[slot - n_seg];
+          if (g.row != slot || g.count <= 0 || g.count > 32 || g.first < 0 || g.first + g.count > (int)s->lrow_seg.size())
+            return tf::fail(TF_ESCHEDULE, "long row %d: bad group %d", lr.row, slot - n_seg);
+          segs.insert(segs.end(), s->lrow_seg.begin() + g.first, s->lrow_seg.begin() + g.first + g.count);
+        } else {
+          segs.push_back(slot);
+        }
+      }
+      for (const int sg : segs) {
+        if (sg < 0 || sg >= n_seg || seg_used[sg]++) return tf::fail(TF_ESCHEDULE, "long row %d: segment %d unknown or used twice", lr.row, sg);
+        const int cls = sg < n_hot_seg ? sg / s->seg_per_xcd : -2;
+        if (s->seg_ptr[sg + 1] - s->seg_ptr[sg] > 64 || s->seg_ptr[sg + 1] <= s->seg_ptr[sg])
+          return tf::fail(TF_ESCHEDULE, "long row %d: segment %d is empty or longer than 64", lr.row, sg);
+        int prev = -1;
+        for (int e = s->seg_ptr[sg]; e < s->seg_ptr[sg + 1]; ++e) {
+          const int k = s->seg_src[e];
+          if (k < Ap[lr.row] || k >= Ap[lr.row + 1] || seen[k]++ || k <= prev || s->seg_col[e] != Ai[k])
+            return tf::fail(TF_ESCHEDULE, "long row %d: segment %d does not hold entries of the row once, in order", lr.row, sg);
+          prev = k;
+          if (cls >= 0) {  // (cold segments may read any row)
+            signed char &ow = reader[Ai[k]];
+            if (ow == -1) ow = (signed char)cls;
+            else if (ow != cls) return tf::fail(TF_ESCHEDULE, "intermediate row %d is read through two partitions", Ai[k]);
+          }
+          ++covered;
+        }
+      }
+      if (covered != Ap[lr.row + 1] - Ap[lr.row]) return tf::fail(TF_ESCHEDULE, "long row %d: segments hold %lld of its %d entries", lr.row, covered, Ap[lr.row + 1] - Ap[lr.row]);
+    }
+    for (int sg = 0; sg < n_seg; ++sg)
+      if (!seg_used[sg] && s->seg_ptr[sg + 1] != s->seg_ptr[sg]) return tf::fail(TF_ESCHEDULE, "segment %d belongs to no row", sg);
+  }
   for (const auto &lr : s->long_rows) {
+    if (s->long_part) break;
     if (tf_status rc = check_rem(lr.row)) return rc;
     if (done[lr.row]++) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled twice", lr.row);
     int k = Ap[lr.row];

@@ -72,6 +72,21 @@ struct tf_schedule {
   int xcd_chunk_rows = 0;           // rows per XCD turn of the row kernels (0: one contiguous run per XCD)
   std::vector<tf::LongChunk> long_chunks;
   std::vector<tf::LongRow> long_rows;
+  // Long rows cut by column instead (long_part): the most-read intermediate rows are dealt to 8
+  // partitions, one per XCD, small enough to stay in that XCD's L2; a long row's entries are
+  // regrouped into segments of one partition (or of none: "cold") and of at most 64 entries,
+  // each worked on like a short row by the XCD that caches its partition.  long_rows then holds
+  // first/count into lrow_seg.
+  bool long_part = false;
+  int seg_per_xcd = 0;            // hot segments per partition, padded with empty ones
+  int hot_cols = 0;               // intermediate rows in the 8 partitions together
+  std::vector<int> seg_ptr;       // [n_seg + 1] into seg_src/seg_col: partition 0's segments, 1's, ..., 7's, the cold ones
+  std::vector<int> seg_src;       // per regrouped entry: its index in A's arrays
+  std::vector<int> ent_src, ent_pos;  // the same pairs (index in A's arrays, regrouped position) sorted by the former
+  std::vector<int> seg_col;       // per regrouped entry: its column
+  std::vector<int> lrow_seg;      // per long row (first, count of tf::LongRow): the partial-sum slots it adds up, in order:
+                                  // segments, or for a row of more than 32 segments groups of up to 32 of them
+  std::vector<tf::LongRow> seg_groups;  // such groups: row = the group's slot (n_seg + its index), first/count into lrow_seg
   long long fused_nnz = 0;
   int n_writeback_rows = 0;
   long long n_producer_rows = 0;

@@ -675,6 +675,44 @@ __global__ __launch_bounds__(kBlock) void long_row_reduce_kernel(const LongRow *
   }
 }
 
+// Column-partitioned long rows: out[pos[i]] = val[src[i]] puts the values of A into the order of
+// the regrouped entries (src ascending: the reads walk A's array once, the writes fall into
+// nine ascending streams), and Y[row] (+)= the row's segment sums, added in the order of its list.
+__global__ void scatter_values_kernel(const int *__restrict__ src, const int *__restrict__ pos,
+                                      const float *__restrict__ val, float *__restrict__ out, int n) {
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) out[pos[i]] = val[src[i]];
+}
+
+// One lane group per long row, every lane four adjacent columns; the partial rows of eight
+// segments are requested before the first is added.
+template <int V, int LPR>
+__global__ __launch_bounds__(kBlock) void long_seg_reduce_kernel(const LongRow *__restrict__ rows, int n_long,
+                                                                 const int *__restrict__ seg_of,
+                                                                 const float *partial, float *Y, int N,
+                                                                 int accumulate) {  // (Y may be `partial` itself: other rows)
+  constexpr int G = kBlock / LPR;
+  const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
+  const int q = blockIdx.x * G + group;
+  if (q >= n_long) return;
+  const LongRow lr = rows[q];
+  for (int c0 = 0; c0 < N; c0 += LPR * V) {
+    const int coff = c0 + glane * V;
+    if (coff >= N) continue;
+    fvec<V> acc = vzero<V>();
+    if (accumulate) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)lr.row * N + coff);
+    for (int p0 = 0; p0 < lr.count; p0 += 8) {
+      fvec<V> x[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (p0 + u < lr.count) x[u] = *reinterpret_cast<const fvec<V> *>(partial + (size_t)seg_of[lr.first + p0 + u] * N + coff);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (p0 + u < lr.count) vadd<V>(x[u], acc);
+    }
+    *reinterpret_cast<fvec<V> *>(Y + (size_t)lr.row * N + coff) = acc;
+  }
+}
+
 // dst (rows x ld_dst) = src (src_rows x ld_src) in its top left corner, zeros elsewhere.
 __global__ void pad_kernel(const float *__restrict__ src, int src_rows, int ld_src, float *__restrict__ dst, int rows,
                            int ld_dst) {
@@ -1580,6 +1618,42 @@ hipError_t launch_long_rows(const LongChunk *chunks, int n_chunks, const LongRow
   if (err != hipSuccess) return err;
   hipLaunchKernelGGL(long_row_reduce_kernel, dim3(n_long), dim3(kBlock), 0, st, rows, partial, Y, N,
                      accumulate);
+  return hipGetLastError();
+}
+
+// Long rows regrouped by column partition: the hot segments (n_hot of them, an eighth per XCD, in
+// XCD order) run on the row kernel with one contiguous run of segments per XCD, the cold ones
+// round-robin; then every long row adds up its segments.
+hipError_t launch_long_rows_partitioned(const int *seg_ptr, const int *seg_col, const int *ent_src, const int *ent_pos,
+                                        float *seg_val, int n_entries, int n_hot, int n_seg, const LongRow *groups,
+                                        int n_groups, const LongRow *rows, int n_long, const int *seg_of,
+                                        const float *Ax, const float *X, float *partial, float *Y, int N,
+                                        int accumulate, hipStream_t st) {
+  if (n_long <= 0) return hipSuccess;
+  if (n_entries > 0) {
+    const int blocks = std::min((n_entries + kBlock - 1) / kBlock, 65536);
+    hipLaunchKernelGGL(scatter_values_kernel, dim3(blocks), dim3(kBlock), 0, st, ent_src, ent_pos, Ax, seg_val, n_entries);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+  }
+  hipError_t err = launch_spmm_rows(nullptr, n_hot, seg_ptr, seg_col, seg_val, X, partial, N, 0, -1, st);
+  if (err != hipSuccess) return err;
+  err = launch_spmm_rows(nullptr, n_seg - n_hot, seg_ptr + n_hot, seg_col, seg_val, X, partial + (size_t)n_hot * N, N, 0,
+                         0, st);
+  if (err != hipSuccess) return err;
+  const Shape s = pick_shape(N);
+  const int G = kBlock / s.LPR;
+  // groups of segments of the rows with many (into their own slots of `partial`), then the rows
+#define CALL(V_, L_)                                                                                      \
+  do {                                                                                                    \
+    if (n_groups > 0)                                                                                     \
+      hipLaunchKernelGGL((long_seg_reduce_kernel<V_, L_>), dim3((n_groups + G - 1) / G), dim3(kBlock), 0, st, groups, \
+                         n_groups, seg_of, partial, partial, N, 0);                                       \
+    hipLaunchKernelGGL((long_seg_reduce_kernel<V_, L_>), dim3((n_long + G - 1) / G), dim3(kBlock), 0, st, rows, n_long, \
+                       seg_of, partial, Y, N, accumulate);                                                \
+  } while (0)
+  TF_DISPATCH_VL(s.V, s.LPR, CALL);
+#undef CALL
   return hipGetLastError();
 }
 
