@@ -217,7 +217,9 @@ def main():
     alg_bytes = w.algorithmic_bytes(cfg)
     gflops = flops / (ms_per_step * 1e-3) / 1e9
     achieved = alg_bytes / (dev_ms * 1e-3) / 1e9
-    n_kernels = 1 + (1 if info["n_remainder_rows"] - info["n_long_rows"] > 0 else 0) + (2 if info["n_long_rows"] else 0)
+    # long rows: chunk kernel + sums, or (by column partition) values, hot segments, cold segments, group sums, row sums
+    n_kernels = 1 + (1 if info["n_remainder_rows"] - info["n_long_rows"] > 0 else 0) + \
+        ((5 if info["long_row_hot_cols"] else 2) if info["n_long_rows"] else 0)
 
     check = None
     if not args.no_check:
@@ -237,7 +239,7 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": cfg["name"], "op": cfg["op"], "rows": int(A.shape[0]), "nnz": int(A.nnz), "N": N, "K": K,
-                   "lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "wide_strips": bool(info["wide_strips"]), "streamed": bool(info["streamed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
+                   "lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "wide_strips": bool(info["wide_strips"]), "long_row_hot_cols": info["long_row_hot_cols"], "streamed": bool(info["streamed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
                    "remainder_rows": info["n_remainder_rows"], "recomputed_rows": info["n_producer_rows"] - A.shape[1],
                    "writeback_rows": info["n_writeback_rows"], "kernels_per_step": n_kernels,
                    "inspector_s": round(inspect_s, 4), **({"reorder_s": round(reorder_s, 4)} if reorder_s is not None else {}), "rel_err_vs_f64": check, "device": dev["arch"]},
