@@ -252,7 +252,7 @@ def test_long_rows_by_column_partition(tf):
     assert info["n_long_rows"] == base.info()["n_long_rows"]
     rl = np.diff(A.indptr)
     long_nnz = int(rl[rl > 32].sum())
-    assert 0 < info["long_row_hot_cols"] <= 8 * (4 << 20) // (128 * 4)
+    assert 0 < info["long_row_hot_cols"] <= 8 * (12 << 20) // (128 * 4)
     # at least one segment per 64 entries, and the eight hot lists are padded to whole workgroups
     assert info["n_long_chunks"] >= long_nnz // 64 and info["n_long_chunks"] % 1 == 0
     assert info["workspace_bytes"] >= info["n_long_chunks"] * 128 * 4 + long_nnz * 4
