@@ -1,0 +1,59 @@
+// Host-only sanitizer harness: the inspector (every kind of schedule), its validator, the file
+// readers and the reordering, compiled with -fsanitize=address,undefined together with
+// csrc/tf_inspector.cpp, tf_io.cpp and tf_reorder.cpp (no GPU code: the three functions those
+// files take from the HIP side are stubbed here).  Exits 0 when every schedule validates.
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+#include "tf_internal.h"
+namespace tf {
+static char g_err[512];
+tf_status fail(tf_status code, const char *fmt, ...) { va_list ap; va_start(ap, fmt); vsnprintf(g_err, sizeof g_err, fmt, ap); va_end(ap); return code; }
+int default_compute_units() { return 256; }
+void release_device_schedule(DeviceSchedule *) {}
+}
+static void band(int M, int bw, int per, unsigned seed, std::vector<int> &p, std::vector<int> &i) {
+  std::mt19937 g(seed); p.assign(1, 0); i.clear();
+  for (int r = 0; r < M; ++r) { std::vector<int> c; for (int k = 0; k < per; ++k) { int x = r - bw / 2 + (int)(g() % bw); if (x >= 0 && x < M) c.push_back(x); }
+    std::sort(c.begin(), c.end()); c.erase(std::unique(c.begin(), c.end()), c.end()); i.insert(i.end(), c.begin(), c.end()); p.push_back((int)i.size()); }
+}
+static void powerlaw(int M, int nnz, unsigned seed, std::vector<int> &p, std::vector<int> &i) {
+  std::mt19937 g(seed); std::vector<std::vector<int>> rows(M);
+  auto pick = [&]() { double u = (g() % 1000000 + 1) / 1000001.0; return (int)((M - 1) * u * u * u * u); };
+  for (int k = 0; k < nnz; ++k) rows[pick()].push_back(pick());
+  p.assign(1, 0); i.clear();
+  for (auto &c : rows) { std::sort(c.begin(), c.end()); c.erase(std::unique(c.begin(), c.end()), c.end()); i.insert(i.end(), c.begin(), c.end()); p.push_back((int)i.size()); }
+}
+static int run(const char *name, int M, const std::vector<int> &p, const std::vector<int> &i, tf_inspect_opts o) {
+  tf_schedule *s = nullptr;
+  tf_status rc = tf_inspect(M, M, p.data(), i.data(), &o, &s);
+  if (rc) { printf("%s: inspect %d %s\n", name, rc, tf::g_err); return o.op < 0 ? 0 : 1; }
+  rc = tf_schedule_validate(s, M, M, p.data(), i.data());
+  tf_schedule_info info; tf_schedule_get_info(s, &info);
+  tf_schedule_view v; tf_schedule_get_view(s, &v);
+  printf("%s: validate %d tiles %d fused %d long %d hot %d wide %d streamed %d ws %lld %s\n", name, rc, info.n_tiles, info.n_fused_rows, info.n_long_rows, info.long_row_hot_cols, info.wide_strips, info.streamed, info.workspace_bytes, rc ? tf::g_err : "");
+  tf_schedule_free(s);
+  return rc != 0;
+}
+int main() {
+  int bad = 0;
+  std::vector<int> p, i;
+  band(40000, 32, 16, 1, p, i);
+  { tf_inspect_opts o{}; o.op = TF_OP_SPMM_SPMM; o.N = 128; o.inner_Ap = p.data(); o.inner_Ai = i.data(); o.inner_cols = 40000; bad += run("band wide", 40000, p, i, o);
+    o.wide_strips = -1; bad += run("band narrow", 40000, p, i, o); o.inner_Ap = nullptr; o.inner_Ai = nullptr; o.wide_strips = 0; bad += run("band general", 40000, p, i, o);
+    tf_inspect_opts g{}; g.op = TF_OP_GEMM_SPMM; g.N = 128; g.K = 100; bad += run("band gemm stream", 40000, p, i, g); g.N = 64; g.K = 20; g.compute_units = 1024; bad += run("band gemm tiles", 40000, p, i, g); }
+  powerlaw(60000, 1500000, 2, p, i);
+  { tf_inspect_opts o{}; o.op = TF_OP_GEMM_SPMM; o.N = 128; o.K = 128; o.long_row_partition = 1; bad += run("powerlaw part", 60000, p, i, o);
+    o.long_row_partition = -1; bad += run("powerlaw chunks", 60000, p, i, o);
+    o.op = TF_OP_SPMM_SPMM; o.K = 0; o.N = 20; o.long_row_partition = 1; bad += run("powerlaw spmm part", 60000, p, i, o); }
+  { std::vector<int> perm(60000); tf_status rc = tf_reorder_rcm(60000, p.data(), i.data(), perm.data()); std::vector<float> x(i.size(), 1.f); int *bp, *bi; float *bx;
+    rc = rc ? rc : tf_permute_csr(60000, p.data(), i.data(), x.data(), perm.data(), &bp, &bi, &bx); printf("rcm+permute %d\n", rc); bad += rc != 0; tf_host_free(bp); tf_host_free(bi); tf_host_free(bx); }
+  { FILE *f = fopen("host_sanitize_t.mtx", "w"); fprintf(f, "%%%%MatrixMarket matrix coordinate real symmetric\n4 4 3\n1 1 2.0\n3 1 -1\n4 4 5e-1\n"); fclose(f);
+    int M, N, nnz, *ap, *ai; float *ax; tf_status rc = tf_read_matrix("host_sanitize_t.mtx", &M, &N, &nnz, &ap, &ai, &ax); printf("read %d nnz %d\n", rc, nnz); bad += rc != 0 || nnz != 4; tf_host_free(ap); tf_host_free(ai); tf_host_free(ax); }
+  printf("bad %d\n", bad);
+  return bad;
+}
