@@ -176,9 +176,9 @@ typedef struct {
                             entries read from the CSR arrays in place (LDS rows of 256 bytes are
                             read without bank conflicts), tile_rows defaults to rows / compute
                             units; -1 = strips of strip_cols columns, the tile's entries staged in
-                            LDS, two workgroups per compute unit; 0 = the first for matrices of
-                            128 rows per compute unit or more when strip_cols, tile_rows and
-                            lds_budget_bytes are left at 0, else the second                    */
+                            LDS, two workgroups per compute unit; 0 = the first when N % 64 == 0 and
+                            strip_cols, tile_rows and lds_budget_bytes are left at 0, else the
+                            second                                                             */
   int long_row_partition; /* long remainder rows (more than long_row_nnz entries): 1 = regroup their entries
                             by column so that each XCD gathers from its own part of the most-read
                             intermediate rows, which then stays in its L2 (power-law graphs); -1 = cut

@@ -201,7 +201,7 @@ def test_windowed_tiles(tf):
     every column the tile's producer rows read."""
     for A, N in ((tf.workloads.banded_random(4096, 32, 16, seed=3), 128), (tf.workloads.laplacian_2d(48), 64)):
         Ah = tf.CsrMatrix.from_scipy(A)
-        S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N, inner=Ah)
+        S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N, inner=Ah, wide_strips=-1)  # the lane-group kernel's tiles
         S.validate()
         info, view = S.info(), S.view()
         assert info["windowed"] == 1 and info["strip_cols"] == 32
@@ -215,9 +215,10 @@ def test_windowed_tiles(tf):
 
 
 def test_wide_strip_tiles(tf):
-    """A matrix with 128 rows per compute unit or more gets one windowed tile per compute unit
-    for the 64-column kernel: LDS holds row pointers, window and slab (no entries), up to
-    160 KB; any explicit strip, tile or LDS choice keeps the lane-group kernel's tiles."""
+    """With the inner pattern given and N a multiple of 64, windowed tiles are built for the
+    64-column kernel, one per compute unit (at least 64 rows): LDS holds row pointers, window
+    and slab (no entries), up to 160 KB; any explicit strip, tile or LDS choice keeps the
+    lane-group kernel's tiles."""
     A = tf.workloads.banded_random(4096, 32, 16, seed=3)
     Ah = tf.CsrMatrix.from_scipy(A)
     S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128, inner=Ah, compute_units=16)
@@ -229,7 +230,8 @@ def test_wide_strip_tiles(tf):
     P = int((tr[:, 1] - tr[:, 0]).max())  # producer rows of the largest tile: window and slab each hold at least as many
     assert 4 * 64 * 2 * P <= info["lds_bytes"] <= 163840
     validate(view, info, A, 163840)
-    for kw in (dict(compute_units=64), dict(compute_units=16, strip_cols=32), dict(compute_units=16, tile_rows=128),
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128, inner=Ah, compute_units=256).info()["n_tiles"] == 64  # 64 rows each
+    for kw in (dict(compute_units=16, strip_cols=32), dict(compute_units=16, tile_rows=128),
                dict(compute_units=16, lds_budget_bytes=65536), dict(compute_units=16, wide_strips=-1)):
         assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128, inner=Ah, **kw).info()["wide_strips"] == 0, kw
     assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=96, inner=Ah, compute_units=16).info()["wide_strips"] == 0

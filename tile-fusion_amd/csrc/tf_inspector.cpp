@@ -105,12 +105,12 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     return tf::fail(TF_EINVAL, "tf_inspect: strip_cols must be 32 or 64");
   const bool have_inner = o.op == TF_OP_SPMM_SPMM && o.inner_Ap && (o.inner_Ai || o.inner_Ap[M] == 0) && o.inner_cols > 0;
   const bool want_window = have_inner && o.N % o.strip_cols == 0 && o.wide_strips <= 0;
-  // (one tile per compute unit: a matrix with fewer than 128 rows per compute unit is better
-  // served by more and smaller tiles)
+  // (measured faster than the lane-group kernel from 1,024 to 2^20 rows of a band, so it is the
+  // default wherever it applies)
   // (the kernel addresses the CSR arrays with 32-bit byte offsets and loads four entries at a time)
   const bool want_wide = have_inner && o.N % 64 == 0 && o.inner_Ap[M] >= 4 && nnz >= 4 && o.inner_Ap[M] < (1 << 30) && nnz < (1 << 30) &&
                          (o.wide_strips > 0 || (o.wide_strips == 0 && user->strip_cols <= 0 && user->lds_budget_bytes <= 0 &&
-                                              user->tile_rows <= 0 && M >= 128LL * o.compute_units));
+                                              user->tile_rows <= 0));
   int r_cap = o.tile_rows > 0 ? o.tile_rows : ceil_div(M, 2 * o.compute_units);
   if (o.op == TF_OP_GEMM_SPMM) r_cap = ceil_div(r_cap, 32) * 32;
   r_cap = std::max(r_cap, o.tile_rows > 0 ? 1 : 64);  // smaller tiles spend most of their work on halo rows
