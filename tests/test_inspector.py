@@ -284,7 +284,8 @@ def test_streamed_runs(tf):
     assert info["streamed"] == 1 and info["ring_rows"] == 256
     assert info["n_fused_rows"] == M and info["n_writeback_rows"] == 0
     tr = view["tile_range"]
-    assert len(tr) == M // 256 and np.all(tr[:, 2] - tr[:, 0] <= 16) and np.all(tr[:, 1] - tr[:, 3] <= 16)
+    assert len(tr) == 256 and np.all(tr[:, 2] - tr[:, 0] <= 16) and np.all(tr[:, 1] - tr[:, 3] <= 16)  # a run per compute unit
+    assert set((tr[:, 3] - tr[:, 2]).tolist()) <= {156, 157}
     for t in range(len(tr)):
         st = view["tile_step"][t]
         steps = -(-(tr[t][1] - tr[t][0]) // 64)

@@ -68,10 +68,11 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     for (int c = 256; c <= 4096 && stream_fixed + (long long)c * (o.N + 4) * 4 <= budget; c *= 2) r = c;
     return r;
   };
-  // (a run needs a few hundred rows to pay for its start-up and halo: with fewer than 128 rows
-  // per compute unit the tile kernel, which spreads over all of them, is the faster one)
+  // (a run needs a hundred rows or more to pay for its start-up and halo: with fewer than 96 rows
+  // per compute unit the tile kernel, which spreads over all of them, is the faster one --
+  // banded matrix, K = N = 128: 16,384 rows 23 us in tiles / 27 us in runs, 24,576 rows 36 / 28)
   if (o.compute_units <= 0) o.compute_units = tf::default_compute_units();
-  const bool long_enough = user->tile_rows > 0 || M >= 128LL * o.compute_units;
+  const bool long_enough = user->tile_rows > 0 || M >= 96LL * o.compute_units;
   const int ring_rows = gemm_regw && long_enough ? ring_for(o.lds_budget_bytes > 0 ? o.lds_budget_bytes : kMaxLds) : 0;
   const bool gemm_stream = ring_rows > 0;
   if (o.lds_budget_bytes <= 0)  // two workgroups per CU, except for the kernels that own a compute unit
@@ -253,7 +254,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     // ring: with q(c) = (c - prod_begin) / 64 that is q(last) - q(first) <= ring_rows/64 - 2.
     if (gemm_stream) {
       int own = user->tile_rows > 0 ? std::max(user->tile_rows, 64)
-                                     : std::max(ceil_div(ceil_div(M, o.compute_units), 64) * 64, 256);  // short runs are mostly halo
+                                     : std::max(ceil_div(M, o.compute_units), 128);  // one run per compute unit: a run
+      // count that leaves compute units idle costs more than short runs do (32,768 rows: 29 us in 256 runs of 128, 43 us in 128 of 256)
       own = std::min(own, 1000 * 64 - 2 * ring_rows);  // a run's step table holds 1024 steps
       const int qspan = ring_rows / 64 - 2;
       // What the consumer wavefronts of the kernel take per step without falling behind, and
@@ -264,9 +266,13 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       const int max_len = 32;
       S->stream_step_cap = step_cap;
       S->stream_max_len = max_len;
+      // without a run length from the caller the rows are dealt evenly: M / own runs, one per compute unit
+      const int n_even = user->tile_rows > 0 ? 0 : std::max({1, std::min(o.compute_units, M / 128), ceil_div(M, own)});
+      int run = 0;
       while (s < M) {
-        int e = std::min(M, s + own);
-        if (M - e < own / 2) e = M;  // a short last run would be mostly halo: the one before takes its rows
+        int e = n_even > 0 ? (int)((long long)(run + 1) * M / n_even) : std::min(M, s + own);
+        ++run;
+        if (n_even == 0 && M - e < own / 2) e = M;  // a short last run would be mostly halo: the one before takes its rows
         tf::TileDesc t{};
         t.own_begin = s; t.own_end = e; t.prod_begin = s; t.prod_end = e;
         t.cons_begin = t.cons_end = (int)S->fused_ids.size();
