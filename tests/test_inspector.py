@@ -236,6 +236,12 @@ def test_wide_strip_tiles(tf):
         assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128, inner=Ah, **kw).info()["wide_strips"] == 0, kw
     assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=96, inner=Ah, compute_units=16).info()["wide_strips"] == 0
     assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah, compute_units=64, wide_strips=1).info()["wide_strips"] == 1
+    # where LDS allows fewer rows than one compute unit's share, the tiles are sized for a whole number of turns
+    for cu in (2, 3, 4, 6, 7):
+        Sm = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128, inner=Ah, compute_units=cu)
+        Sm.validate()
+        n = Sm.info()["n_tiles"]
+        assert n > cu and n % cu == 0 and Sm.info()["n_fused_rows"] == 4096, (cu, n)
 
 
 def test_long_rows_by_column_partition(tf):

@@ -162,11 +162,11 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     // unit: long matrices).  Narrow strips: 32 or 64 columns, the tile's entries staged in LDS
     // as well, two workgroups per compute unit.
     bool windowed = false, win_wide = false;
-    auto build_window = [&](bool wide) {
+    auto build_window = [&](bool wide, int wide_cap = 0) {
       const int *Bp = o.inner_Ap, *Bi = o.inner_Ai;
       const int SW = wide ? 64 : o.strip_cols;
       const int budget = wide ? (user->lds_budget_bytes > 0 ? user->lds_budget_bytes : kMaxLds) : o.lds_budget_bytes;
-      const int cap = wide ? (user->tile_rows > 0 ? user->tile_rows : std::max(64, ceil_div(M, o.compute_units))) : r_cap;
+      const int cap = wide ? (wide_cap > 0 ? wide_cap : user->tile_rows > 0 ? user->tile_rows : std::max(64, ceil_div(M, o.compute_units))) : r_cap;
       std::vector<int> blo(M), bhi(M);
       bool ok = (Bp[0] == 0);
       for (int r = 0; r < M && ok; ++r) {
@@ -234,6 +234,25 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       return true;
     };
     if (want_wide) windowed = win_wide = build_window(true);
+    if (win_wide && user->tile_rows <= 0 && (int)S->tiles.size() > o.compute_units) {
+      // More tiles than compute units (LDS, not the row count, set the tile size): every compute
+      // unit takes several tiles in turn, so size them for a whole number of turns.
+      auto keep_tiles = S->tiles; auto keep_ids = S->fused_ids; auto keep_win = S->win;
+      const long long keep_prod = S->n_producer_rows; const int keep_slab = S->slab_rows, keep_lds = S->lds_bytes;
+      const int first_turns = ceil_div((int)S->tiles.size(), o.compute_units);
+      bool done = (int)S->tiles.size() == o.compute_units * first_turns;
+      for (int turns = first_turns; !done && turns <= first_turns + 2; ++turns) {
+        const int cap2 = ceil_div(M, o.compute_units * turns);
+        if (cap2 < 64) break;
+        done = build_window(true, cap2) && (int)S->tiles.size() <= o.compute_units * turns &&
+               (int)S->tiles.size() > o.compute_units * (turns - 1) + o.compute_units / 2;
+      }
+      if (!done) {  // (keeps the first tiling)
+        S->tiles.swap(keep_tiles); S->fused_ids.swap(keep_ids); S->win.swap(keep_win);
+        S->n_producer_rows = keep_prod; S->slab_rows = keep_slab; S->lds_bytes = keep_lds;
+        S->opts.tile_rows = std::max(64, ceil_div(M, o.compute_units));
+      }
+    }
     if (!windowed && want_window) windowed = build_window(false);
     S->win_wide = win_wide;
     S->windowed = windowed;
