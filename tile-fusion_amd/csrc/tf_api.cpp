@@ -59,7 +59,7 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *, const int *, int, c
                                            const float *, int, const float *, const int *, const int *,
                                            const float *, int, float *, int, int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
-                            float *, int, int, int, hipStream_t);
+                            float *, int, int, int, int, hipStream_t);
 hipError_t launch_long_rows_partitioned(const int *, const int *, const int *, const int *, float *, int, int, int, const LongRow *, int, const LongRow *, int,
                                         const int *, const float *, const float *, float *, float *, int, int,
                                         hipStream_t);
@@ -74,6 +74,12 @@ hipError_t launch_fused_gemm_spmm_stream(const TileDesc *, int, const int *, con
 hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t);
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 hipError_t launch_pad(const float *, int, int, float *, int, int, hipStream_t);
+
+// An intermediate larger than the 256 MB last-level cache is gone from it before its readers
+// come: such rows leave through streaming stores.
+inline int inter_streams(const tf_schedule *s) {
+  return (size_t)s->M * s->opts.N * sizeof(float) > ((size_t)256 << 20) ? 1 : 0;
+}
 
 static thread_local char g_err[512] = "";
 
@@ -187,7 +193,7 @@ static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int
   if (!s->rem_rows.empty()) {
     // identity list: no indirection needed
     TF_HIP(launch_spmm_rows(s->rem_identity ? nullptr : d->rem_rows, (int)s->rem_rows.size(), A->p, A->i,
-                            A->x, d->inter, D->d, N, accumulate, s->xcd_chunk_rows, st));
+                            A->x, d->inter, D->d, N, accumulate, s->xcd_chunk_rows, /*streaming=*/1, st));
   }
   if (s->long_part)
     TF_HIP(launch_long_rows_partitioned(d->seg_ptr, d->seg_col, d->ent_src, d->ent_pos, d->seg_val, (int)s->seg_src.size(),
@@ -449,7 +455,7 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
   if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
     const bool all = (int)s->plain_rows.size() == s->M;
     TF_HIP(tf::launch_spmm_rows(all ? nullptr : d->plain_rows, (int)s->plain_rows.size(), B->p, B->i, B->x,
-                                C->d, d->inter, s->opts.N, 0, s->xcd_chunk_rows, st));
+                                C->d, d->inter, s->opts.N, 0, s->xcd_chunk_rows, tf::inter_streams(s), st));
   }
   return tf::run_remainder(A, D, s, acc, st);
 }
@@ -495,7 +501,7 @@ extern "C" tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, un
   if (X->M != A->N || Y->M != A->M || X->N != Y->N)
     return fail(TF_EINVAL, "tf_spmm: shapes A %d x %d, X %d x %d, Y %d x %d", A->M, A->N, X->M, X->N, Y->M, Y->N);
   TF_HIP(tf::launch_spmm_rows(nullptr, A->M, A->p, A->i, A->x, X->d, Y->d, X->N,
-                              (flags & TF_ACCUMULATE) ? 1 : 0, 0, static_cast<hipStream_t>(stream)));
+                              (flags & TF_ACCUMULATE) ? 1 : 0, 0, /*streaming=*/1, static_cast<hipStream_t>(stream)));
   return TF_OK;
 }
 

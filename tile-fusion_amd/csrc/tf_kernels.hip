@@ -37,6 +37,17 @@ template <int V> __device__ __forceinline__ void vadd(const fvec<V> &x, fvec<V> 
 #pragma unroll
   for (int i = 0; i < V; ++i) acc.v[i] += x.v[i];
 }
+// Output that this library does not read again leaves through a streaming (nontemporal) store.
+template <int V> __device__ __forceinline__ void store_streaming(float *dst, const fvec<V> &v) {
+  typedef float fv __attribute__((ext_vector_type(V)));
+  fv x;
+#pragma unroll
+  for (int u = 0; u < V; ++u) x[u] = v.v[u];
+  __builtin_nontemporal_store(x, reinterpret_cast<fv *>(dst));
+}
+template <> __device__ __forceinline__ void store_streaming<1>(float *dst, const fvec<1> &v) {
+  __builtin_nontemporal_store(v.v[0], dst);
+}
 
 // Consecutive workgroup ids land on different XCDs (each with its own 4 MB L2).  Work items
 // are cut into chunks of `bpc` consecutive items and chunk c goes to XCD c % 8, so that an
@@ -197,7 +208,7 @@ __global__ __launch_bounds__(kBlock) void fused_spmm_spmm_kernel(
       fvec<V> acc = vzero<V>();
       if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)i * N + coff);
       row_dot<V, LPR>(Ai, Ax, Ap[i], Ap[i + 1], glane, ok, tsrc, acc);
-      if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)i * N + coff) = acc;
+      if (ok) store_streaming<V>(D + (size_t)i * N + coff, acc);
     }
   }
 }
@@ -412,7 +423,7 @@ __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
       // this loop wait for the one before it)
       if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
       acc = lds_row_dot_quad(ent, rp[r], rp[r + 1] - kWinPad, tbase, glane & 3, acc);
-      *reinterpret_cast<fvec<4> *>(dst) = acc;
+      store_streaming<4>(dst, acc);
     }
   }
 }
@@ -494,7 +505,11 @@ __device__ __forceinline__ fvec<4> row_dot_quad_regs(const QuadEntries &first, c
 __device__ __forceinline__ fvec<4> window64_unit(const float *__restrict__ C, int first_row, int N, int c0, int n4,
                                                  int u) {
   const int uu = u < n4 ? u : 0;
-  return *reinterpret_cast<const fvec<4> *>(C + (size_t)(first_row + uu / 16) * N + c0 + (uu % 16) * 4);
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const f4 x = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(C + (size_t)(first_row + uu / 16) * N + c0 + (uu % 16) * 4));
+  fvec<4> r;
+  r.v[0] = x[0]; r.v[1] = x[1]; r.v[2] = x[2]; r.v[3] = x[3];
+  return r;
 }
 
 template <bool ACC>
@@ -567,8 +582,7 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
       {
         fvec<4> acc = vzero<4>();
         if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
-        *reinterpret_cast<fvec<4> *>(dst) =
-            row_dot_quad_regs<EXACT>(ea, Ai, Ax, ea.kb, ea.ke, nnzA, offA, tbase, q, acc);
+        store_streaming<4>(dst, row_dot_quad_regs<EXACT>(ea, Ai, Ax, ea.kb, ea.ke, nnzA, offA, tbase, q, acc));
         dst += round_stride;
       }
       if (i + G >= R) break;
@@ -576,8 +590,7 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
       {
         fvec<4> acc = vzero<4>();
         if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
-        *reinterpret_cast<fvec<4> *>(dst) =
-            row_dot_quad_regs<EXACT>(eb, Ai, Ax, eb.kb, eb.ke, nnzA, offA, tbase, q, acc);
+        store_streaming<4>(dst, row_dot_quad_regs<EXACT>(eb, Ai, Ax, eb.kb, eb.ke, nnzA, offA, tbase, q, acc));
         dst += round_stride;
       }
     }
@@ -611,7 +624,7 @@ template <int V, int LPR>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
     const int *__restrict__ rows, int n_rows, int n_blocks, int per_xcd, const int *__restrict__ Ap,
     const int *__restrict__ Ai, const float *__restrict__ Ax, const float *__restrict__ X, int ldx,
-    float *__restrict__ Y, int N, int accumulate) {
+    float *__restrict__ Y, int N, int accumulate, int streaming) {
   constexpr int G = kBlock / LPR;
   const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
   const int b = xcd_contiguous(blockIdx.x, per_xcd);
@@ -627,7 +640,10 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
     fvec<V> acc = vzero<V>();
     if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
     row_dot_direct<V, LPR>(Ai, Ax, kb, ke, ok, src, acc);
-    if (ok) *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
+    if (ok) {
+      if (streaming) store_streaming<V>(Y + (size_t)i * N + coff, acc);
+      else *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
+    }
   }
 }
 
@@ -849,7 +865,7 @@ __global__ __launch_bounds__(kBlock) void fused_gemm_spmm_kernel(
     fvec<V> acc = vzero<V>();
     if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)i * N + coff);
     row_dot<V, LPR>(Ai, Ax, Ap[i], Ap[i + 1], glane, ok, tsrc, acc);
-    if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)i * N + coff) = acc;
+    if (ok) store_streaming<V>(D + (size_t)i * N + coff, acc);
   }
 }
 
@@ -1201,7 +1217,7 @@ __global__ __launch_bounds__(kGemmBlock) void fused_gemm_spmm_regw_kernel(
       if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)ci.x * N + coff);
       row_dot_loaded<V, LPR>(pc[r], pa[r], min(LPR, ci.z - ci.y), ok, tsrc, acc);
       row_dot<V, LPR>(Ai, Ax, ci.y + LPR, ci.z, glane, ok, tsrc, acc);
-      if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)ci.x * N + coff) = acc;
+      if (ok) store_streaming<V>(D + (size_t)ci.x * N + coff, acc);
     }
   }
   for (int x = RND * G + group; x < R; x += G) {
@@ -1209,7 +1225,7 @@ __global__ __launch_bounds__(kGemmBlock) void fused_gemm_spmm_regw_kernel(
     fvec<V> acc = vzero<V>();
     if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(D + (size_t)ci.x * N + coff);
     row_dot<V, LPR>(Ai, Ax, ci.y, ci.z, glane, ok, tsrc, acc);
-    if (ok) *reinterpret_cast<fvec<V> *>(D + (size_t)ci.x * N + coff) = acc;
+    if (ok) store_streaming<V>(D + (size_t)ci.x * N + coff, acc);
   }
 }
 
@@ -1398,7 +1414,7 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
         acc = lds_row_dot8(scratch, 0, cnt, rbase, acc);
       }
     }
-    if (ok) *reinterpret_cast<fvec<4> *>(dst) = acc;
+    if (ok) store_streaming<4>(dst, acc);
   };
   // Entries glane, glane + LPR, .. of a row (lanes past the row's end re-read its last entry;
   // the row's length decides what is used).
@@ -1589,7 +1605,7 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *tiles, const int *win
 
 hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const int *Ai, const float *Ax,
                             const float *X, float *Y, int N, int accumulate, int xcd_chunk_rows,
-                            hipStream_t st) {
+                            int streaming, hipStream_t st) {
   if (n_rows <= 0) return hipSuccess;
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
@@ -1598,7 +1614,7 @@ hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const in
   const int bpc = xcd_chunk_rows == 0 ? 0 : chunk_bpc(n_blocks, xcd_chunk_rows > 0 ? std::max(1, xcd_chunk_rows / G) : 0);
 #define CALL(V_, L_)                                                                                   \
   hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(grid_chunked(n_blocks, bpc)), dim3(kBlock), 0, st, \
-                     rows, n_rows, n_blocks, bpc, Ap, Ai, Ax, X, N, Y, N, accumulate)
+                     rows, n_rows, n_blocks, bpc, Ap, Ai, Ax, X, N, Y, N, accumulate, streaming)
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
 #undef CALL
   return hipGetLastError();
@@ -1636,10 +1652,10 @@ hipError_t launch_long_rows_partitioned(const int *seg_ptr, const int *seg_col, 
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
   }
-  hipError_t err = launch_spmm_rows(nullptr, n_hot, seg_ptr, seg_col, seg_val, X, partial, N, 0, -1, st);
+  hipError_t err = launch_spmm_rows(nullptr, n_hot, seg_ptr, seg_col, seg_val, X, partial, N, 0, -1, 0, st);
   if (err != hipSuccess) return err;
   err = launch_spmm_rows(nullptr, n_seg - n_hot, seg_ptr + n_hot, seg_col, seg_val, X, partial + (size_t)n_hot * N, N, 0,
-                         0, st);
+                         0, 0, st);
   if (err != hipSuccess) return err;
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
