@@ -48,6 +48,14 @@ template <int V> __device__ __forceinline__ void store_streaming(float *dst, con
 template <> __device__ __forceinline__ void store_streaming<1>(float *dst, const fvec<1> &v) {
   __builtin_nontemporal_store(v.v[0], dst);
 }
+// ... and input that is read once, whole cache lines per instruction, comes through a streaming load.
+__device__ __forceinline__ fvec<4> load_streaming4(const float *src) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const f4 x = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(src));
+  fvec<4> r;
+  r.v[0] = x[0]; r.v[1] = x[1]; r.v[2] = x[2]; r.v[3] = x[3];
+  return r;
+}
 
 // Consecutive workgroup ids land on different XCDs (each with its own 4 MB L2).  Work items
 // are cut into chunks of `bpc` consecutive items and chunk c goes to XCD c % 8, so that an
@@ -345,7 +353,7 @@ template <int LPR>
 __device__ __forceinline__ fvec<4> window_unit(const float *__restrict__ C, int first_row, int N, int c0,
                                                int n4, int u) {
   const int uu = u < n4 ? u : 0;
-  return *reinterpret_cast<const fvec<4> *>(C + (size_t)(first_row + uu / LPR) * N + c0 + (uu % LPR) * 4);
+  return load_streaming4(C + (size_t)(first_row + uu / LPR) * N + c0 + (uu % LPR) * 4);
 }
 
 template <int SW, int BLOCK, bool ACC>
@@ -505,11 +513,7 @@ __device__ __forceinline__ fvec<4> row_dot_quad_regs(const QuadEntries &first, c
 __device__ __forceinline__ fvec<4> window64_unit(const float *__restrict__ C, int first_row, int N, int c0, int n4,
                                                  int u) {
   const int uu = u < n4 ? u : 0;
-  typedef float f4 __attribute__((ext_vector_type(4)));
-  const f4 x = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(C + (size_t)(first_row + uu / 16) * N + c0 + (uu % 16) * 4));
-  fvec<4> r;
-  r.v[0] = x[0]; r.v[1] = x[1]; r.v[2] = x[2]; r.v[3] = x[3];
-  return r;
+  return load_streaming4(C + (size_t)(first_row + uu / 16) * N + c0 + (uu % 16) * 4);
 }
 
 template <bool ACC>
@@ -1283,7 +1287,7 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
     auto chunk_unit = [&](int ch) -> fvec<4> {
       const int q = min(ch / NKC, S - 1), k = min((ch % NKC) * kXChunk + sk, K - 4);
       const int row = t.prod_begin + min(q * kXRows + sr, P - 1);
-      return *reinterpret_cast<const fvec<4> *>(B + (size_t)row * K + k);
+      return load_streaming4(B + (size_t)row * K + k);
     };
     auto unit_or_zero = [&](const fvec<4> &x, int kc) -> fvec<4> {
       return kc * kXChunk + sk < K ? x : vzero<4>();
