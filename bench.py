@@ -217,9 +217,10 @@ def main():
     alg_bytes = w.algorithmic_bytes(cfg)
     gflops = flops / (ms_per_step * 1e-3) / 1e9
     achieved = alg_bytes / (dev_ms * 1e-3) / 1e9
-    # long rows: chunk kernel + sums, or (by column partition) values, hot segments, cold segments, group sums, row sums
+    # long rows: chunk kernel + sums, or (by column partition) hot segments, cold segments, group sums, row sums
+    # (the values of the uploaded matrix are put in segment order by one more kernel on the first call only)
     n_kernels = 1 + (1 if info["n_remainder_rows"] - info["n_long_rows"] > 0 else 0) + \
-        ((5 if info["long_row_hot_cols"] else 2) if info["n_long_rows"] else 0)
+        ((4 if info["long_row_hot_cols"] else 2) if info["n_long_rows"] else 0)
 
     check = None
     if not args.no_check:

@@ -418,6 +418,23 @@ def test_long_rows_by_column_partition(gpu, tf, orc, N):
     D.fill(float("nan"))
     tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(C2), D, S)
     assert orc.rel_err(D.to_numpy(), want2) <= TOL
+    first = D.to_numpy()
+    # the regrouped values of an uploaded matrix are kept by the schedule: the same call again, then
+    # the same schedule with another uploaded matrix of the same pattern, then the first one again
+    Ah.to_device()
+    for _ in range(2):
+        D.fill(float("nan"))
+        tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(C2), D, S)
+        assert np.array_equal(D.to_numpy(), first)
+    A3 = A.copy()
+    A3.data = rng.uniform(-1, 1, A.nnz).astype(np.float32)
+    A3h = tf.CsrMatrix.from_scipy(A3).to_device()
+    D.fill(float("nan"))
+    tf.spmm_spmm(A3h, Ah, tf.DenseMatrix.from_numpy(C2), D, S)
+    assert orc.rel_err(D.to_numpy(), oracle_spmm_spmm(orc, A3, A, C2)) <= TOL
+    D.fill(float("nan"))
+    tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(C2), D, S)
+    assert np.array_equal(D.to_numpy(), first)
 
 
 def test_gemm_spmm_reductions_and_accumulate(gpu, tf, orc):

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -17,6 +18,9 @@ struct tf_csr {
   int *p = nullptr, *i = nullptr;
   float *x = nullptr;
   bool owns = false;
+  // > 0 for an uploaded matrix: its device arrays never change, so work derived from its values
+  // (the regrouped values of column-partitioned long rows) is done once per schedule
+  unsigned long long serial = 0;
 };
 
 struct tf_dense {
@@ -44,6 +48,7 @@ struct DeviceSchedule {
   float *partial = nullptr;  // n_long_chunks (or segments) x N
   int *seg_ptr = nullptr, *ent_src = nullptr, *ent_pos = nullptr, *seg_col = nullptr, *lrow_seg = nullptr;  // column-partitioned long rows
   float *seg_val = nullptr;  // A's values in the order of the regrouped entries
+  unsigned long long seg_val_serial = 0;  // the uploaded matrix they were taken from (0: none)
   float *Bpad = nullptr;     // M x K' and K' x N copies of B and C, zero-padded, when K is not a multiple of 8
   float *Cpad = nullptr;
 };
@@ -195,11 +200,18 @@ static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int
     TF_HIP(launch_spmm_rows(s->rem_identity ? nullptr : d->rem_rows, (int)s->rem_rows.size(), A->p, A->i,
                             A->x, d->inter, D->d, N, accumulate, s->xcd_chunk_rows, /*streaming=*/1, st));
   }
-  if (s->long_part)
-    TF_HIP(launch_long_rows_partitioned(d->seg_ptr, d->seg_col, d->ent_src, d->ent_pos, d->seg_val, (int)s->seg_src.size(),
+  if (s->long_part) {
+    // The values in the order of the regrouped entries -- what the reference's reordered
+    // adjacency (createReorderedAdj, GCN_Single_Layer_SP_Demo_Utils.h:618-653) is to its
+    // executors -- are built on the first call with an uploaded matrix and kept; a wrapped
+    // matrix can change between calls, so its values are regrouped every time.
+    const bool have_values = A->serial != 0 && s->dev->seg_val_serial == A->serial;
+    TF_HIP(launch_long_rows_partitioned(d->seg_ptr, d->seg_col, d->ent_src, d->ent_pos, d->seg_val, have_values ? 0 : (int)s->seg_src.size(),
                                         8 * s->seg_per_xcd, (int)s->seg_ptr.size() - 1, d->seg_groups, (int)s->seg_groups.size(), d->long_rows,
                                         (int)s->long_rows.size(), d->lrow_seg, A->x, d->inter, d->partial, D->d, N,
                                         accumulate, st));
+    s->dev->seg_val_serial = A->serial;
+  }
   if (!s->long_chunks.empty())
     TF_HIP(launch_long_rows(d->long_chunks, (int)s->long_chunks.size(), d->long_rows,
                             (int)s->long_rows.size(), A->i, A->x, d->inter, d->partial, D->d, N,
@@ -307,6 +319,8 @@ extern "C" tf_status tf_csr_upload(int M, int N, const int *Ap, const int *Ai, c
   auto *a = new (std::nothrow) tf_csr();
   if (!a) return fail(TF_ENOMEM, "out of host memory");
   a->M = M; a->N = N; a->nnz = nnz; a->owns = true;
+  static std::atomic<unsigned long long> next_serial{1};
+  a->serial = next_serial.fetch_add(1);
   hipError_t e = hipMalloc(reinterpret_cast<void **>(&a->p), (size_t)(M + 1) * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&a->i), (size_t)std::max(nnz, 1) * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&a->x), (size_t)std::max(nnz, 1) * sizeof(float));
