@@ -183,7 +183,13 @@ typedef struct {
                             by column so that each XCD gathers from its own part of the most-read
                             intermediate rows, which then stays in its L2 (power-law graphs); -1 = cut
                             them into chunks of consecutive entries; 0 = the first when the long rows
-                            hold a million entries or more and the intermediate exceeds 64 MB      */
+                            hold a million entries or more and the intermediate exceeds 64 MB.
+                            With 1 the schedule keeps A's values in the regrouped order (what the
+                            reference's reordered adjacency, createReorderedAdj in
+                            fusion/gcn/SingleLayer/GCN_Single_Layer_SP_Demo_Utils.h:618-653, is to its
+                            executors): built on the first call with a matrix from tf_csr_upload, whose
+                            device arrays never change, and on every call with one from
+                            tf_csr_wrap_device, whose owner may change them between calls            */
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
