@@ -1656,10 +1656,10 @@ hipError_t launch_long_rows_partitioned(const int *seg_ptr, const int *seg_col, 
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
   }
-  hipError_t err = launch_spmm_rows(nullptr, n_hot, seg_ptr, seg_col, seg_val, X, partial, N, 0, -1, 0, st);
+  hipError_t err = launch_spmm_rows(nullptr, n_hot, seg_ptr, seg_col, seg_val, X, partial, N, 0, -1, 1, st);
   if (err != hipSuccess) return err;
   err = launch_spmm_rows(nullptr, n_seg - n_hot, seg_ptr + n_hot, seg_col, seg_val, X, partial + (size_t)n_hot * N, N, 0,
-                         0, 0, st);
+                         0, 1, st);
   if (err != hipSuccess) return err;
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
