@@ -62,7 +62,7 @@ hipError_t launch_fused_spmm_spmm_window(const TileDesc *, const int *, int, con
                                          int, int, hipStream_t);
 hipError_t launch_fused_spmm_spmm_window64(const TileDesc *, const int *, int, const int *, const int *,
                                            const float *, int, const float *, const int *, const int *,
-                                           const float *, int, float *, int, int, int, hipStream_t);
+                                           const float *, int, float *, int, int, int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
                             float *, int, int, int, int, hipStream_t);
 hipError_t launch_long_rows_partitioned(const int *, const int *, const int *, const int *, float *, int, int, int, const LongRow *, int, const LongRow *, int,
@@ -451,7 +451,7 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
     if (s->win_wide && A->nnz >= 4) {  // reads B's entries for the first product and A's for the second, in place
       TF_HIP(tf::launch_fused_spmm_spmm_window64(d->tiles, d->win, (int)s->launch_tiles.size(), B->p, B->i, B->x,
                                                  B->nnz, C->d, A->p, A->i, A->x, A->nnz, D->d, s->opts.N,
-                                                 s->lds_bytes, acc, st));
+                                                 s->lds_bytes, acc, s->opts.compute_units, st));
       return TF_OK;
     }
     if (same) {

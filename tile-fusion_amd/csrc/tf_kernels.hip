@@ -446,7 +446,7 @@ __global__ __launch_bounds__(BLOCK) void fused_spmm_spmm_window_kernel(
 // loads its four of every sixteen from the CSR arrays (the rest reach it through its quad),
 // one row ahead of the row it works on.  Same fma sequence per element as the kernels above.
 // ---------------------------------------------------------------------------------
-constexpr int kW64Strip = 64, kW64Block = 1024, kW64Units = 6;
+constexpr int kW64Strip = 64, kW64Block = 1024;
 typedef int int4u __attribute__((ext_vector_type(4), aligned(4)));
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
 
@@ -521,7 +521,7 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
     const TileDesc *__restrict__ tiles, const int2 *__restrict__ win, int n_tiles, int per_xcd,
     const int *__restrict__ Bp, const int *__restrict__ Bi, const float *__restrict__ Bx, int nnzB,
     const float *__restrict__ C, const int *__restrict__ Ap, const int *__restrict__ Ai,
-    const float *__restrict__ Ax, int nnzA, float *__restrict__ D, int N) {
+    const float *__restrict__ Ax, int nnzA, float *__restrict__ D, int N, int n_loaders) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int SW = kW64Strip, LPR = SW / 4, G = kW64Block / LPR, ROWB = SW * 4;
   const int tile = xcd_contiguous(blockIdx.x, per_xcd);
@@ -536,9 +536,19 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
   float *Tbuf = Cbuf + Wc * SW;
   const int tid = threadIdx.x, group = tid / LPR, glane = tid % LPR, q = glane & 3;
   const int n4 = Wc * LPR;
-  fvec<4> pre[kW64Units];
-#pragma unroll
-  for (int j = 0; j < kW64Units; ++j) pre[j] = window64_unit(C, w.x, N, 0, n4, tid + j * kW64Block);
+  // The window of C goes from global memory straight into LDS (no registers): one instruction of
+  // a wavefront moves 64 units of 16 bytes, i.e. four window rows, to consecutive LDS addresses.
+  const int wave = tid / 64, lane = tid % 64;
+  auto stage_window = [&](int c0, int first_wave, int n_waves) {
+    for (int u0 = (wave - first_wave) * 64; u0 < n4; u0 += n_waves * 64) {
+      const int u = u0 + lane;
+      if (u < n4)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void *)(C + (size_t)(w.x + u / 16) * N + c0 + (u % 16) * 4),
+            (__attribute__((address_space(3))) void *)(Cbuf + u0 * 4), 16, 0, 0);
+    }
+  };
+  stage_window(0, 0, kW64Block / 64);
   for (int i = tid; i <= P; i += kW64Block) rpB[i] = Bp[t.prod_begin + i];
   for (int i = tid; i <= R; i += kW64Block) rpA[i] = Ap[t.own_begin + i];
   // column c of B is row c - w.x of the window, column c of A row c - prod_begin of the slab
@@ -548,6 +558,7 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
   // (only the last tile of the matrix can come within a load of the end of the arrays)
   const bool near_end = Bp[t.prod_end] + 16 > nnzB || Ap[t.own_begin + R] + 16 > nnzA;
   auto products = [&](auto exact_tag, int c0) {
+    const bool more = c0 + SW < N;  // another strip follows: its window is fetched during the second product
     constexpr bool EXACT = decltype(exact_tag)::value;
     QuadEntries ea, eb;
     auto fetchB = [&](int r) {
@@ -564,7 +575,6 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
       e.kb = kb; e.ke = ke;
       return e;
     };
-    lds_barrier();
     // first product: slab rows 0 .. P-1, a lane group per row, the next row's entries on their way
     ea = fetchB(group);
     for (int r = group; r < P; r += 2 * G) {
@@ -577,42 +587,40 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
           row_dot_quad_regs<EXACT>(eb, Bi, Bx, eb.kb, eb.ke, nnzB, offB, cbase, q, vzero<4>());
     }
     lds_barrier();
-    // then the fused rows out of the slab
-    if (R > 0) ea = fetchA(group);
-    float *dst = D + (size_t)(t.own_begin + group) * N + c0 + glane * 4;
-    const size_t round_stride = (size_t)G * N;
-    for (int i = group; i < R; i += 2 * G) {
-      eb = fetchA(i + G);
-      {
-        fvec<4> acc = vzero<4>();
-        if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
-        store_streaming<4>(dst, row_dot_quad_regs<EXACT>(ea, Ai, Ax, ea.kb, ea.ke, nnzA, offA, tbase, q, acc));
-        dst += round_stride;
-      }
-      if (i + G >= R) break;
-      ea = fetchA(i + 2 * G);
-      {
-        fvec<4> acc = vzero<4>();
-        if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
-        store_streaming<4>(dst, row_dot_quad_regs<EXACT>(eb, Ai, Ax, eb.kb, eb.ke, nnzA, offA, tbase, q, acc));
-        dst += round_stride;
+    // then the fused rows out of the slab.  The window is free now: while another strip follows,
+    // the last n_loaders wavefronts fetch its window instead of taking rows (their loads would
+    // otherwise stand in front of every entry load of this product: loads return in order).
+    const int g2 = more ? G - n_loaders * (64 / LPR) : G;
+    if (more && group >= g2) {
+      stage_window(c0 + SW, kW64Block / 64 - n_loaders, n_loaders);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
+      if (R > 0) ea = fetchA(group);
+      float *dst = D + (size_t)(t.own_begin + group) * N + c0 + glane * 4;
+      const size_t round_stride = (size_t)g2 * N;
+      for (int i = group; i < R; i += 2 * g2) {
+        eb = fetchA(i + g2);
+        {
+          fvec<4> acc = vzero<4>();
+          if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
+          store_streaming<4>(dst, row_dot_quad_regs<EXACT>(ea, Ai, Ax, ea.kb, ea.ke, nnzA, offA, tbase, q, acc));
+          dst += round_stride;
+        }
+        if (i + g2 >= R) break;
+        ea = fetchA(i + 2 * g2);
+        {
+          fvec<4> acc = vzero<4>();
+          if constexpr (ACC) acc = *reinterpret_cast<const fvec<4> *>(dst);
+          store_streaming<4>(dst, row_dot_quad_regs<EXACT>(eb, Ai, Ax, eb.kb, eb.ke, nnzA, offA, tbase, q, acc));
+          dst += round_stride;
+        }
       }
     }
+    lds_barrier();  // slab consumed, next window (if any) in LDS
   };
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of the first window has landed
+  lds_barrier();                                    // ... and everybody's, and the row pointers
   for (int c0 = 0; c0 < N; c0 += SW) {
-    lds_barrier();  // previous strip fully consumed (and, first time, row pointers visible)
-    {
-      fvec<4> *cb = reinterpret_cast<fvec<4> *>(Cbuf);
-#pragma unroll
-      for (int j = 0; j < kW64Units; ++j)
-        if (tid + j * kW64Block < n4) cb[tid + j * kW64Block] = pre[j];
-      for (int u = tid + kW64Units * kW64Block; u < n4; u += kW64Block)  // windows beyond the prefetch capacity
-        cb[u] = window64_unit(C, w.x, N, c0, n4, u);
-    }
-    if (c0 + SW < N) {
-#pragma unroll
-      for (int j = 0; j < kW64Units; ++j) pre[j] = window64_unit(C, w.x, N, c0 + SW, n4, tid + j * kW64Block);
-    }
     if (near_end) products(std::true_type{}, c0);
     else products(std::false_type{}, c0);
   }
@@ -1591,8 +1599,11 @@ hipError_t launch_fused_spmm_spmm_window(const TileDesc *tiles, const int *win, 
 hipError_t launch_fused_spmm_spmm_window64(const TileDesc *tiles, const int *win, int n_tiles, const int *Bp,
                                            const int *Bi, const float *Bx, int nnzB, const float *C, const int *Ap,
                                            const int *Ai, const float *Ax, int nnzA, float *D, int N, int lds_bytes,
-                                           int accumulate, hipStream_t st) {
+                                           int accumulate, int compute_units, hipStream_t st) {
   if (n_tiles <= 0) return hipSuccess;
+  // wavefronts that fetch the next strip's window during the second product: two are enough for one
+  // more strip of one tile per compute unit, four keep up when tiles or strips queue
+  const int n_loaders = (n_tiles > compute_units || N > 2 * kW64Strip) ? 4 : 2;
   if (N % kW64Strip != 0 || nnzA < 4 || nnzB < 4 || nnzA >= (1 << 30) || nnzB >= (1 << 30)) return hipErrorInvalidValue;
   const int per = per_xcd_of(n_tiles);
   const int2 *w2 = reinterpret_cast<const int2 *>(win);
@@ -1601,7 +1612,7 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *tiles, const int *win
   err = allow_lds(fused_spmm_spmm_window64_kernel<ACC_>, lds_bytes);                                    \
   if (err == hipSuccess)                                                                                \
     hipLaunchKernelGGL((fused_spmm_spmm_window64_kernel<ACC_>), dim3(grid_of(n_tiles)), dim3(kW64Block), \
-                       lds_bytes, st, tiles, w2, n_tiles, per, Bp, Bi, Bx, nnzB, C, Ap, Ai, Ax, nnzA, D, N)
+                       lds_bytes, st, tiles, w2, n_tiles, per, Bp, Bi, Bx, nnzB, C, Ap, Ai, Ax, nnzA, D, N, n_loaders)
   if (accumulate) { CALL64(true); } else { CALL64(false); }
 #undef CALL64
   return err != hipSuccess ? err : hipGetLastError();
