@@ -510,12 +510,6 @@ __device__ __forceinline__ fvec<4> row_dot_quad_regs(const QuadEntries &first, c
   return acc;
 }
 
-__device__ __forceinline__ fvec<4> window64_unit(const float *__restrict__ C, int first_row, int N, int c0, int n4,
-                                                 int u) {
-  const int uu = u < n4 ? u : 0;
-  return load_streaming4(C + (size_t)(first_row + uu / 16) * N + c0 + (uu % 16) * 4);
-}
-
 template <bool ACC>
 __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
     const TileDesc *__restrict__ tiles, const int2 *__restrict__ win, int n_tiles, int per_xcd,
