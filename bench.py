@@ -2,17 +2,26 @@
 """Benchmark of the fused executors on one MI355X.
 
 One "step" is one pass of the hot path, D = A*(B*C), over one synthetic workload whose
-operands are already resident in HBM.  Default workload: the banded SpMM-SpMM
-configuration (65,536 rows, bandwidth 32, N = 128).  Prints ONE JSON line.
+operands are already resident in HBM.  With no flags the timed line is the largest
+single-GPU configuration, the power-law GeMM-SpMM (R-MAT, 2^21 nodes, K = N = 128), and the
+other four configurations are measured in the same process and reported under
+"per_config".  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {1..6}] [--unfused]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {1..6}] [--only] [--unfused]
 """
-import argparse
-import importlib
-import json
 import os
-import sys
-import time
+
+# the CPU leg follows the reference's protocol: threads pinned close together, no dynamic teams
+# (must be in the environment before an OpenMP runtime is loaded)
+os.environ.setdefault("OMP_PROC_BIND", "close")
+os.environ.setdefault("OMP_DYNAMIC", "FALSE")
+
+import argparse  # noqa: E402
+import gc  # noqa: E402
+import importlib  # noqa: E402
+import json  # noqa: E402
+import sys  # noqa: E402
+import time  # noqa: E402
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 for p in (ROOT, os.path.join(ROOT, "tests")):
@@ -23,53 +32,117 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 MFMA_FP32_PEAK_TF = 157.3  # MI355X dense fp32 MFMA, published
+LLC_BYTES = 256 << 20      # Infinity Cache
 METRIC = "fused GeMM-SpMM / SpMM-SpMM GFLOP/s and % HBM roofline, 1 MI355X vs CPU"
+HEADLINE = 4               # largest single-GPU configuration, the power-law target
 
 
-def cpu_baseline(cfg, budget_s=20.0):
-    """The reference's CPU executor on this box's host cores, on the same operands.
-    SpMM-SpMM: the reference's own AVX2 kernel compiled from its sources (oracle/_ref),
-    over schedules from the restated variable-tile inspector; GeMM-SpMM: the C restatement
-    (its GEMM is MKL in the reference).  Median of up to 7 trials per cache budget, best
-    budget kept (the reference's protocol), bounded by `budget_s` seconds."""
+def _usable_cores():
+    have = os.cpu_count() or 1
+    try:
+        have = min(have, len(os.sched_getaffinity(0)))
+    except (AttributeError, OSError):
+        pass
+    return have
+
+
+# taken before any OpenMP region runs: with OMP_PROC_BIND the runtime pins the calling thread to one
+# core, after which the affinity mask no longer shows what the process may use
+_USABLE_CORES = _usable_cores()
+
+
+def cpu_threads():
+    """Threads of the CPU leg: the cores this process may use.  The GPU boxes give a one-GPU job a
+    share of the host and export it as OMP_NUM_THREADS; without that, every core the OS shows."""
+    have = _USABLE_CORES
+    env = os.environ.get("OMP_NUM_THREADS", "")
+    limit = int(env.split(",")[0]) if env.split(",")[0].strip().isdigit() else 0
+    return (min(have, limit) if limit > 0 else have), have, limit
+
+
+def cpu_baseline(cfg, budget_s=25.0):
+    """The reference's CPU executors on this box's host cores, on the same operands, by the
+    reference's own protocol (scripts/run_exp.sh:133-158, scripts/plot.py:26-34): fused executor
+    over variable-tile schedules for its six cache budgets and over fixed tiles of 16..2048
+    rows, and the unfused pair of products; median of up to 7 trials each, best variant kept.
+    SpMM-SpMM runs the reference's own AVX2 translation units (oracle/_ref) where they were
+    built; GeMM-SpMM runs the C restatement, whose tile GEMM is a plain blocked fma loop where the
+    reference calls MKL's cblas_sgemm (not shipped here), so expect it to be several times
+    slower than the reference with MKL.  The whole leg is bounded by `budget_s` seconds: the trials
+    per variant shrink (never below one) when the budget runs short."""
     import oracle_lib as O
-    threads = min(os.cpu_count() or 1, O.max_threads(), 16)
+    threads, have, limit = cpu_threads()
+    threads = max(1, min(threads, O.max_threads()))
     A, N = cfg["A"], cfg["N"]
     flops = importlib.import_module("tile-fusion_amd").workloads.flops(cfg)
-    best, best_cache, trials_done = None, None, 0
+    gemm = cfg["op"] == "gemm_spmm"
+    use_ref = (not gemm) and O.ref() is not None and N % 32 == 0 and cfg["B"] is A
+    variants = [("variable tiles", c) for c in (500000, 1000000, 100000, 1500000, 60000, 1280000)]
+    variants += [("fixed tiles", ip) for ip in (512, 128, 2048, 32, 1024, 256, 64, 16)]
+    variants.insert(2, ("unfused", 0))
     t_start = time.perf_counter()
-    use_ref = cfg["op"] == "spmm_spmm" and O.ref() is not None and N % 32 == 0
-    for cache in (500000, 1000000, 100000, 1500000, 60000, 1280000):
-        if time.perf_counter() - t_start > budget_s:
+    results = []
+    t_trial = None
+
+    def make(kind, par):
+        if kind == "unfused":
+            return None
+        if kind == "variable tiles":
+            return O.inspect_vt_gemm_spmm(A, cfg["K"], N, par) if gemm else O.inspect_vt_both_wavefronts(A, N, par, threads)
+        return O.inspect_fixed_tiles(A, par, threads)
+
+    def run(kind, S):
+        t0 = time.perf_counter()
+        if kind == "unfused":
+            if gemm:
+                O.spmm(A, O.gemm(cfg["B"], cfg["C"], nthreads=threads), nthreads=threads)
+            elif use_ref:
+                O.ref_spmm(A, O.ref_spmm(cfg["B"], cfg["C"], threads), threads)
+            else:
+                O.spmm(A, O.spmm(cfg["B"], cfg["C"], nthreads=threads), nthreads=threads)
+        elif gemm:
+            O.gemm_spmm(A, cfg["B"], cfg["C"], S, nthreads=threads)
+        elif use_ref and kind == "fixed tiles":
+            O.spmm_spmm_separated(A, cfg["C"], S, nthreads=threads, impl="ref")
+        else:
+            O.spmm_spmm(A, cfg["B"], cfg["C"], S, nthreads=threads, impl="ref_vec32" if use_ref else "oracle")
+        return time.perf_counter() - t0
+
+    for vi, (kind, par) in enumerate(variants):
+        left = budget_s - (time.perf_counter() - t_start)
+        if left <= 0 and results:
             break
         try:
-            if cfg["op"] == "spmm_spmm":
-                S = O.inspect_vt_both_wavefronts(A, N, cache, threads)
-            else:
-                S = O.inspect_vt_gemm_spmm(A, cfg["K"], N, cache)
+            S = make(kind, par)
         except ValueError:
             continue
+        # trials this variant can have if the remaining ones are to get at least one each
+        n = 7 if t_trial is None else int(max(1, min(7, left / max(t_trial, 1e-6) / max(1, len(variants) - vi))))
         times = []
-        for _ in range(7):
-            t0 = time.perf_counter()
-            if cfg["op"] == "spmm_spmm":
-                O.spmm_spmm(A, cfg["B"], cfg["C"], S, nthreads=threads, impl="ref_vec32" if use_ref else "oracle")
-            else:
-                O.gemm_spmm(A, cfg["B"], cfg["C"], S, nthreads=threads)
-            times.append(time.perf_counter() - t0)
-            trials_done += 1
-            if time.perf_counter() - t_start > budget_s and len(times) >= 3:
+        for _ in range(n):
+            times.append(run(kind, S))
+            t_trial = times[-1] if t_trial is None else 0.5 * (t_trial + times[-1])
+            if time.perf_counter() - t_start > budget_s and len(times) >= 1:
                 break
-        med = float(np.median(times))
-        if best is None or med < best:
-            best, best_cache = med, cache
-    if best is None:
+        results.append((float(np.median(times)), kind, par, len(times)))
+    if not results:
         return None
-    return {"value": round(flops / best / 1e9, 2), "unit": "GFLOP/s", "cores": threads,
+    best = min(results)
+    fused = [r for r in results if r[1] != "unfused"]
+    unf = [r for r in results if r[1] == "unfused"]
+    return {"value": round(flops / best[0] / 1e9, 2), "unit": "GFLOP/s", "cores": threads,
             "kind": "reference" if use_ref else "port",
-            "sample": f"full workload incl. zeroing of D and the intermediate, median of <=7 trials per cache budget, "
-                      f"best budget {best_cache} B, {trials_done} trials in {time.perf_counter() - t_start:.1f} s",
-            "ms": round(best * 1e3, 3)}
+            "sample": f"full workload ({cfg['name']}) incl. zeroing of D and the intermediate; {len(results)} of {len(variants)} "
+                      f"variants of the reference's sweep, {sum(r[3] for r in results)} trials in {time.perf_counter() - t_start:.1f} s, median per variant",
+            "ms": round(best[0] * 1e3, 3),
+            "best_variant": f"{best[1]} {best[2]}" if best[1] != "unfused" else "unfused",
+            "best_fused_ms": round(min(fused)[0] * 1e3, 3) if fused else None,
+            "unfused_ms": round(unf[0][0] * 1e3, 3) if unf else None,
+            "os_cpu_count": os.cpu_count(), "usable_cores": have, "omp_num_threads_env": limit or None,
+            "omp_proc_bind": os.environ.get("OMP_PROC_BIND"), "omp_dynamic": os.environ.get("OMP_DYNAMIC"),
+            "note": ("the reference's own AVX2 kernels compiled from its sources" if use_ref else
+                     "C restatement of the reference executor; its tile GEMM stands in for MKL cblas_sgemm, which is not "
+                     "available here -- several times slower than MKL would be")}
 
 
 def calibrate(tf, rows=1 << 20, N=128, reps=5):
@@ -91,12 +164,141 @@ def calibrate(tf, rows=1 << 20, N=128, reps=5):
                       "copy_GBps_read_plus_write": round(2 * rows * N * 4 / dt / 1e9, 1)}))
 
 
+def check_result(cfg, got, max_rows=1 << 17):
+    """max |got - want| / max |want| against float64, on every row or -- for the configurations with
+    millions of rows -- on a fixed sample of rows that includes the longest ones."""
+    A = cfg["A"]
+    L = A.shape[0]
+    t = cfg["B"].astype(np.float64) @ cfg["C"].astype(np.float64)
+    if L <= max_rows:
+        rows = None
+        want = A.astype(np.float64) @ t
+    else:
+        rng = np.random.default_rng(1234)
+        longest = np.argsort(np.diff(A.indptr))[-64:]
+        rows = np.unique(np.concatenate([rng.choice(L, max_rows, replace=False), longest]))
+        want = A[rows].astype(np.float64) @ t
+        got = got[rows]
+    err = float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+    return err, (L if rows is None else int(rows.size))
+
+
+def kernel_names(info, op_is_gemm, unfused):
+    if unfused:
+        return "gemm_rows_kernel + spmm_rows_kernel"
+    if not op_is_gemm:
+        return ("fused_spmm_spmm_window64_kernel" if info["wide_strips"] else
+                "fused_spmm_spmm_window_kernel" if info["windowed"] else
+                "fused_spmm_spmm_kernel" if info["n_fused_rows"] else "spmm_rows_kernel (twice)")
+    if info["n_fused_rows"] == 0:
+        return "gemm_rows_kernel + spmm_rows_kernel" + (" (+ long-row segments)" if info["n_long_rows"] else "")
+    return "fused_gemm_spmm_stream_kernel" if info["streamed"] else "fused_gemm_spmm_kernel"
+
+
+def run_config(tf, cfg, idx, steps, warmup, args):
+    """Builds the schedule, times `steps` steps after `warmup`, checks the result."""
+    w = tf.workloads
+    A, N, K = cfg["A"], cfg["N"], cfg["K"]
+    gemm = cfg["op"] == "gemm_spmm"
+    op = tf.OP_GEMM_SPMM if gemm else tf.OP_SPMM_SPMM
+    Ah = tf.CsrMatrix.from_scipy(A).to_device()
+    t0 = time.perf_counter()
+    inner = Ah if (not gemm and cfg["B"] is A and not args.no_window) else None
+    S = tf.inspector(Ah, 1, op=op, N=N, K=K, lds_budget_bytes=args.lds, tile_rows=args.tile_rows,
+                     max_redundancy=args.max_redundancy, inner=inner, strip_cols=args.strip, wide_strips=args.wide,
+                     long_row_nnz=args.long_row, xcd_chunk_rows=args.xcd_chunk, long_row_partition=args.long_part)
+    inspect_s = time.perf_counter() - t0
+    S.validate()
+    info = S.info()
+    Cd = tf.DenseMatrix.from_numpy(cfg["C"])
+    D = tf.DenseMatrix(A.shape[0], N)
+    second = bool(args.second_stream)
+    if not gemm:
+        Bh = Ah if cfg["B"] is A else tf.CsrMatrix.from_scipy(cfg["B"]).to_device()
+        step = lambda st: tf.spmm_spmm(Ah, Bh, Cd, D, S, stream=st, second_stream=second)  # noqa: E731
+    else:
+        Bd = tf.DenseMatrix.from_numpy(cfg["B"])
+        step = lambda st: tf.gemm_spmm(Ah, Bd, Cd, D, S, stream=st, second_stream=second)  # noqa: E731
+        if args.unfused:  # the two products as separate launches, the intermediate through HBM
+            T = tf.DenseMatrix(A.shape[1], N)
+            step = lambda st: (tf.gemm(Bd, Cd, T, stream=st), tf.spmm(Ah, T, D, stream=st))  # noqa: E731
+
+    st = tf.Stream()
+    for _ in range(warmup):
+        step(st)
+    st.synchronize()
+    tf.device_synchronize()
+    e0, e1 = tf.Event(), tf.Event()
+    t0 = time.perf_counter()
+    e0.record(st)
+    for _ in range(steps):
+        step(st)
+    e1.record(st)
+    st.synchronize()
+    tf.device_synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = e0.elapsed_ms(e1) / steps   # HIP events on the launch stream
+    ms_per_step = wall * 1e3 / steps
+
+    # one more step with events around every launch
+    kernels = []
+    if not args.unfused:
+        S.set_profiling(True)
+        step(st)
+        kernels = [{"name": n, "ms": round(ms, 5)} for n, ms in S.profile()]
+        S.set_profiling(False)
+
+    err, rows_checked = (None, 0)
+    if not args.no_check:
+        err, rows_checked = check_result(cfg, D.to_numpy())
+        if not err <= 1e-4:
+            print(f"bench.py: result check failed on {cfg['name']}, rel err {err:.3e}", file=sys.stderr)
+            sys.exit(1)
+
+    flops = w.flops(cfg)
+    alg_bytes = w.algorithmic_bytes(cfg)
+    gemm_flops = 2.0 * A.shape[1] * K * N if gemm else 0.0
+    t_hbm = alg_bytes / (HBM_PEAK_GBS * 1e9)
+    t_mfma = gemm_flops / (MFMA_FP32_PEAK_TF * 1e12)
+    bound = "mfma" if t_mfma > t_hbm else "hbm"
+    dev_s = dev_ms * 1e-3
+    operand_bytes = alg_bytes + (4.0 * A.shape[1] * N if info["n_writeback_rows"] else 0.0)
+    res = {
+        "cfg": idx, "workload": cfg["name"], "op": cfg["op"], "rows": int(A.shape[0]), "nnz": int(A.nnz), "N": N, "K": K,
+        "ms_per_step": round(ms_per_step, 5), "kernel_ms": round(dev_ms, 5),
+        "gflops": round(flops / (ms_per_step * 1e-3) / 1e9, 2),
+        "bound": bound, "frac": round(max(t_hbm, t_mfma) / dev_s, 4),
+        "hbm_frac": round(t_hbm / dev_s, 4), "mfma_frac": round(t_mfma / dev_s, 4) if gemm else None,
+        "algorithmic_bytes": int(alg_bytes), "gemm_flops": int(gemm_flops), "flops": int(flops),
+        "working_set_vs_llc": round(operand_bytes / LLC_BYTES, 2),
+        "rel_err_vs_f64": err, "rows_checked": rows_checked,
+        "kernels": kernels, "kernel": kernel_names(info, gemm, args.unfused),
+        "schedule": {"lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "wide_strips": bool(info["wide_strips"]),
+                     "streamed": bool(info["streamed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
+                     "remainder_rows": info["n_remainder_rows"], "long_rows": info["n_long_rows"],
+                     "long_row_hot_cols": info["long_row_hot_cols"],
+                     "recomputed_rows": info["n_producer_rows"] - A.shape[1], "writeback_rows": info["n_writeback_rows"],
+                     "inspector_s": round(inspect_s, 4)},
+    }
+    try:  # measured HBM traffic of the step's kernels, if a committed profile covers this schedule
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            t = json.load(f).get(f"cfg{idx}")
+        if t and t["kernel"] == res["kernel"] and t["tiles"] == info["n_tiles"]:
+            res["traffic"] = t["fetch_bytes"] + t["write_bytes"]
+            res["traffic_source"] = t["source"]
+    except (OSError, ValueError, KeyError):
+        pass
+    return res, (Ah, S)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5, 6])
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=HEADLINE, choices=[1, 2, 3, 4, 5, 6],
+                    help="the configuration of the timed line (default: 4, the largest)")
+    ap.add_argument("--only", action="store_true", help="skip the per_config table of the other configurations")
     ap.add_argument("--lds", type=int, default=0, help="LDS budget per tile in bytes (0 = library default)")
     ap.add_argument("--tile-rows", type=int, default=0)
     ap.add_argument("--max-redundancy", type=float, default=0.0)
@@ -108,6 +310,7 @@ def main():
     ap.add_argument("--long-row", type=int, default=0, help="rows with more entries than this are chunked")
     ap.add_argument("--long-part", type=int, default=0, choices=[-1, 0, 1],
                     help="long rows: 1 = regrouped by the XCD partition of their columns, -1 = chunks of consecutive entries, 0 = library's choice")
+    ap.add_argument("--second-stream", action="store_true", help="hot long-row segments on the executor's second stream, beside the GEMM (TF_SECOND_STREAM)")
     ap.add_argument("--matrix", default=None, help="run on a .mtx / .smtx file instead of a synthetic configuration "
                     "(square; symmetric files are expanded), with --op, --N and --K")
     ap.add_argument("--op", default="spmm_spmm", choices=["spmm_spmm", "gemm_spmm"])
@@ -138,6 +341,7 @@ def main():
     if args.calibrate:
         calibrate(tf)
         return
+    custom = bool(args.matrix or args.scramble or args.rcm or args.unfused)
     if args.matrix:
         Af = tf.read_matrix(args.matrix)
         if Af.shape[0] != Af.shape[1]:
@@ -172,100 +376,46 @@ def main():
         cfg["A"] = A0
         if same_b:
             cfg["B"] = A0
-    A, N, K = cfg["A"], cfg["N"], cfg["K"]
-    op = tf.OP_GEMM_SPMM if cfg["op"] == "gemm_spmm" else tf.OP_SPMM_SPMM
 
-    Ah = tf.CsrMatrix.from_scipy(A).to_device()
-    t0 = time.perf_counter()
-    inner = Ah if (op == tf.OP_SPMM_SPMM and cfg["B"] is A and not args.no_window) else None
-    S = tf.inspector(Ah, 1, op=op, N=N, K=K, lds_budget_bytes=args.lds, tile_rows=args.tile_rows,
-                     max_redundancy=args.max_redundancy, inner=inner, strip_cols=args.strip, wide_strips=args.wide,
-                     long_row_nnz=args.long_row, xcd_chunk_rows=args.xcd_chunk, long_row_partition=args.long_part)
-    inspect_s = time.perf_counter() - t0
-    S.validate()
-    info = S.info()
-    Cd = tf.DenseMatrix.from_numpy(cfg["C"])
-    D = tf.DenseMatrix(A.shape[0], N)
-    if op == tf.OP_SPMM_SPMM:
-        Bh = Ah if cfg["B"] is A else tf.CsrMatrix.from_scipy(cfg["B"]).to_device()
-        step = lambda st: tf.spmm_spmm(Ah, Bh, Cd, D, S, stream=st)  # noqa: E731
-    else:
-        Bd = tf.DenseMatrix.from_numpy(cfg["B"])
-        step = lambda st: tf.gemm_spmm(Ah, Bd, Cd, D, S, stream=st)  # noqa: E731
-        if args.unfused:  # the two products as separate launches, the intermediate through HBM
-            T = tf.DenseMatrix(A.shape[1], N)
-            step = lambda st: (tf.gemm(Bd, Cd, T, stream=st), tf.spmm(Ah, T, D, stream=st))  # noqa: E731
+    # steps for the small configurations: enough launches for a stable mean
+    def steps_for(c):
+        return args.steps if c["A"].shape[0] >= 1 << 20 else max(args.steps, 200)
 
-    st = tf.Stream()
-    for _ in range(args.warmup):
-        step(st)
-    st.synchronize()
-    tf.device_synchronize()
-    e0, e1 = tf.Event(), tf.Event()
-    t0 = time.perf_counter()
-    e0.record(st)
-    for _ in range(args.steps):
-        step(st)
-    e1.record(st)
-    st.synchronize()
-    tf.device_synchronize()
-    wall = time.perf_counter() - t0
-    dev_ms = e0.elapsed_ms(e1) / args.steps   # HIP events on the launch stream
-    ms_per_step = wall * 1e3 / args.steps
-
-    flops = w.flops(cfg)
-    alg_bytes = w.algorithmic_bytes(cfg)
-    gflops = flops / (ms_per_step * 1e-3) / 1e9
-    achieved = alg_bytes / (dev_ms * 1e-3) / 1e9
-    # long rows: chunk kernel + sums, or (by column partition) hot segments, cold segments, group sums, row sums
-    # (the values of the uploaded matrix are put in segment order by one more kernel on the first call only)
-    n_kernels = 1 + (1 if info["n_remainder_rows"] - info["n_long_rows"] > 0 else 0) + \
-        ((4 if info["long_row_hot_cols"] else 2) if info["n_long_rows"] else 0)
-
-    check = None
-    if not args.no_check:
-        got = D.to_numpy()
-        if op == tf.OP_SPMM_SPMM:
-            t = cfg["B"].astype(np.float64) @ cfg["C"].astype(np.float64)
-        else:
-            t = cfg["B"].astype(np.float64) @ cfg["C"].astype(np.float64)
-        want = A.astype(np.float64) @ t
-        check = float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
-        if not check <= 1e-4:
-            print(f"bench.py: result check failed, rel err {check:.3e}", file=sys.stderr)
-            sys.exit(1)
-
+    head_steps = args.steps  # the timed line runs exactly the steps asked for
+    head, keep = run_config(tf, cfg, args.config, head_steps, args.warmup, args)
+    A = cfg["A"]
     out = {
-        "metric": METRIC, "value": round(gflops, 2), "unit": "GFLOP/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "metric": METRIC, "value": head["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
+        "steps": head_steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": cfg["name"], "op": cfg["op"], "rows": int(A.shape[0]), "nnz": int(A.nnz), "N": N, "K": K,
-                   "lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "wide_strips": bool(info["wide_strips"]), "long_row_hot_cols": info["long_row_hot_cols"], "streamed": bool(info["streamed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
-                   "remainder_rows": info["n_remainder_rows"], "recomputed_rows": info["n_producer_rows"] - A.shape[1],
-                   "writeback_rows": info["n_writeback_rows"], "kernels_per_step": n_kernels,
-                   "inspector_s": round(inspect_s, 4), **({"reorder_s": round(reorder_s, 4)} if reorder_s is not None else {}), "rel_err_vs_f64": check, "device": dev["arch"]},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "algorithmic_bytes": int(alg_bytes), "kernel_ms": round(dev_ms, 5),
-                     "kernel": ("fused_spmm_spmm_window64_kernel" if info["wide_strips"] else
-                                "fused_spmm_spmm_window_kernel" if info["windowed"] else
-                                "fused_spmm_spmm_kernel" if info["n_fused_rows"] else "spmm_rows_kernel (twice)")
-                     if op == tf.OP_SPMM_SPMM else ("gemm_rows_kernel + spmm_rows_kernel" if args.unfused or info["n_fused_rows"] == 0 else
-                                                    "fused_gemm_spmm_stream_kernel" if info["streamed"] else "fused_gemm_spmm_kernel"),
-                     "note": "kernel_ms = HIP-event time on the launch stream / steps (all kernels of a step)"},
+        "config": {"workload": cfg["name"], "op": cfg["op"], "rows": int(A.shape[0]), "nnz": int(A.nnz), "N": cfg["N"], "K": cfg["K"],
+                   **head["schedule"], "kernels_per_step": len(head["kernels"]) or None,
+                   "working_set_vs_llc": head["working_set_vs_llc"],
+                   **({"reorder_s": round(reorder_s, 4)} if reorder_s is not None else {}),
+                   "rel_err_vs_f64": head["rel_err_vs_f64"], "rows_checked": head["rows_checked"], "device": dev["arch"]},
     }
-    try:  # measured HBM traffic of the dominant kernel, if a committed profile covers this schedule
-        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            t = json.load(f).get(f"cfg{args.config}")
-        if t and t["kernel"] == out["roofline"]["kernel"] and t["tiles"] == info["n_tiles"]:
-            out["roofline"]["traffic"] = t["fetch_bytes"] + t["write_bytes"]
-            out["roofline"]["traffic_source"] = t["source"]
-    except (OSError, ValueError, KeyError):
-        pass
-    if op == tf.OP_GEMM_SPMM:
-        gemm_flops = 2.0 * A.shape[1] * K * N
-        out["roofline"]["mfma_frac_if_gemm_only"] = round(gemm_flops / (dev_ms * 1e-3) / 1e12 / MFMA_FP32_PEAK_TF, 4)
+    dev_s = head["kernel_ms"] * 1e-3
+    hbm = {"achieved": round(head["algorithmic_bytes"] / dev_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head["hbm_frac"]}
+    if head["bound"] == "mfma":
+        ach = head["gemm_flops"] / dev_s / 1e12
+        roof = {"bound": "mfma", "achieved": round(ach, 2), "peak": MFMA_FP32_PEAK_TF, "unit": "TFLOP/s", "frac": round(ach / MFMA_FP32_PEAK_TF, 4),
+                "hbm": hbm}
+    else:
+        roof = {"bound": "hbm", **hbm}
+    roof.update({"traffic": head.get("traffic"), "algorithmic_bytes": head["algorithmic_bytes"], "gemm_flops": head["gemm_flops"],
+                 "kernel_ms": head["kernel_ms"], "kernel": head["kernel"], "kernels": head["kernels"],
+                 "note": "a step is several launches: achieved = algorithmic work of the whole step / HIP-event time of the step on the "
+                         "launch stream; `kernels` = each launch timed by its own events in one extra step (launches on the "
+                         "executor's second stream run beside the others, so the list can add up to more than kernel_ms)"})
+    if "traffic_source" in head:
+        roof["traffic_source"] = head["traffic_source"]
+    out["roofline"] = roof
+
     if args.host_buffers:  # PCIe-inclusive: every operand crosses the bus each step
+        N = cfg["N"]
+        op = tf.OP_GEMM_SPMM if cfg["op"] == "gemm_spmm" else tf.OP_SPMM_SPMM
+        S = keep[1]
         reps = 5
         t0 = time.perf_counter()
         for _ in range(reps):
@@ -278,6 +428,22 @@ def main():
                 tf.gemm_spmm(Ah2, tf.DenseMatrix.from_numpy(cfg["B"]), Cd2, D2, S, accumulate=True)
             D2.to_numpy()
         out["host_buffer_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / reps, 3)
+    del keep
+    gc.collect()
+
+    if not custom and not args.only:  # the other configurations, same process, same protocol
+        per = []
+        for idx in (1, 2, 3, 4, 5):
+            if idx == args.config:
+                continue
+            c = w.make_config(idx)
+            r, keep = run_config(tf, c, idx, steps_for(c), args.warmup, args)
+            r.pop("schedule")
+            per.append(r)
+            del c, keep
+            gc.collect()
+        out["per_config"] = per
+    # last, because the OpenMP runtime pins this thread once its first region has run
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(out))

@@ -130,12 +130,17 @@ class FusedSchedule {
   // The schedule for this operation and these widths (built once, then cached).
   // inner_is_outer: SpMM-SpMM whose inner matrix B is A itself (every run of the reference,
   // fusion/example/SpMM_SpMM_Demo_Utils.h:53-54); lets the inspector build windowed tiles.
-  tf_schedule *get(int op, int N, int K, bool inner_is_outer = false) {
+  // The flat arrays above are those of the schedule an executor last used.
+  tf_schedule *get(int op, int N, int K, bool inner_is_outer = false) { return lookup(op, N, K, inner_is_outer, true); }
+
+ private:
+  tf_schedule *lookup(int op, int N, int K, bool inner_is_outer, bool expose) {
     if (!st_) throw std::runtime_error("FusedSchedule: empty schedule (call inspector first)");
     auto key = std::make_tuple(op, N, inner_is_outer ? -1 : K);
     auto it = st_->built.find(key);
     if (it == st_->built.end()) {
       tf_inspect_opts o = st_->base;
+      o.struct_size = sizeof(o);
       o.op = op; o.N = N; o.K = K;
       if (inner_is_outer && st_->L == st_->M) {
         o.inner_Ap = st_->Ap.data(); o.inner_Ai = st_->Ai.data(); o.inner_cols = st_->M;
@@ -144,19 +149,47 @@ class FusedSchedule {
       detail::check(tf_inspect(st_->L, st_->M, st_->Ap.data(), st_->Ai.data(), &o, &s), "inspector");
       it = st_->built.emplace(key, std::shared_ptr<tf_schedule>(s, tf_schedule_free)).first;
     }
-    tf_schedule_view v;
-    detail::check(tf_schedule_get_view(it->second.get(), &v), "FusedSchedule");
-    n1_ = v.n1; ptr1_ = v.ptr1; ptr2_ = v.ptr2; ker_begin_ = v.ker_begin; id_ = v.id; type_ = v.type;
+    if (expose) {
+      st_->last_used = it->second.get();
+      refresh();
+    }
     return it->second.get();
   }
-  // Exact check of the schedule for (op, N, K) against the pattern it was built from.
-  void validate(int op, int N, int K) {
-    tf_schedule *s = get(op, N, K);
-    detail::check(tf_schedule_validate(s, st_->L, st_->M, st_->Ap.data(), st_->Ai.data()), "FusedSchedule::validate");
+
+ public:
+  // Points n1_ ... type_ at the schedule an executor last used.  The executors receive the
+  // FusedSchedule by value (README.md:30-31), so the caller's own copy is brought up to date by
+  // this call; validate(), validateAll() and info() make it too.
+  void refresh() {
+    if (!st_ || !st_->last_used) return;
+    tf_schedule_view v;
+    detail::check(tf_schedule_get_view(st_->last_used, &v), "FusedSchedule");
+    n1_ = v.n1; ptr1_ = v.ptr1; ptr2_ = v.ptr2; ker_begin_ = v.ker_begin; id_ = v.id; type_ = v.type;
   }
-  tf_schedule_info info(int op, int N, int K) {
+  // Exact check of the schedule for (op, N, K) against the pattern it was built from.  Pass
+  // inner_is_outer = true for the schedule spMMSpMMExecutor uses when B is A (windowed tiles).
+  void validate(int op, int N, int K, bool inner_is_outer = false) {
+    tf_schedule *s = lookup(op, N, K, inner_is_outer, false);
+    const bool inner = inner_is_outer && st_->L == st_->M;
+    detail::check(tf_schedule_validate_inner(s, st_->L, st_->M, st_->Ap.data(), st_->Ai.data(), inner ? st_->Ap.data() : nullptr,
+                                             inner ? st_->Ai.data() : nullptr, inner ? st_->M : 0),
+                  "FusedSchedule::validate");
+    refresh();
+  }
+  // Checks every schedule built so far (the ones the executors have run).
+  void validateAll() {
+    for (auto &kv : st_->built) {
+      const bool inner = std::get<2>(kv.first) == -1 && st_->L == st_->M;
+      detail::check(tf_schedule_validate_inner(kv.second.get(), st_->L, st_->M, st_->Ap.data(), st_->Ai.data(),
+                                               inner ? st_->Ap.data() : nullptr, inner ? st_->Ai.data() : nullptr, inner ? st_->M : 0),
+                    "FusedSchedule::validateAll");
+    }
+    refresh();
+  }
+  tf_schedule_info info(int op, int N, int K, bool inner_is_outer = false) {
     tf_schedule_info i;
-    detail::check(tf_schedule_get_info(get(op, N, K), &i), "FusedSchedule::info");
+    detail::check(tf_schedule_get_info(lookup(op, N, K, inner_is_outer, false), &i), "FusedSchedule::info");
+    refresh();
     return i;
   }
 
@@ -166,6 +199,7 @@ class FusedSchedule {
     std::vector<int> Ap, Ai;
     tf_inspect_opts base{};
     std::map<std::tuple<int, int, int>, std::shared_ptr<tf_schedule>> built;
+    tf_schedule *last_used = nullptr;  // owned by `built`
   };
   std::shared_ptr<State> st_;
 };

@@ -84,6 +84,14 @@ tf_status tf_csr_upload(int M, int N, const int *Ap, const int *Ai, const float 
 /* Wraps CSR arrays that already live in device memory; nothing is copied or owned. */
 tf_status tf_csr_wrap_device(int M, int N, int nnz, const int *dAp, const int *dAi,
                              const float *dAx, tf_csr **out);
+/* 64-bit fingerprint of a sparsity pattern (row pointers and column indices, host arrays); never 0.
+ * tf_csr_upload and tf_inspect compute it, and the executors compare: a schedule is only run on
+ * operands with the pattern it was built from (TF_ESCHEDULE otherwise).  The reference has no
+ * such check: its executors trust whatever schedule they are handed. */
+uint64_t tf_pattern_hash(int M, const int *Ap, const int *Ai);
+/* A wrapped matrix has no host arrays to fingerprint, so its pattern is not checked unless the
+ * caller, who knows the host copy, provides the fingerprint here (0 = unknown again). */
+tf_status tf_csr_set_pattern_hash(tf_csr *a, uint64_t hash);
 void tf_csr_free(tf_csr *a);
 
 tf_status tf_dense_upload(int M, int N, const float *host, tf_dense **out);
@@ -133,8 +141,12 @@ tf_status tf_permute_csr(int M, const int *Ap, const int *Ai, const float *Ax, c
 
 enum { TF_OP_SPMM_SPMM = 0, TF_OP_GEMM_SPMM = 1 };
 
-/* Parameters of the gfx950 schedule.  Zero in any field means "default". */
+/* Parameters of the gfx950 schedule.  Zero in any field (but struct_size) means "default". */
 typedef struct {
+  size_t struct_size;    /* sizeof(tf_inspect_opts) as the caller was compiled; fields are only
+                            ever appended, so the library reads this many bytes and takes the
+                            defaults for fields a caller built against an older header does not
+                            have.  Must be set (TF_EINVAL when it is 0 or too small to hold N). */
   int op;                /* TF_OP_SPMM_SPMM or TF_OP_GEMM_SPMM                               */
   int N;                 /* columns of C and D (reference: bCols / EmbedDim)                 */
   int K;                 /* GeMM-SpMM: columns of dense B = rows of C (FeatureDim); else 0.
@@ -266,12 +278,24 @@ tf_status tf_schedule_get_view(const tf_schedule *s, tf_schedule_view *view);
  * naming the first violation.  (The reference never checks its schedules.) */
 tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, const int *Ap,
                                const int *Ai);
+/* The same, and for a schedule built with an inner pattern (tf_inspect_opts.inner_Ap) also
+ * what only that pattern shows: every windowed tile's window of C holds all rows its producer
+ * rows read, and window, slab and tables fit the LDS the kernel is launched with. */
+tf_status tf_schedule_validate_inner(const tf_schedule *s, int L, int M, const int *Ap, const int *Ai,
+                                     const int *inner_Ap, const int *inner_Ai, int inner_cols);
 
 /* ---- executors ---------------------------------------------------------------- */
 
 enum {
-  TF_ACCUMULATE = 1u /* D += A*(B*C), the reference's convention (its callers zero D
-                        first); without it D is overwritten and need not be initialised */
+  TF_ACCUMULATE = 1u,   /* D += A*(B*C), the reference's convention (its callers zero D
+                           first); without it D is overwritten and need not be initialised */
+  TF_SECOND_STREAM = 2u /* GeMM-SpMM with column-partitioned long rows: run the hot long-row segments
+                           on a second stream of the schedule's own (same priority), forked from and
+                           joined to the given one with events, beside the GEMM of the other rows.
+                           Without it every kernel of a call runs on the given stream, one after
+                           another -- which measured as fast on the R-MAT configuration (2.32 ms
+                           against 2.35 ms: the gathers and the GEMM's operand traffic meet in the
+                           same memory system), so it is not the default */
 };
 
 /* D = A * (B * C), A and B sparse.  Stands in for
@@ -297,6 +321,19 @@ tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, unsigned flag
 /* Y = X * W   (the cblas_sgemm call at fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:1144).
  * Needs K % 8 == 0, N % 32 == 0 and N <= 256 (TF_EUNSUPPORTED otherwise): it has no workspace to pad into. */
 tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, void *stream);
+
+/* Benchmark aid, no counterpart in the reference (its harness times whole executor calls):
+ * when switched on, the executors record events around every kernel launch of a call with this
+ * schedule; tf_schedule_get_profile waits for the last call and reports each launch's name and
+ * duration in ms (kernels that ran side by side on two streams each report their own). */
+#define TF_PROFILE_MAX 16
+typedef struct {
+  int n;
+  const char *name[TF_PROFILE_MAX];
+  float ms[TF_PROFILE_MAX];
+} tf_profile;
+tf_status tf_schedule_set_profiling(tf_schedule *s, int enable);
+tf_status tf_schedule_get_profile(tf_schedule *s, tf_profile *out);
 
 #ifdef __cplusplus
 }

@@ -39,7 +39,8 @@ int main() {
   std::vector<float> ones((size_t)M * N, 1.f), D((size_t)M * N, 0.f), t, want;
   def::Matrix C(M, N, ones.data()), Dm(M, N, D.data());
   fusion::spMMSpMMExecutor(A, A, C, Dm, sched, 8);
-  sched.validate(TF_OP_SPMM_SPMM, N, 0);
+  sched.validateAll();  // the schedule the executor just ran (built with B = A: windowed tiles)
+  sched.validate(TF_OP_SPMM_SPMM, N, 0, true);
   stencil(n, N, ones, t);
   stencil(n, N, t, want);
   for (size_t i = 0; i < D.size(); ++i)
@@ -55,6 +56,7 @@ int main() {
   A.toDevice(); B.toDevice(); W.toDevice(); D2m.toDevice();
   fusion::geMMSpMMExecutor(A, B, W, D2m, sched, 8);
   sched.validate(TF_OP_GEMM_SPMM, N, K);
+  sched.validateAll();
   D2m.toHost();
   stencil(n, N, kk, want);
   for (size_t i = 0; i < D2.size(); ++i)

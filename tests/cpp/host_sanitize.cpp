@@ -43,11 +43,11 @@ int main() {
   int bad = 0;
   std::vector<int> p, i;
   band(40000, 32, 16, 1, p, i);
-  { tf_inspect_opts o{}; o.op = TF_OP_SPMM_SPMM; o.N = 128; o.inner_Ap = p.data(); o.inner_Ai = i.data(); o.inner_cols = 40000; bad += run("band wide", 40000, p, i, o);
+  { tf_inspect_opts o{}; o.struct_size = sizeof(o); o.op = TF_OP_SPMM_SPMM; o.N = 128; o.inner_Ap = p.data(); o.inner_Ai = i.data(); o.inner_cols = 40000; bad += run("band wide", 40000, p, i, o);
     o.wide_strips = -1; bad += run("band narrow", 40000, p, i, o); o.inner_Ap = nullptr; o.inner_Ai = nullptr; o.wide_strips = 0; bad += run("band general", 40000, p, i, o);
-    tf_inspect_opts g{}; g.op = TF_OP_GEMM_SPMM; g.N = 128; g.K = 100; bad += run("band gemm stream", 40000, p, i, g); g.N = 64; g.K = 20; g.compute_units = 1024; bad += run("band gemm tiles", 40000, p, i, g); }
+    tf_inspect_opts g{}; g.struct_size = sizeof(g); g.op = TF_OP_GEMM_SPMM; g.N = 128; g.K = 100; bad += run("band gemm stream", 40000, p, i, g); g.N = 64; g.K = 20; g.compute_units = 1024; bad += run("band gemm tiles", 40000, p, i, g); }
   powerlaw(60000, 1500000, 2, p, i);
-  { tf_inspect_opts o{}; o.op = TF_OP_GEMM_SPMM; o.N = 128; o.K = 128; o.long_row_partition = 1; bad += run("powerlaw part", 60000, p, i, o);
+  { tf_inspect_opts o{}; o.struct_size = sizeof(o); o.op = TF_OP_GEMM_SPMM; o.N = 128; o.K = 128; o.long_row_partition = 1; bad += run("powerlaw part", 60000, p, i, o);
     o.long_row_partition = -1; bad += run("powerlaw chunks", 60000, p, i, o);
     o.op = TF_OP_SPMM_SPMM; o.K = 0; o.N = 20; o.long_row_partition = 1; bad += run("powerlaw spmm part", 60000, p, i, o); }
   { std::vector<int> perm(60000); tf_status rc = tf_reorder_rcm(60000, p.data(), i.data(), perm.data()); std::vector<float> x(i.size(), 1.f); int *bp, *bi; float *bx;

@@ -145,6 +145,15 @@ def spmm(A, X, nthreads=1):
     return out
 
 
+def ref_spmm(A, X, nthreads=1):
+    """Y = A*X by the reference's own spmmCsrParallel<float> (fusion/src/SpMM_SpMM.cpp:37-55)."""
+    M, N = A.shape[0], X.shape[1]
+    ap, ai, ax, x = _i(A.indptr), _i(A.indices), _f(A.data), _f(X)
+    out = np.zeros((M, N), np.float32)
+    ref().ref_spmm_csr_parallel(M, N, A.shape[1], pi(ap), pi(ai), pf(ax), pf(x), pf(out), nthreads)
+    return out
+
+
 def spmm_spmm(A, B, Cd, sched, nthreads=1, impl="oracle"):
     """D = A*(B*C) (README naming) over an interleaved schedule.  impl: 'oracle' |
     'ref_scalar' | 'ref_vec32' (the last two run the reference's compiled code)."""

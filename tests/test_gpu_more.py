@@ -1,0 +1,145 @@
+"""More parity cases on the GPU, through the C ABI: operands that arrive as files, schedules
+handed the wrong operands, the full-size GCN layer, launches timed one by one."""
+import numpy as np
+import pytest
+import scipy.io
+import scipy.sparse as sp
+
+from test_gpu_parity import TOL, oracle_spmm_spmm, say
+
+pytestmark = pytest.mark.gpu
+
+
+def test_matrix_files_through_both_executors(gpu, tf, orc, tmp_path):
+    """A symmetric MatrixMarket file (lower triangle stored, expanded as the reference's drivers
+    do with make_full) and a DLMC .smtx file (pattern only, every value 1) are read by
+    tf_read_matrix, run through both executors and compared with the oracle on the matrix that
+    scipy reads from the same file / that the file was written from."""
+    say("files: .mtx symmetric + .smtx -> HIP -> oracle")
+    n = 48
+    L = tf.workloads.laplacian_2d(n)                       # symmetric, 2304 rows
+    rng = np.random.default_rng(81)
+    L.data = L.data * rng.uniform(0.5, 1.5, L.nnz).astype(np.float32)
+    L = sp.csr_matrix((L + L.T) * 0.5, dtype=np.float32)   # symmetric values
+    mtx = tmp_path / "lap.mtx"
+    scipy.io.mmwrite(str(mtx), sp.tril(L).tocoo(), symmetry="symmetric", precision=9)
+    G = tf.workloads.banded_random(3000, 32, 12, seed=82)
+    smtx = tmp_path / "band.smtx"
+    with open(smtx, "w") as f:
+        f.write(f"{G.shape[0]}, {G.shape[1]}, {G.nnz}\n")
+        f.write(" ".join(map(str, G.indptr)) + "\n")
+        f.write(" ".join(map(str, G.indices)) + "\n")
+    want_mtx = sp.csr_matrix(scipy.io.mmread(str(mtx)), dtype=np.float32)
+    want_mtx.sort_indices()
+    want_smtx = sp.csr_matrix((np.ones(G.nnz, np.float32), G.indices, G.indptr), shape=G.shape)
+    for path, ref in ((mtx, want_mtx), (smtx, want_smtx)):
+        A = tf.read_matrix(path)
+        assert A.shape == ref.shape and np.array_equal(A.indptr, ref.indptr) and np.array_equal(A.indices, ref.indices)
+        assert np.array_equal(A.data, ref.data)
+        M = A.shape[0]
+        Ah = tf.CsrMatrix.from_scipy(A)
+        # SpMM-SpMM, bit for bit
+        Cd = tf.workloads.uniform((M, 64), 83)
+        S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah)
+        S.validate()
+        D = tf.DenseMatrix(M, 64)
+        tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(Cd), D, S)
+        assert np.array_equal(D.to_numpy(), oracle_spmm_spmm(orc, ref, ref, Cd)), path
+        # GeMM-SpMM, 1e-4
+        B, W = tf.workloads.uniform((M, 40), 84), tf.workloads.uniform((40, 64), 85)
+        S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=64, K=40)
+        S.validate()
+        D = tf.DenseMatrix(M, 64)
+        tf.gemm_spmm(Ah, tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W), D, S)
+        want, _ = orc.gemm_spmm(ref, B, W, orc.unfused_schedule(M))
+        assert orc.rel_err(D.to_numpy(), want) <= TOL, path
+
+
+def test_schedule_refuses_another_pattern(gpu, tf, orc):
+    """The windowed kernels turn B's columns into LDS offsets inside a tile's window, and every
+    kernel trusts the schedule's row lists: operands with the right shape and entry count but
+    another pattern are refused (TF_ESCHEDULE), for A and for B, on the wide and the lane-group
+    windowed kernels.  A wrapped matrix is checked once its owner provides the fingerprint."""
+    say("pattern fingerprints")
+    M, N = 4000, 128
+    A = tf.workloads.banded_random(M, 32, 16, seed=3)
+    X = tf.workloads.banded_random(M, 32, 16, seed=9)      # same shape, same nnz, other pattern
+    assert X.nnz == A.nnz
+    Ah, Xh = tf.CsrMatrix.from_scipy(A), tf.CsrMatrix.from_scipy(X)
+    Cd = tf.DenseMatrix.from_numpy(tf.workloads.uniform((M, N), 86))
+    D = tf.DenseMatrix(M, N)
+    for kw in (dict(), dict(wide_strips=-1, strip_cols=32)):
+        S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N, inner=Ah, **kw)
+        assert S.info()["windowed"] == 1
+        for a, b in ((Ah, Xh), (Xh, Ah), (Xh, Xh)):
+            with pytest.raises(tf.TileFusionError) as e:
+                tf.spmm_spmm(a, b, Cd, D, S)
+            assert e.value.status == -4 and "pattern" in str(e.value)
+        tf.spmm_spmm(Ah, Ah, Cd, D, S)                      # the right operands still run
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=64, K=64)
+    B = tf.DenseMatrix.from_numpy(tf.workloads.uniform((M, 64), 87))
+    W = tf.DenseMatrix.from_numpy(tf.workloads.uniform((64, 64), 88))
+    D = tf.DenseMatrix(M, 64)
+    with pytest.raises(tf.TileFusionError) as e:
+        tf.gemm_spmm(Xh, B, W, D, S)
+    assert e.value.status == -4
+
+
+def test_gcn_layer_full_size_all_ones_features(gpu, tf):
+    """The GCN-layer configuration at full size (200,000 nodes, K = 256, N = 128): with all-ones
+    features every row of the intermediate is the column sums of the weights, so
+    D = rowsum(A) * colsum(C)^T -- a check that needs no oracle run at this size."""
+    say("gemm_spmm GCN layer 200k nodes, B = ones")
+    cfg = tf.workloads.make_config(3)
+    A, W = cfg["A"], cfg["C"]
+    M, K, N = A.shape[0], cfg["K"], cfg["N"]
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=N, K=K)
+    S.validate()
+    B = tf.DenseMatrix(M, K); B.fill(1.0)
+    D = tf.DenseMatrix(M, N); D.fill(float("nan"))
+    tf.gemm_spmm(Ah, B, tf.DenseMatrix.from_numpy(W), D, S)
+    tf.device_synchronize()
+    want = np.asarray(A.astype(np.float64).sum(axis=1)) * W.astype(np.float64).sum(axis=0)[None, :]
+    got = D.to_numpy()
+    assert np.abs(got - want).max() / np.abs(want).max() <= TOL
+    # and with the configuration's own features, against fp64 on a sample of rows
+    D.fill(float("nan"))
+    tf.gemm_spmm(Ah, tf.DenseMatrix.from_numpy(cfg["B"]), tf.DenseMatrix.from_numpy(W), D, S)
+    rows = np.random.default_rng(89).choice(M, 4096, replace=False)
+    T = cfg["B"].astype(np.float64) @ W.astype(np.float64)
+    want = A[rows].astype(np.float64) @ T
+    assert np.abs(D.to_numpy()[rows] - want).max() / np.abs(want).max() <= TOL
+
+
+def test_launch_times_and_second_stream(gpu, tf, orc):
+    """tf_schedule_set_profiling: every launch of a call is timed; and a power-law product run
+    on one stream and with the hot segments on the executor's second stream (TF_SECOND_STREAM)
+    gives the same bits (the summation order is fixed by the schedule, not by timing)."""
+    say("per-launch times, second stream")
+    cfg = tf.workloads.make_config(4, 2.0 ** -5)
+    A, B, W = cfg["A"], cfg["B"], cfg["C"]
+    M = A.shape[0]
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1)
+    S.validate()
+    assert S.info()["long_row_hot_cols"] > 0
+    Bd, Wd = tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W)
+    D1, D2 = tf.DenseMatrix(M, 128), tf.DenseMatrix(M, 128)
+    S.set_profiling(True)
+    tf.gemm_spmm(Ah, Bd, Wd, D1, S)
+    prof1 = S.profile()
+    tf.gemm_spmm(Ah, Bd, Wd, D2, S, second_stream=True)
+    prof2 = S.profile()
+    S.set_profiling(False)
+    tf.device_synchronize()
+    assert len(prof1) >= 4 and all(ms > 0 for _, ms in prof1), prof1
+    assert any("hot long-row segments" in n for n, _ in prof2), prof2
+    assert any("hot rows" in n for n, _ in prof2), prof2
+    a, b = D1.to_numpy(), D2.to_numpy()
+    assert np.array_equal(a, b)
+    want, _ = orc.gemm_spmm(A, B, W, orc.unfused_schedule(M), nthreads=8)
+    assert orc.rel_err(a, want) <= TOL
+    for _ in range(3):                                       # replays keep giving the same bits
+        tf.gemm_spmm(Ah, Bd, Wd, D2, S)
+        assert np.array_equal(D2.to_numpy(), a)

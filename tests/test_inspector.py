@@ -319,3 +319,64 @@ def test_streamed_runs(tf):
         S4, view4, info4 = inspect(tf, A, op=tf.OP_GEMM_SPMM, N=N, K=K, compute_units=256)
         validate(view4, info4, A, 163840)
         assert info4["streamed"] == 1 and info4["n_fused_rows"] == M
+
+
+# ---- options struct, pattern fingerprint, inner-pattern check --------------------------------
+
+def test_opts_struct_size_is_honoured(tf):
+    """A caller compiled against an older, shorter tf_inspect_opts passes its own size: the
+    library reads only that many bytes and takes defaults for the rest; 0 is rejected."""
+    import ctypes as C
+    from importlib import import_module
+    b = import_module("tile-fusion_amd.binding")
+    A = tf.workloads.banded_random(2000, 32, 16, seed=3)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    full = b.InspectOpts(C.sizeof(b.InspectOpts), tf.OP_SPMM_SPMM, 64)
+    h = C.c_void_p()
+    assert b.lib().tf_inspect(A.shape[0], A.shape[1], Ah._pp, Ah._pi, C.byref(full), C.byref(h)) == 0
+    ref = b.FusedSchedule(h, Ah).info()
+    # the same options in a buffer that ends right after K, followed by garbage the library must not read
+    short_size = b.InspectOpts.K.offset + C.sizeof(C.c_int)
+    raw = (C.c_ubyte * C.sizeof(b.InspectOpts))(*([0xAB] * C.sizeof(b.InspectOpts)))
+    C.memmove(raw, C.byref(full), short_size)
+    C.cast(raw, C.POINTER(C.c_size_t))[0] = short_size
+    h2 = C.c_void_p()
+    assert b.lib().tf_inspect(A.shape[0], A.shape[1], Ah._pp, Ah._pi, C.cast(raw, C.POINTER(b.InspectOpts)), C.byref(h2)) == 0
+    assert b.FusedSchedule(h2, Ah).info() == ref
+    zero = b.InspectOpts(0, tf.OP_SPMM_SPMM, 64)
+    h3 = C.c_void_p()
+    assert b.lib().tf_inspect(A.shape[0], A.shape[1], Ah._pp, Ah._pi, C.byref(zero), C.byref(h3)) == -1
+    assert b"struct_size" in b.lib().tf_last_error_string()
+
+
+def test_pattern_hash(tf):
+    A = tf.workloads.banded_random(1000, 32, 16, seed=3)
+    h = tf.pattern_hash(A)
+    assert h != 0 and h == tf.pattern_hash(A.copy()) == tf.pattern_hash(tf.CsrMatrix.from_scipy(A))
+    B = A.copy()
+    B.data[:] = 7.0                      # values do not enter
+    assert tf.pattern_hash(B) == h
+    B = A.copy()
+    B.indices[5], B.indices[6] = B.indices[6], B.indices[5]   # same entries of the row, other order
+    assert tf.pattern_hash(B) != h
+    B = tf.workloads.banded_random(1000, 32, 16, seed=4)       # same shape and entry count
+    assert B.nnz == A.nnz and tf.pattern_hash(B) != h
+    assert tf.pattern_hash(A[:999]) != h
+
+
+def test_validate_checks_windows_against_the_inner_pattern(tf):
+    A = tf.workloads.banded_random(4000, 32, 16, seed=3)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    for kw in (dict(), dict(wide_strips=-1, strip_cols=32)):
+        S = tf.inspector(Ah, op=tf.OP_SPMM_SPMM, N=128, inner=Ah, **kw)
+        assert S.info()["windowed"] == 1
+        S.validate()                       # windows hold every row of C the producer rows read
+        other = tf.CsrMatrix.from_scipy(tf.workloads.banded_random(4000, 32, 16, seed=9))
+        S._inner = other                   # same shape and entry count, another pattern
+        with pytest.raises(tf.TileFusionError) as e:
+            S.validate()
+        assert e.value.status == -4 and "inner pattern" in str(e.value)
+        S._inner = None
+        with pytest.raises(tf.TileFusionError) as e:
+            S.validate()
+        assert e.value.status == -1

@@ -9,6 +9,7 @@ The directory name is not a Python identifier; import it with
 from .binding import (  # noqa: F401
     TileFusionError, lib, lib_path, device_init, device_synchronize, CsrMatrix, DenseMatrix,
     FusedSchedule, inspector, spmm_spmm, gemm_spmm, spmm, gemm, Stream, Event,
-    OP_SPMM_SPMM, OP_GEMM_SPMM, ACCUMULATE, read_matrix, read_dense, reorder_rcm, permute_csr,
+    OP_SPMM_SPMM, OP_GEMM_SPMM, ACCUMULATE, SECOND_STREAM,
+    pattern_hash, read_matrix, read_dense, reorder_rcm, permute_csr,
 )
 from . import workloads  # noqa: F401

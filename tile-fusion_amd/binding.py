@@ -12,6 +12,7 @@ import numpy as np
 OP_SPMM_SPMM = 0
 OP_GEMM_SPMM = 1
 ACCUMULATE = 1
+SECOND_STREAM = 2
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -33,7 +34,7 @@ class DeviceInfo(C.Structure):
 
 
 class InspectOpts(C.Structure):
-    _fields_ = [("op", C.c_int), ("N", C.c_int), ("K", C.c_int), ("lds_budget_bytes", C.c_int),
+    _fields_ = [("struct_size", C.c_size_t), ("op", C.c_int), ("N", C.c_int), ("K", C.c_int), ("lds_budget_bytes", C.c_int),
                 ("tile_rows", C.c_int), ("max_redundancy", C.c_float), ("long_row_nnz", C.c_int),
                 ("compute_units", C.c_int), ("inner_Ap", C.POINTER(C.c_int)), ("inner_Ai", C.POINTER(C.c_int)),
                 ("inner_cols", C.c_int), ("strip_cols", C.c_int), ("xcd_chunk_rows", C.c_int), ("wide_strips", C.c_int), ("long_row_partition", C.c_int)]
@@ -58,6 +59,13 @@ class ScheduleView(C.Structure):
                 ("step_ptr", C.POINTER(C.c_int)), ("n_step_ptr", C.c_int)]
 
 
+PROFILE_MAX = 16
+
+
+class Profile(C.Structure):
+    _fields_ = [("n", C.c_int), ("name", C.c_char_p * PROFILE_MAX), ("ms", C.c_float * PROFILE_MAX)]
+
+
 _PI = C.POINTER(C.c_int)
 _PF = C.POINTER(C.c_float)
 _VP = C.c_void_p
@@ -78,6 +86,8 @@ SIGNATURES = {
     "tf_event_elapsed_ms": (C.c_int, [_VP, _VP, _PF]),
     "tf_csr_upload": (C.c_int, [C.c_int, C.c_int, _PI, _PI, _PF, C.POINTER(_VP)]),
     "tf_csr_wrap_device": (C.c_int, [C.c_int, C.c_int, C.c_int, _VP, _VP, _VP, C.POINTER(_VP)]),
+    "tf_pattern_hash": (C.c_uint64, [C.c_int, _PI, _PI]),
+    "tf_csr_set_pattern_hash": (C.c_int, [_VP, C.c_uint64]),
     "tf_csr_free": (None, [_VP]),
     "tf_dense_upload": (C.c_int, [C.c_int, C.c_int, _PF, C.POINTER(_VP)]),
     "tf_dense_alloc": (C.c_int, [C.c_int, C.c_int, C.POINTER(_VP)]),
@@ -97,6 +107,10 @@ SIGNATURES = {
     "tf_schedule_get_info": (C.c_int, [_VP, C.POINTER(ScheduleInfo)]),
     "tf_schedule_get_view": (C.c_int, [_VP, C.POINTER(ScheduleView)]),
     "tf_schedule_validate": (C.c_int, [_VP, C.c_int, C.c_int, _PI, _PI]),
+    "tf_schedule_validate_inner": (C.c_int, [_VP, C.c_int, C.c_int, _PI, _PI, _PI, _PI, C.c_int]),
+    "tf_schedule_set_profiling": (C.c_int, [_VP, C.c_int]),
+    "tf_schedule_get_profile": (C.c_int, [_VP, C.POINTER(Profile)]),
+
     "tf_spmm_spmm": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
     "tf_gemm_spmm": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
     "tf_spmm": (C.c_int, [_VP, _VP, _VP, C.c_uint, _VP]),
@@ -267,9 +281,10 @@ class FusedSchedule:
     """swiftware::def::FusedSchedule: owns the schedule; exposes the reference's flat
     arrays (n1_, ptr1_, ptr2_, ker_begin_, id_, type_) plus the tile ranges."""
 
-    def __init__(self, handle, A):
+    def __init__(self, handle, A, inner=None):
         self.h = handle
         self._A = A
+        self._inner = inner
 
     def info(self):
         s = ScheduleInfo()
@@ -291,8 +306,20 @@ class FusedSchedule:
                 "step_ptr": arr(v.step_ptr, v.n_step_ptr) if v.n_step_ptr else None}
 
     def validate(self, A=None):
+        """Exact check against the pattern (and the inner pattern, when the schedule was built with one)."""
         A = A or self._A
-        _check(lib().tf_schedule_validate(self.h, A.M, A.N, A._pp, A._pi))
+        B = self._inner
+        _check(lib().tf_schedule_validate_inner(self.h, A.M, A.N, A._pp, A._pi, B._pp if B is not None else None,
+                                                B._pi if B is not None else None, B.N if B is not None else 0))
+
+    def set_profiling(self, on=True):
+        _check(lib().tf_schedule_set_profiling(self.h, 1 if on else 0))
+
+    def profile(self):
+        """[(launch name, ms)] of the last executor call with this schedule (profiling switched on)."""
+        p = Profile()
+        _check(lib().tf_schedule_get_profile(self.h, C.byref(p)))
+        return [(p.name[i].decode(), float(p.ms[i])) for i in range(p.n)]
 
     def __del__(self):
         if getattr(self, "h", None):
@@ -309,26 +336,36 @@ def inspector(A, NumThreads=1, *, op, N, K=0, lds_budget_bytes=0, tile_rows=0, m
     sparse matrix B of an SpMM-SpMM (pass A itself when B is A, as in every run of the
     reference); with it the inspector can build windowed tiles."""
     del NumThreads
-    o = InspectOpts(op, N, K, lds_budget_bytes, tile_rows, max_redundancy, long_row_nnz, compute_units,
+    o = InspectOpts(C.sizeof(InspectOpts), op, N, K, lds_budget_bytes, tile_rows, max_redundancy, long_row_nnz, compute_units,
                     inner._pp if inner is not None else None, inner._pi if inner is not None else None,
                     inner.N if inner is not None else 0, strip_cols, xcd_chunk_rows, wide_strips, long_row_partition)
     h = _VP()
     _check(lib().tf_inspect(A.M, A.N, A._pp, A._pi, C.byref(o), C.byref(h)))
-    return FusedSchedule(h, A)
+    return FusedSchedule(h, A, inner)
 
 
-def spmm_spmm(A, B, Cm, D, schedule, NumThreads=1, *, accumulate=False, stream=None):
+def spmm_spmm(A, B, Cm, D, schedule, NumThreads=1, *, accumulate=False, stream=None, second_stream=False):
     """spMMSpMMExecutor(A, B, C, D, schedule, NumThreads) (README.md:30): D = A*(B*C)."""
     del NumThreads
     _check(lib().tf_spmm_spmm(A.to_device().h, B.to_device().h, Cm.h, D.h, schedule.h,
-                              ACCUMULATE if accumulate else 0, stream.h if stream else None))
+                              (ACCUMULATE if accumulate else 0) | (SECOND_STREAM if second_stream else 0),
+                              stream.h if stream else None))
 
 
-def gemm_spmm(A, B, Cm, D, schedule, NumThreads=1, *, accumulate=False, stream=None):
+def gemm_spmm(A, B, Cm, D, schedule, NumThreads=1, *, accumulate=False, stream=None, second_stream=False):
     """geMMSpMMExecutor(A, B, C, D, schedule, NumThreads) (README.md:31): D = A*(B*C)."""
     del NumThreads
     _check(lib().tf_gemm_spmm(A.to_device().h, B.h, Cm.h, D.h, schedule.h,
-                              ACCUMULATE if accumulate else 0, stream.h if stream else None))
+                              (ACCUMULATE if accumulate else 0) | (SECOND_STREAM if second_stream else 0),
+                              stream.h if stream else None))
+
+
+def pattern_hash(A):
+    """tf_pattern_hash of a scipy CSR matrix or a CsrMatrix."""
+    if isinstance(A, CsrMatrix):
+        return int(lib().tf_pattern_hash(A.M, A._pp, A._pi))
+    ap, ai = _as_i32(A.indptr), _as_i32(A.indices)
+    return int(lib().tf_pattern_hash(A.shape[0], ap.ctypes.data_as(_PI), ai.ctypes.data_as(_PI)))
 
 
 def spmm(A, X, Y, *, accumulate=False, stream=None):

@@ -21,6 +21,7 @@ struct tf_csr {
   // > 0 for an uploaded matrix: its device arrays never change, so work derived from its values
   // (the regrouped values of column-partitioned long rows) is done once per schedule
   unsigned long long serial = 0;
+  uint64_t hash = 0;  // tf_pattern_hash of the host arrays it was uploaded from (0: unknown, wrapped)
 };
 
 struct tf_dense {
@@ -51,6 +52,14 @@ struct DeviceSchedule {
   unsigned long long seg_val_serial = 0;  // the uploaded matrix they were taken from (0: none)
   float *Bpad = nullptr;     // M x K' and K' x N copies of B and C, zero-padded, when K is not a multiple of 8
   float *Cpad = nullptr;
+  // A second stream of the same priority for kernels that may run beside the caller's stream (the
+  // hot long-row segments beside the rest of the GEMM), with the events that fork it off and join it.
+  hipStream_t side = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+  // per-launch timing, when tf_schedule_set_profiling switched it on
+  int prof_n = 0;
+  const char *prof_name[TF_PROFILE_MAX] = {};
+  hipEvent_t prof_ev[TF_PROFILE_MAX][2] = {};
 };
 
 // launchers in tf_kernels.hip
@@ -65,9 +74,8 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *, const int *, int, c
                                            const float *, int, float *, int, int, int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
                             float *, int, int, int, int, hipStream_t);
-hipError_t launch_long_rows_partitioned(const int *, const int *, const int *, const int *, float *, int, int, int, const LongRow *, int, const LongRow *, int,
-                                        const int *, const float *, const float *, float *, float *, int, int,
-                                        hipStream_t);
+hipError_t launch_scatter_values(const int *, const int *, const float *, float *, int, hipStream_t);
+hipError_t launch_seg_reduce(const LongRow *, int, const int *, const float *, float *, int, int, hipStream_t);
 hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const int *, const float *,
                             const float *, float *, float *, int, int, hipStream_t);
 hipError_t launch_fused_gemm_spmm(const TileDesc *, int, const int *, const float *, const float *,
@@ -122,6 +130,12 @@ void release_device_schedule(DeviceSchedule *d) {
   (void)hipFree(d->seg_ptr); (void)hipFree(d->ent_src); (void)hipFree(d->ent_pos); (void)hipFree(d->seg_col); (void)hipFree(d->lrow_seg); (void)hipFree(d->seg_val);
   (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
   (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad);
+  if (d->side) (void)hipStreamDestroy(d->side);
+  if (d->fork) (void)hipEventDestroy(d->fork);
+  if (d->join) (void)hipEventDestroy(d->join);
+  for (auto &pair : d->prof_ev)
+    for (hipEvent_t e : pair)
+      if (e) (void)hipEventDestroy(e);
   delete d;
 }
 
@@ -184,38 +198,91 @@ static tf_status ensure_device(tf_schedule *s) {
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->partial), s->long_chunks.size() * (size_t)s->opts.N * sizeof(float));
     if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(partials)");
   }
+  if (!rc && s->long_part && s->plain_hot > 0) {
+    hipError_t e = hipStreamCreateWithFlags(&d->side, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&d->fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&d->join, hipEventDisableTiming);
+    if (e != hipSuccess) rc = hip_fail(e, "hipStreamCreate(side stream)");
+  }
   if (rc) { release_device_schedule(d); return rc; }
   s->dev = d;
   return TF_OK;
 }
 
+// Timing of one launch (or group of launches) of an executor call: events around it on its stream.
+static hipError_t prof_begin(tf_schedule *s, const char *name, hipStream_t st) {
+  DeviceSchedule *d = s->dev;
+  if (!s->profiling || d->prof_n >= TF_PROFILE_MAX) return hipSuccess;
+  const int n = d->prof_n;
+  for (int q = 0; q < 2; ++q)
+    if (!d->prof_ev[n][q]) {
+      hipError_t e = hipEventCreate(&d->prof_ev[n][q]);
+      if (e != hipSuccess) return e;
+    }
+  d->prof_name[n] = name;
+  return hipEventRecord(d->prof_ev[n][0], st);
+}
+static hipError_t prof_end(tf_schedule *s, hipStream_t st) {
+  DeviceSchedule *d = s->dev;
+  if (!s->profiling || d->prof_n >= TF_PROFILE_MAX) return hipSuccess;
+  return hipEventRecord(d->prof_ev[d->prof_n++][1], st);
+}
+#define TF_PHASE(sched, name, st, call)        \
+  do {                                         \
+    TF_HIP(tf::prof_begin(sched, name, st));   \
+    TF_HIP(call);                              \
+    TF_HIP(tf::prof_end(sched, st));           \
+  } while (0)
+
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Second-op rows that no tile fused: served from the intermediate in HBM.
-static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int accumulate, hipStream_t st) {
-  const DeviceSchedule *d = s->dev;
+// The hot segments of column-partitioned long rows: segments of partition p are worked on by the
+// workgroups that land on XCD p.  The values in the order of the regrouped entries -- what the
+// reference's reordered adjacency (createReorderedAdj, GCN_Single_Layer_SP_Demo_Utils.h:618-653)
+// is to its executors -- are built on the first call with an uploaded matrix and kept; a wrapped
+// matrix can change between calls, so its values are regrouped every time.
+static tf_status run_hot_segments(const tf_csr *A, tf_schedule *s, hipStream_t st) {
+  DeviceSchedule *d = s->dev;
+  const bool have_values = A->serial != 0 && d->seg_val_serial == A->serial;
+  if (!have_values)
+    TF_PHASE(s, "scatter_values_kernel", st, launch_scatter_values(d->ent_src, d->ent_pos, A->x, d->seg_val, (int)s->seg_src.size(), st));
+  d->seg_val_serial = A->serial;
+  TF_PHASE(s, "spmm_rows_kernel (hot long-row segments)", st,
+           launch_spmm_rows(nullptr, 8 * s->seg_per_xcd, d->seg_ptr, d->seg_col, d->seg_val, d->inter, d->partial, s->opts.N, 0, -1, 1, st));
+  return TF_OK;
+}
+
+// Second-op rows that no tile fused: served from the intermediate in HBM.  hot_on_side: the hot
+// long-row segments were launched on the side stream already and are joined here.
+static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int accumulate, bool hot_on_side, hipStream_t st) {
+  DeviceSchedule *d = s->dev;
   const int N = s->opts.N;
   if (!s->rem_rows.empty()) {
     // identity list: no indirection needed
-    TF_HIP(launch_spmm_rows(s->rem_identity ? nullptr : d->rem_rows, (int)s->rem_rows.size(), A->p, A->i,
-                            A->x, d->inter, D->d, N, accumulate, s->xcd_chunk_rows, /*streaming=*/1, st));
+    TF_PHASE(s, "spmm_rows_kernel (short remainder rows)", st,
+             launch_spmm_rows(s->rem_identity ? nullptr : d->rem_rows, (int)s->rem_rows.size(), A->p, A->i,
+                              A->x, d->inter, D->d, N, accumulate, s->xcd_chunk_rows, /*streaming=*/1, st));
   }
   if (s->long_part) {
-    // The values in the order of the regrouped entries -- what the reference's reordered
-    // adjacency (createReorderedAdj, GCN_Single_Layer_SP_Demo_Utils.h:618-653) is to its
-    // executors -- are built on the first call with an uploaded matrix and kept; a wrapped
-    // matrix can change between calls, so its values are regrouped every time.
-    const bool have_values = A->serial != 0 && s->dev->seg_val_serial == A->serial;
-    TF_HIP(launch_long_rows_partitioned(d->seg_ptr, d->seg_col, d->ent_src, d->ent_pos, d->seg_val, have_values ? 0 : (int)s->seg_src.size(),
-                                        8 * s->seg_per_xcd, (int)s->seg_ptr.size() - 1, d->seg_groups, (int)s->seg_groups.size(), d->long_rows,
-                                        (int)s->long_rows.size(), d->lrow_seg, A->x, d->inter, d->partial, D->d, N,
-                                        accumulate, st));
-    s->dev->seg_val_serial = A->serial;
+    const int n_hot = 8 * s->seg_per_xcd, n_seg = (int)s->seg_ptr.size() - 1;
+    if (!hot_on_side)
+      if (tf_status rc = run_hot_segments(A, s, st)) return rc;
+    TF_PHASE(s, "spmm_rows_kernel (cold long-row segments)", st,
+             launch_spmm_rows(nullptr, n_seg - n_hot, d->seg_ptr + n_hot, d->seg_col, d->seg_val, d->inter,
+                              d->partial + (size_t)n_hot * N, N, 0, 0, 1, st));
+    if (hot_on_side) TF_HIP(hipStreamWaitEvent(st, d->join, 0));
+    // groups of segments of the rows with many (into their own slots of `partial`), then the rows
+    if (!s->seg_groups.empty())
+      TF_PHASE(s, "long_seg_reduce_kernel (groups)", st,
+               launch_seg_reduce(d->seg_groups, (int)s->seg_groups.size(), d->lrow_seg, d->partial, d->partial, N, 0, st));
+    TF_PHASE(s, "long_seg_reduce_kernel (rows)", st,
+             launch_seg_reduce(d->long_rows, (int)s->long_rows.size(), d->lrow_seg, d->partial, D->d, N, accumulate, st));
   }
   if (!s->long_chunks.empty())
-    TF_HIP(launch_long_rows(d->long_chunks, (int)s->long_chunks.size(), d->long_rows,
-                            (int)s->long_rows.size(), A->i, A->x, d->inter, d->partial, D->d, N,
-                            accumulate, st));
+    TF_PHASE(s, "spmm_long_chunk_kernel + long_row_reduce_kernel", st,
+             launch_long_rows(d->long_chunks, (int)s->long_chunks.size(), d->long_rows,
+                              (int)s->long_rows.size(), A->i, A->x, d->inter, d->partial, D->d, N,
+                              accumulate, st));
   return TF_OK;
 }
 
@@ -321,6 +388,7 @@ extern "C" tf_status tf_csr_upload(int M, int N, const int *Ap, const int *Ai, c
   a->M = M; a->N = N; a->nnz = nnz; a->owns = true;
   static std::atomic<unsigned long long> next_serial{1};
   a->serial = next_serial.fetch_add(1);
+  a->hash = tf_pattern_hash(M, Ap, Ai);
   hipError_t e = hipMalloc(reinterpret_cast<void **>(&a->p), (size_t)(M + 1) * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&a->i), (size_t)std::max(nnz, 1) * sizeof(int));
   if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&a->x), (size_t)std::max(nnz, 1) * sizeof(float));
@@ -343,6 +411,12 @@ extern "C" tf_status tf_csr_wrap_device(int M, int N, int nnz, const int *dAp, c
   a->M = M; a->N = N; a->nnz = nnz; a->owns = false;
   a->p = const_cast<int *>(dAp); a->i = const_cast<int *>(dAi); a->x = const_cast<float *>(dAx);
   *out = a;
+  return TF_OK;
+}
+
+extern "C" tf_status tf_csr_set_pattern_hash(tf_csr *a, uint64_t hash) {
+  if (!a) return fail(TF_EINVAL, "tf_csr_set_pattern_hash: null argument");
+  a->hash = hash;
   return TF_OK;
 }
 
@@ -424,6 +498,8 @@ static tf_status check_common(const char *who, const tf_csr *A, const tf_dense *
   if (A->M != s->L || A->N != s->M || A->nnz != s->nnz)
     return fail(TF_ESCHEDULE, "%s: schedule was built for a %d x %d pattern with %lld entries, A is %d x %d with %d",
                 who, s->L, s->M, s->nnz, A->M, A->N, A->nnz);
+  if (A->hash && A->hash != s->pattern_hash)
+    return fail(TF_ESCHEDULE, "%s: A has the shape and entry count the schedule was built for, but another sparsity pattern", who);
   if (C->N != s->opts.N || D->N != s->opts.N)
     return fail(TF_ESCHEDULE, "%s: schedule was built for N = %d, C has %d and D has %d columns", who, s->opts.N, C->N, D->N);
   if (D->M != A->M) return fail(TF_EINVAL, "%s: D has %d rows, A has %d", who, D->M, A->M);
@@ -441,37 +517,48 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
   if (rc) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
-  const tf::DeviceSchedule *d = s->dev;
+  tf::DeviceSchedule *d = s->dev;
+  d->prof_n = 0;
+  const int n_launch = (int)s->launch_tiles.size();
   if (s->windowed) {
     if (B->nnz != s->inner_nnz || B->N != s->opts.inner_cols)
       return fail(TF_ESCHEDULE, "tf_spmm_spmm: schedule was built for an inner pattern with %lld entries and %d columns, B has %d and %d",
                   s->inner_nnz, s->opts.inner_cols, B->nnz, B->N);
+    // the windowed kernels turn B's columns into LDS offsets inside the tile's window of C: another
+    // pattern would read outside it
+    if (B->hash && B->hash != s->inner_hash)
+      return fail(TF_ESCHEDULE, "tf_spmm_spmm: B has the shape and entry count of the inner pattern the schedule was built on, but another sparsity pattern");
     // The windowed kernel walks one staged CSR chunk for both products: B must be A.
     const bool same = (B == A) || (B->p == A->p && B->i == A->i && B->x == A->x);
     if (s->win_wide && A->nnz >= 4) {  // reads B's entries for the first product and A's for the second, in place
-      TF_HIP(tf::launch_fused_spmm_spmm_window64(d->tiles, d->win, (int)s->launch_tiles.size(), B->p, B->i, B->x,
-                                                 B->nnz, C->d, A->p, A->i, A->x, A->nnz, D->d, s->opts.N,
-                                                 s->lds_bytes, acc, s->opts.compute_units, st));
+      TF_PHASE(s, "fused_spmm_spmm_window64_kernel", st,
+               tf::launch_fused_spmm_spmm_window64(d->tiles, d->win, n_launch, B->p, B->i, B->x,
+                                                   B->nnz, C->d, A->p, A->i, A->x, A->nnz, D->d, s->opts.N,
+                                                   s->lds_bytes, acc, s->opts.compute_units, st));
       return TF_OK;
     }
     if (same) {
-      TF_HIP(tf::launch_fused_spmm_spmm_window(d->tiles, d->win, (int)s->launch_tiles.size(), d->fused_ids, A->p,
-                                               A->i, A->x, C->d, D->d, s->opts.N, s->opts.strip_cols,
-                                               s->lds_bytes, acc, st));
+      TF_PHASE(s, "fused_spmm_spmm_window_kernel", st,
+               tf::launch_fused_spmm_spmm_window(d->tiles, d->win, n_launch, d->fused_ids, A->p,
+                                                 A->i, A->x, C->d, D->d, s->opts.N, s->opts.strip_cols,
+                                                 s->lds_bytes, acc, st));
       return TF_OK;
     }
     if (s->lds_bytes_general > 163840)
       return fail(TF_ESCHEDULE, "tf_spmm_spmm: this schedule needs B to be the same matrix as A");
   }
-  TF_HIP(tf::launch_fused_spmm_spmm(d->tiles, (int)s->launch_tiles.size(), d->fused_ids, B->p, B->i, B->x,
-                                    C->d, A->p, A->i, A->x, D->d, d->inter, s->opts.N,
-                                    s->windowed ? s->lds_bytes_general : s->lds_bytes, acc, st));
+  if (n_launch > 0)
+    TF_PHASE(s, "fused_spmm_spmm_kernel", st,
+             tf::launch_fused_spmm_spmm(d->tiles, n_launch, d->fused_ids, B->p, B->i, B->x,
+                                        C->d, A->p, A->i, A->x, D->d, d->inter, s->opts.N,
+                                        s->windowed ? s->lds_bytes_general : s->lds_bytes, acc, st));
   if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
     const bool all = (int)s->plain_rows.size() == s->M;
-    TF_HIP(tf::launch_spmm_rows(all ? nullptr : d->plain_rows, (int)s->plain_rows.size(), B->p, B->i, B->x,
-                                C->d, d->inter, s->opts.N, 0, s->xcd_chunk_rows, tf::inter_streams(s), st));
+    TF_PHASE(s, "spmm_rows_kernel (intermediate rows)", st,
+             tf::launch_spmm_rows(all ? nullptr : d->plain_rows, (int)s->plain_rows.size(), B->p, B->i, B->x,
+                                  C->d, d->inter, s->opts.N, 0, s->xcd_chunk_rows, tf::inter_streams(s), st));
   }
-  return tf::run_remainder(A, D, s, acc, st);
+  return tf::run_remainder(A, D, s, acc, false, st);
 }
 
 extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf_dense *D,
@@ -486,28 +573,74 @@ extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_d
   if (rc) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
-  const tf::DeviceSchedule *d = s->dev;
+  tf::DeviceSchedule *d = s->dev;
+  d->prof_n = 0;
   const float *Bd = B->d, *Cd = C->d;
   if (s->user_K != s->opts.K) {  // zero-padded copies with K rounded up to 8 (the kernels' k step)
-    TF_HIP(tf::launch_pad(B->d, B->M, B->N, d->Bpad, B->M, s->opts.K, st));
-    TF_HIP(tf::launch_pad(C->d, C->M, C->N, d->Cpad, s->opts.K, C->N, st));
+    TF_PHASE(s, "pad_kernel (B)", st, tf::launch_pad(B->d, B->M, B->N, d->Bpad, B->M, s->opts.K, st));
+    TF_PHASE(s, "pad_kernel (C)", st, tf::launch_pad(C->d, C->M, C->N, d->Cpad, s->opts.K, C->N, st));
     Bd = d->Bpad;
     Cd = d->Cpad;
   }
-  if (s->gemm_stream)
-    TF_HIP(tf::launch_fused_gemm_spmm_stream(d->tiles, (int)s->launch_tiles.size(), d->step_begin, d->step_ptr,
-                                             d->fused_rec, Bd, Cd, s->opts.K, s->opts.N, s->ring_rows,
-                                             A->i, A->x, D->d, d->inter, s->lds_bytes, acc, st));
-  else
-    TF_HIP(tf::launch_fused_gemm_spmm(d->tiles, (int)s->launch_tiles.size(), d->fused_ids, Bd, Cd,
-                                      s->opts.K, s->gemm_kc, A->p, A->i, A->x, D->d, d->inter,
-                                      s->opts.N, s->lds_bytes, acc, s->opts.compute_units, s->gemm_regw ? 1 : 0, st));
-  if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
-    const bool all = (int)s->plain_rows.size() == s->M;
-    TF_HIP(tf::launch_gemm(Bd, Cd, d->inter, all ? nullptr : d->plain_rows, (int)s->plain_rows.size(),
-                           s->opts.K, s->opts.N, s->opts.compute_units, st));
+  const int n_launch = (int)s->launch_tiles.size();
+  if (n_launch > 0) {
+    if (s->gemm_stream)
+      TF_PHASE(s, "fused_gemm_spmm_stream_kernel", st,
+               tf::launch_fused_gemm_spmm_stream(d->tiles, n_launch, d->step_begin, d->step_ptr,
+                                                 d->fused_rec, Bd, Cd, s->opts.K, s->opts.N, s->ring_rows,
+                                                 A->i, A->x, D->d, d->inter, s->lds_bytes, acc, st));
+    else
+      TF_PHASE(s, s->gemm_regw ? "fused_gemm_spmm_regw_kernel" : "fused_gemm_spmm_kernel", st,
+               tf::launch_fused_gemm_spmm(d->tiles, n_launch, d->fused_ids, Bd, Cd,
+                                          s->opts.K, s->gemm_kc, A->p, A->i, A->x, D->d, d->inter,
+                                          s->opts.N, s->lds_bytes, acc, s->opts.compute_units, s->gemm_regw ? 1 : 0, st));
   }
-  return tf::run_remainder(A, D, s, acc, st);
+  // Column-partitioned long rows read the most-read ("hot") intermediate rows only through their
+  // hot segments.  Those rows are produced first; on request (TF_SECOND_STREAM) the hot segments
+  // then run on a second stream beside the rest of the GEMM and are joined before the rows' sums.
+  const bool overlap = d->side && s->plain_hot > 0 && (flags & TF_SECOND_STREAM);
+  if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
+    const int n_plain = (int)s->plain_rows.size();
+    const bool all = n_plain == s->M && s->plain_hot == 0;
+    if (overlap) {
+      TF_PHASE(s, "gemm_rows_kernel (hot rows)", st,
+               tf::launch_gemm(Bd, Cd, d->inter, d->plain_rows, s->plain_hot, s->opts.K, s->opts.N, s->opts.compute_units, st));
+      TF_HIP(hipEventRecord(d->fork, st));
+      TF_HIP(hipStreamWaitEvent(d->side, d->fork, 0));
+      if (tf_status rc2 = tf::run_hot_segments(A, s, d->side)) return rc2;
+      TF_HIP(hipEventRecord(d->join, d->side));
+      if (n_plain > s->plain_hot)
+        TF_PHASE(s, "gemm_rows_kernel (other rows)", st,
+                 tf::launch_gemm(Bd, Cd, d->inter, d->plain_rows + s->plain_hot, n_plain - s->plain_hot, s->opts.K, s->opts.N,
+                                 s->opts.compute_units, st));
+    } else {
+      TF_PHASE(s, "gemm_rows_kernel", st,
+               tf::launch_gemm(Bd, Cd, d->inter, all ? nullptr : d->plain_rows, n_plain, s->opts.K, s->opts.N, s->opts.compute_units, st));
+    }
+  }
+  return tf::run_remainder(A, D, s, acc, overlap && !s->plain_rows.empty(), st);
+}
+
+// ---- benchmark aid: per-launch times of the last executor call -------------------------
+
+extern "C" tf_status tf_schedule_set_profiling(tf_schedule *s, int enable) {
+  if (!s) return fail(TF_EINVAL, "tf_schedule_set_profiling: null argument");
+  s->profiling = enable != 0;
+  return TF_OK;
+}
+
+extern "C" tf_status tf_schedule_get_profile(tf_schedule *s, tf_profile *out) {
+  if (!s || !out) return fail(TF_EINVAL, "tf_schedule_get_profile: null argument");
+  std::memset(out, 0, sizeof(*out));
+  if (!s->dev || !s->profiling) return TF_OK;
+  tf::DeviceSchedule *d = s->dev;
+  for (int q = 0; q < d->prof_n; ++q) {
+    TF_HIP(hipEventSynchronize(d->prof_ev[q][1]));
+    TF_HIP(hipEventElapsedTime(&out->ms[q], d->prof_ev[q][0], d->prof_ev[q][1]));
+    out->name[q] = d->prof_name[q];
+  }
+  out->n = d->prof_n;
+  return TF_OK;
 }
 
 extern "C" tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, unsigned flags, void *stream) {

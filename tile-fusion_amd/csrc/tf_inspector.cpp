@@ -13,6 +13,7 @@
 #include <numeric>
 #include <climits>
 #include <cstdio>
+#include <cstddef>
 #include <cstring>
 
 #include "tf_internal.h"
@@ -25,6 +26,21 @@ int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 }  // namespace
 
+// Multiply-xorshift over the row pointers and column indices; 0 is kept for "unknown".
+extern "C" uint64_t tf_pattern_hash(int M, const int *Ap, const int *Ai) {
+  if (M <= 0 || !Ap) return 0;
+  uint64_t h = 0x9E3779B97F4A7C15ull ^ (uint64_t)(uint32_t)M;
+  auto mix = [&h](const int *p, long long n) {
+    for (long long k = 0; k < n; ++k) {
+      h = (h ^ (uint32_t)p[k]) * 0xD6E8FEB86659FD93ull;
+      h ^= h >> 32;
+    }
+  };
+  mix(Ap, (long long)M + 1);
+  if (Ai && Ap[M] > 0) mix(Ai, Ap[M]);
+  return h ? h : 1;
+}
+
 extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
                                 const tf_inspect_opts *user, tf_schedule **out) {
   if (!out) return tf::fail(TF_EINVAL, "tf_inspect: out is null");
@@ -36,7 +52,14 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   const long long nnz = Ap[L];
   if (nnz > 0 && !Ai) return tf::fail(TF_EINVAL, "tf_inspect: Ai is null");
 
-  tf_inspect_opts o = *user;
+  // Only the bytes the caller's header knew about are read; later fields keep their defaults.
+  if (user->struct_size < offsetof(tf_inspect_opts, K) || user->struct_size > 4096)
+    return tf::fail(TF_EINVAL, "tf_inspect: opts.struct_size is %zu: set it to sizeof(tf_inspect_opts)", user->struct_size);
+  tf_inspect_opts given{};
+  std::memcpy(&given, user, std::min(user->struct_size, sizeof(given)));
+  given.struct_size = sizeof(given);
+  user = &given;
+  tf_inspect_opts o = given;
   if (o.op != TF_OP_SPMM_SPMM && o.op != TF_OP_GEMM_SPMM)
     return tf::fail(TF_EINVAL, "tf_inspect: unknown op %d", o.op);
   if (o.N <= 0) return tf::fail(TF_EINVAL, "tf_inspect: N must be positive");
@@ -127,6 +150,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     S->L = L;
     S->M = M;
     S->nnz = nnz;
+    S->pattern_hash = tf_pattern_hash(L, Ap, Ai);
     S->gemm_kc = gemm_kc;
     S->user_K = user_K;
     S->gemm_regw = gemm_regw;
@@ -222,6 +246,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       }
       if (!(ok && L <= M)) return false;
       S->inner_nnz = Bp[M];
+      if (!S->inner_hash) S->inner_hash = (Bp == Ap && Bi == Ai && L == M) ? S->pattern_hash : tf_pattern_hash(M, Bp, Bi);
       S->tiles.swap(tiles);
       S->fused_ids.swap(ids);
       S->win.swap(win);
@@ -417,6 +442,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     // inside a group), and a group is worked on, like a short row, by the XCD of its partition;
     // entries outside all partitions ("cold") go to all XCDs as before.  Groups are cut into
     // segments of at most 64 entries; a row's segments are added up in a fixed order.
+    std::vector<signed char> part;  // per intermediate row: its hot partition, or -1 (empty without long_part)
     {
       long long long_nnz = 0;
       for (const auto &lr : S->long_rows) long_nnz += Ap[lr.row + 1] - Ap[lr.row];
@@ -437,7 +463,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         std::partial_sort(hot.begin(), hot.begin() + n_hot, hot.end(),
                           [&](int a, int b) { return reads[a] != reads[b] ? reads[a] > reads[b] : a < b; });
         hot.resize(n_hot);
-        std::vector<signed char> part(M, -1);
+        part.assign(M, -1);
         for (size_t h = 0; h < n_hot; ++h) {  // dealt in turn, snake-wise, so that the partitions' read counts match
           const int lap = (int)(h / kParts), pos = (int)(h % kParts);
           part[hot[h]] = (signed char)((lap & 1) ? kParts - 1 - pos : pos);
@@ -567,6 +593,14 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
           if (need[r]) S->plain_rows.push_back(r);
         S->n_writeback_rows += cnt;
       }
+    }
+    // With column-partitioned long rows the rows of the hot partitions come first in the list: the
+    // executor produces them first and starts the hot segments beside the rest of the GEMM.  (Only
+    // when every hot row is a plain row: a hot row stored by a fused tile is ready even earlier.)
+    if (S->long_part && o.op == TF_OP_GEMM_SPMM && !S->plain_rows.empty()) {
+      auto mid = std::stable_partition(S->plain_rows.begin(), S->plain_rows.end(), [&](int r) { return part[r] >= 0; });
+      S->plain_hot = (int)(mid - S->plain_rows.begin());
+      if (S->plain_hot == (int)S->plain_rows.size()) S->plain_hot = 0;  // nothing left to run beside them
     }
     S->slab_rows = slab_rows;
     S->lds_bytes_general = gemm_stream ? stream_fixed + ring_rows * (o.N + 4) * 4 : slab_rows * row_bytes + staging;
@@ -823,5 +857,35 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
   }
   for (int i = 0; i < L; ++i)
     if (done[i] != 1) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled %d times", i, done[i]);
+  return TF_OK;
+}
+
+// The same check, plus what only the inner pattern can show: that a windowed tile's window of C
+// holds every row its producer rows read, and that window, slab and tables fit the tile's LDS.
+extern "C" tf_status tf_schedule_validate_inner(const tf_schedule *s, int L, int M, const int *Ap, const int *Ai,
+                                                const int *inner_Ap, const int *inner_Ai, int inner_cols) {
+  if (tf_status rc = tf_schedule_validate(s, L, M, Ap, Ai)) return rc;
+  if (!s->windowed) return TF_OK;
+  if (!inner_Ap || (!inner_Ai && inner_Ap[M] > 0))
+    return tf::fail(TF_EINVAL, "tf_schedule_validate_inner: the schedule has windowed tiles; the inner pattern is needed");
+  if (inner_cols != s->opts.inner_cols || inner_Ap[M] != s->inner_nnz || tf_pattern_hash(M, inner_Ap, inner_Ai) != s->inner_hash)
+    return tf::fail(TF_ESCHEDULE, "the schedule's windows were built from another inner pattern");
+  if (s->win.size() != 2 * s->tiles.size()) return tf::fail(TF_ESCHEDULE, "windowed schedule: %zu windows for %zu tiles", s->win.size() / 2, s->tiles.size());
+  auto a16 = [](long long x) { return (x + 15) / 16 * 16; };
+  const int SW = s->opts.strip_cols;
+  for (size_t ti = 0; ti < s->tiles.size(); ++ti) {
+    const auto &t = s->tiles[ti];
+    const int w0 = s->win[2 * ti], w1 = s->win[2 * ti + 1];
+    if (w0 < 0 || w1 < w0 || w1 > inner_cols) return tf::fail(TF_ESCHEDULE, "tile %zu: bad window [%d,%d)", ti, w0, w1);
+    for (int r = t.prod_begin; r < t.prod_end; ++r)
+      for (int k = inner_Ap[r]; k < inner_Ap[r + 1]; ++k)
+        if (inner_Ai[k] < w0 || inner_Ai[k] >= w1)
+          return tf::fail(TF_ESCHEDULE, "tile %zu: producer row %d reads row %d of C outside the window [%d,%d)", ti, r, inner_Ai[k], w0, w1);
+    const long long P = t.prod_end - t.prod_begin, R = t.own_end - t.own_begin, nz = (long long)inner_Ap[t.prod_end] - inner_Ap[t.prod_begin];
+    const long long lds = s->win_wide ? a16(4 * (P + 1)) + a16(4 * (R + 1)) + 4LL * SW * (w1 - w0 + P)
+                                      : a16(4 * (P + 1)) + a16(4 * R) + a16(8 * (nz + 2 * P)) + 4LL * SW * (w1 - w0 + P);
+    if (lds > s->lds_bytes || lds > kMaxLds)
+      return tf::fail(TF_ESCHEDULE, "tile %zu: window, slab and tables take %lld bytes of LDS, the kernel is launched with %d", ti, lds, s->lds_bytes);
+  }
   return TF_OK;
 }

@@ -35,6 +35,16 @@ struct LongRow {
 
 struct DeviceSchedule;  // device copies + workspace, defined in tf_api.cpp
 
+// Marching runs: LDS layout and list format shared by the inspector, the validator and the kernel.
+constexpr int kMarchW = 8;               // entries per ELL row (longer rows do not march)
+constexpr int kMarchRowBytes = 256;      // an LDS slot: 64 columns of one row
+constexpr int kMarchTabBytes = 4096;     // per-iteration table of a run, staged at the start of LDS
+constexpr int kMarchMaxIter = kMarchTabBytes / 8 - 2;
+constexpr int kMarchZeroOff = kMarchTabBytes;                    // a row of zeros, read by padding entries
+constexpr int kMarchSlot0 = kMarchTabBytes + kMarchRowBytes;     // first slot
+constexpr int kMarchSrcA = 1 << 30;      // flag in march_ell_src: the value is one of A's (else of B's)
+constexpr int kMarchGroups = 64;         // lane groups (of 16 lanes) per workgroup
+
 }  // namespace tf
 
 struct tf_schedule {
@@ -65,6 +75,9 @@ struct tf_schedule {
   std::vector<tf::TileDesc> launch_tiles;  // the tiles that fuse something: one workgroup each
   std::vector<int> plain_rows;      // intermediate rows of tiles that fuse nothing, computed by the
                                     // row kernels -- only the rows some remainder row reads
+  int plain_hot = 0;                // with long_part: the first plain_hot of them are the rows of the hot
+                                    // partitions (produced first, so that the hot segments can start early)
+  bool profiling = false;           // executors record events around every launch
   std::vector<int> fused_ids;       // second-op rows per tile, tile after tile
   std::vector<int> rem_rows;        // remainder rows handled one row per lane group, ordered by
                                     // length class so that a workgroup's rows cost about the same
@@ -87,6 +100,28 @@ struct tf_schedule {
   std::vector<int> lrow_seg;      // per long row (first, count of tf::LongRow): the partial-sum slots it adds up, in order:
                                   // segments, or for a row of more than 32 segments groups of up to 32 of them
   std::vector<tf::LongRow> seg_groups;  // such groups: row = the group's slot (n_seg + its index), first/count into lrow_seg
+  // Marching runs (SpMM-SpMM on stencil-like patterns whose dependences no contiguous tile holds): a run
+  // is one workgroup that walks a sequence of steps (a column of grid points, plane by plane) and keeps
+  // the rows of C and of the intermediate that its next rows need in numbered LDS slots of one
+  // 64-column row each.  Iteration i of a run first has the C rows of load list i in LDS, then computes
+  // the ELL rows [row_ptr[i], row_ptr[i+1]): intermediate rows first needed by the run's step i (into
+  // slots; halo rows of neighbouring runs are recomputed), then the second-op rows of step i-1 (to D).
+  // Every entry of an ELL row names the LDS byte offset of the row it reads; the inspector assigns the
+  // slots so that a row stays until its last reader has run.
+  bool march = false;
+  int march_grid[3] = {0, 0, 0};     // the grid the runs were cut from (x fastest)
+  int march_tile[2] = {0, 0};        // grid points per run and plane: x, y
+  int march_slots = 0;               // LDS slots in use by the fullest run
+  int march_rpg = 0, march_lpg = 0;  // ELL rows / C rows a lane group handles per iteration, at most
+  std::vector<int> march_runs;       // (first iteration, iterations) per run
+  std::vector<int> march_row_ptr;    // [iterations + 1] into the ELL rows
+  std::vector<int> march_load_ptr;   // [iterations + 1] into the load list
+  std::vector<int> march_load;       // (row of C, LDS byte offset) pairs
+  std::vector<int> march_row_out;    // per ELL row: >= 0 row of D, < 0 ~(LDS byte offset) of an intermediate row
+  std::vector<int> march_row_id;     // per ELL row: the matrix row it computes (of B when out < 0, of A otherwise)
+  std::vector<int> march_ell_off;    // [kMarchW per ELL row] LDS byte offset of the row read (the zero row for padding)
+  std::vector<int> march_ell_src;    // ... and where its value comes from: index into B's values, or into A's
+                                     // with kMarchSrcA set; -1 for padding (value 0)
   long long fused_nnz = 0;
   int n_writeback_rows = 0;
   long long n_producer_rows = 0;
@@ -94,12 +129,19 @@ struct tf_schedule {
   std::vector<int> ptr1, ptr2, ker_begin, id, type, tile_range, writeback;
   // pattern fingerprint, checked by the executors against their operands
   long long nnz = 0;
+  uint64_t pattern_hash = 0;  // tf_pattern_hash of the pattern the schedule was built from
+  uint64_t inner_hash = 0;    // ... and of the inner pattern, when one was given (0: none)
   tf::DeviceSchedule *dev = nullptr;
 };
 
 namespace tf {
 
 tf_status fail(tf_status code, const char *fmt, ...);
+// tf_march.cpp: builds marching runs into S (returns false, S untouched, when the pattern does not
+// suit them), and checks such a schedule exactly against both patterns.
+bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int *Bp, const int *Bi,
+                 const tf_inspect_opts &o, const tf_inspect_opts &given);
+tf_status validate_march(const tf_schedule *s, int M, const int *Ap, const int *Ai, const int *Bp, const int *Bi);
 void release_device_schedule(DeviceSchedule *d);
 int default_compute_units();
 

@@ -97,9 +97,22 @@ tf_status read_banner(std::ifstream &f, const char *path, Banner *b, std::string
 
 }  // namespace
 
+static tf_status read_matrix_impl(const char *path, int *M, int *N, int *nnz, int **Ap, int **Ai, float **Ax);
+
+// No C++ exception leaves the C ABI: a malformed size line must not end the process.
 extern "C" tf_status tf_read_matrix(const char *path, int *M, int *N, int *nnz, int **Ap, int **Ai, float **Ax) {
   if (!path || !M || !N || !nnz || !Ap || !Ai || !Ax) return tf::fail(TF_EINVAL, "tf_read_matrix: null argument");
   *Ap = nullptr; *Ai = nullptr; *Ax = nullptr;
+  try {
+    return read_matrix_impl(path, M, N, nnz, Ap, Ai, Ax);
+  } catch (const std::bad_alloc &) {
+    return tf::fail(TF_ENOMEM, "%s: out of host memory", path);
+  } catch (const std::exception &e) {
+    return tf::fail(TF_EINVAL, "%s: %s", path, e.what());
+  }
+}
+
+static tf_status read_matrix_impl(const char *path, int *M, int *N, int *nnz, int **Ap, int **Ai, float **Ax) {
   const std::string p(path);
   std::ifstream f(path);
   if (!f.is_open()) return tf::fail(TF_EINVAL, "%s: cannot open", path);
@@ -117,7 +130,6 @@ extern "C" tf_status tf_read_matrix(const char *path, int *M, int *N, int *nnz, 
     for (auto &v : ptr)
       if (!(f >> v)) return tf::fail(TF_EINVAL, "%s: row pointers end early", path);
     if (ptr[0] != 0 || ptr[(size_t)rows] != n) return tf::fail(TF_EINVAL, "%s: row pointers do not span the entries", path);
-    t.reserve((size_t)n);
     for (long long i = 0; i < rows; ++i) {
       if (ptr[i + 1] < ptr[i]) return tf::fail(TF_EINVAL, "%s: row pointers decrease at row %lld", path, i);
       for (long long k = ptr[i]; k < ptr[i + 1]; ++k) {
@@ -139,8 +151,18 @@ extern "C" tf_status tf_read_matrix(const char *path, int *M, int *N, int *nnz, 
   else { ss >> rows >> cols; n = rows * cols; }
   if (rows < 0 || cols < 0 || n < 0 || rows > INT32_MAX || cols > INT32_MAX)
     return tf::fail(TF_EINVAL, "%s: bad size line", path);
+  // int32 indexing: a symmetric file may double its entries on expansion
+  if (b.coordinate && n > (b.sym ? INT32_MAX / 2 : INT32_MAX))
+    return tf::fail(TF_EUNSUPPORTED, "%s: %lld entries exceed int32 indexing", path, n);
   if (b.sym != 0 && rows != cols) return tf::fail(TF_EINVAL, "%s: a symmetric matrix must be square", path);
-  t.reserve((size_t)(b.sym ? 2 * n : n));
+  {  // an entry takes at least two bytes of the file, whatever the size line claims
+    const std::streampos here = f.tellg();
+    f.seekg(0, std::ios::end);
+    const long long left = (long long)(f.tellg() - here);
+    f.seekg(here);
+    const long long cap = std::max<long long>(left / 2 + 1, 0);
+    t.reserve((size_t)std::min<long long>(b.sym ? 2 * std::min(n, cap) : std::min(n, cap), (long long)INT32_MAX));
+  }
   if (b.coordinate) {
     for (long long k = 0; k < n; ++k) {
       long long r, c;

@@ -1646,37 +1646,27 @@ hipError_t launch_long_rows(const LongChunk *chunks, int n_chunks, const LongRow
   return hipGetLastError();
 }
 
-// Long rows regrouped by column partition: the hot segments (n_hot of them, an eighth per XCD, in
-// XCD order) run on the row kernel with one contiguous run of segments per XCD, the cold ones
-// round-robin; then every long row adds up its segments.
-hipError_t launch_long_rows_partitioned(const int *seg_ptr, const int *seg_col, const int *ent_src, const int *ent_pos,
-                                        float *seg_val, int n_entries, int n_hot, int n_seg, const LongRow *groups,
-                                        int n_groups, const LongRow *rows, int n_long, const int *seg_of,
-                                        const float *Ax, const float *X, float *partial, float *Y, int N,
-                                        int accumulate, hipStream_t st) {
-  if (n_long <= 0) return hipSuccess;
-  if (n_entries > 0) {
-    const int blocks = std::min((n_entries + kBlock - 1) / kBlock, 65536);
-    hipLaunchKernelGGL(scatter_values_kernel, dim3(blocks), dim3(kBlock), 0, st, ent_src, ent_pos, Ax, seg_val, n_entries);
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess) return err;
-  }
-  hipError_t err = launch_spmm_rows(nullptr, n_hot, seg_ptr, seg_col, seg_val, X, partial, N, 0, -1, 1, st);
-  if (err != hipSuccess) return err;
-  err = launch_spmm_rows(nullptr, n_seg - n_hot, seg_ptr + n_hot, seg_col, seg_val, X, partial + (size_t)n_hot * N, N, 0,
-                         0, 1, st);
-  if (err != hipSuccess) return err;
+// Long rows regrouped by column partition.  The executor runs the hot segments (an eighth per
+// XCD, in XCD order) on the row kernel with one contiguous run of segments per XCD and the cold
+// ones round-robin; these two put A's values into segment order and add up a row's segments.
+hipError_t launch_scatter_values(const int *ent_src, const int *ent_pos, const float *Ax, float *seg_val, int n_entries,
+                                 hipStream_t st) {
+  if (n_entries <= 0) return hipSuccess;
+  const int blocks = std::min((n_entries + kBlock - 1) / kBlock, 65536);
+  hipLaunchKernelGGL(scatter_values_kernel, dim3(blocks), dim3(kBlock), 0, st, ent_src, ent_pos, Ax, seg_val, n_entries);
+  return hipGetLastError();
+}
+
+// Y[rows[q].row] (+)= the sums in partial[seg_of[first .. first + count)], in that order (Y may be
+// `partial` itself for the groups of segments of rows with many).
+hipError_t launch_seg_reduce(const LongRow *rows, int n_rows, const int *seg_of, const float *partial, float *Y, int N,
+                             int accumulate, hipStream_t st) {
+  if (n_rows <= 0) return hipSuccess;
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
-  // groups of segments of the rows with many (into their own slots of `partial`), then the rows
-#define CALL(V_, L_)                                                                                      \
-  do {                                                                                                    \
-    if (n_groups > 0)                                                                                     \
-      hipLaunchKernelGGL((long_seg_reduce_kernel<V_, L_>), dim3((n_groups + G - 1) / G), dim3(kBlock), 0, st, groups, \
-                         n_groups, seg_of, partial, partial, N, 0);                                       \
-    hipLaunchKernelGGL((long_seg_reduce_kernel<V_, L_>), dim3((n_long + G - 1) / G), dim3(kBlock), 0, st, rows, n_long, \
-                       seg_of, partial, Y, N, accumulate);                                                \
-  } while (0)
+#define CALL(V_, L_)                                                                                                \
+  hipLaunchKernelGGL((long_seg_reduce_kernel<V_, L_>), dim3((n_rows + G - 1) / G), dim3(kBlock), 0, st, rows, n_rows, \
+                     seg_of, partial, Y, N, accumulate)
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
 #undef CALL
   return hipGetLastError();

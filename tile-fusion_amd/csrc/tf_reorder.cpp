@@ -4,7 +4,9 @@
 // (fusion/scripts/reorder_graphs.py:3,21-22) so that rows that depend on each other sit close
 // together and tiles fuse; this is the same step as a library call.  Host-only code.
 #include <algorithm>
+#include <climits>
 #include <cstdlib>
+#include <stdexcept>
 #include <numeric>
 #include <vector>
 
@@ -15,9 +17,11 @@ namespace {
 // Adjacency of A + A^T without the diagonal, as CSR (neighbours sorted by index).
 void symmetrise(int M, const int *Ap, const int *Ai, std::vector<int> *ptr, std::vector<int> *adj) {
   std::vector<int> cnt(M + 1, 0);
+  long long total = 0;
   for (int i = 0; i < M; ++i)
     for (int k = Ap[i]; k < Ap[i + 1]; ++k)
-      if (Ai[k] != i) { ++cnt[i + 1]; ++cnt[Ai[k] + 1]; }
+      if (Ai[k] != i) { ++cnt[i + 1]; ++cnt[Ai[k] + 1]; total += 2; }
+  if (total > INT_MAX) throw std::length_error("the symmetrised pattern exceeds int32 indexing");
   for (int i = 0; i < M; ++i) cnt[i + 1] += cnt[i];
   std::vector<int> raw(cnt[M]), pos(cnt.begin(), cnt.end() - 1);
   for (int i = 0; i < M; ++i)
@@ -111,6 +115,8 @@ extern "C" tf_status tf_reorder_rcm(int M, const int *Ap, const int *Ai, int *pe
     for (int i = 0; i < M; ++i) perm[i] = order[M - 1 - i];  // reversed
   } catch (const std::bad_alloc &) {
     return tf::fail(TF_ENOMEM, "tf_reorder_rcm: out of host memory");
+  } catch (const std::exception &e) {
+    return tf::fail(TF_EUNSUPPORTED, "tf_reorder_rcm: %s", e.what());
   }
   return TF_OK;
 }
@@ -127,6 +133,14 @@ extern "C" tf_status tf_permute_csr(int M, const int *Ap, const int *Ai, const f
   } catch (const std::bad_alloc &) {
     return tf::fail(TF_ENOMEM, "tf_permute_csr: out of host memory");
   }
+  std::vector<std::pair<int, float>> row;
+  try {  // room for the longest row now, so that nothing below allocates
+    int longest = 0;
+    for (int i = 0; i < M; ++i) longest = std::max(longest, Ap[i + 1] - Ap[i]);
+    row.reserve((size_t)std::max(longest, 0));
+  } catch (const std::exception &) {
+    return tf::fail(TF_ENOMEM, "tf_permute_csr: out of host memory");
+  }
   for (int i = 0; i < M; ++i) {
     if (perm[i] < 0 || perm[i] >= M || inv[perm[i]] >= 0) return tf::fail(TF_EINVAL, "tf_permute_csr: perm is not a permutation of 0..%d", M - 1);
     inv[perm[i]] = i;
@@ -139,7 +153,6 @@ extern "C" tf_status tf_permute_csr(int M, const int *Ap, const int *Ai, const f
     return tf::fail(TF_ENOMEM, "tf_permute_csr: out of host memory");
   }
   p[0] = 0;
-  std::vector<std::pair<int, float>> row;
   for (int i = 0; i < M; ++i) {  // new row i is old row perm[i], old column c becomes inv[c]
     const int o = perm[i];
     row.clear();

@@ -97,6 +97,9 @@ class _Adjacency:
             _b._check(_b.lib().tf_csr_wrap_device(self.shape[0], self.shape[1], int(self.Ap[-1]), _VP(crow.data_ptr()),
                                                  _VP(col.data_ptr()), _VP(val.data_ptr()), C.byref(h)))
             self.h = h
+            # the device arrays were copied from the same tensors as the host pattern: let the executors
+            # check schedules against it
+            _b._check(_b.lib().tf_csr_set_pattern_hash(h, _b.pattern_hash(self.host)))
 
     def schedule(self, K, N):
         key = (K, N)
@@ -134,7 +137,10 @@ _CACHE_SIZE = 32
 
 def _ctx(adj):
     crow, col, val = adj.crow_indices(), adj.col_indices(), adj.values()
-    key = (crow.data_ptr(), col.data_ptr(), val.data_ptr(), tuple(adj.shape), int(val.numel()), str(adj.device))
+    # the version counters change with every in-place update of the tensors: a cached host pattern,
+    # schedule or transpose is never used for values or indices that were changed afterwards
+    key = (crow.data_ptr(), col.data_ptr(), val.data_ptr(), tuple(adj.shape), int(val.numel()), str(adj.device),
+           crow._version, col._version, val._version)
     c = _cache.get(key)
     if c is None:
         c = _Adjacency(adj)

@@ -27,7 +27,9 @@ def laplacian_2d(nx, ny=None):
     ex, ey = np.ones(nx), np.ones(ny)
     tx = sp.diags([-ex[:-1], 2 * ex, -ex[:-1]], [-1, 0, 1])
     ty = sp.diags([-ey[:-1], 2 * ey, -ey[:-1]], [-1, 0, 1])
-    return _csr32(sp.kron(sp.identity(ny), tx) + sp.kron(ty, sp.identity(nx)))
+    m = sp.csr_matrix(sp.kron(sp.identity(ny), tx) + sp.kron(ty, sp.identity(nx)))
+    m.eliminate_zeros()  # (kron stores small dense factors as blocks, zeros included)
+    return _csr32(m)
 
 
 def laplacian_3d(n):
@@ -35,7 +37,9 @@ def laplacian_3d(n):
     e = np.ones(n)
     t = sp.diags([-e[:-1], 2 * e, -e[:-1]], [-1, 0, 1])
     i = sp.identity(n)
-    return _csr32(sp.kron(sp.kron(i, i), t) + sp.kron(sp.kron(i, t), i) + sp.kron(sp.kron(t, i), i))
+    m = sp.csr_matrix(sp.kron(sp.kron(i, i), t) + sp.kron(sp.kron(i, t), i) + sp.kron(sp.kron(t, i), i))
+    m.eliminate_zeros()
+    return _csr32(m)
 
 
 def banded_random(M, bandwidth=32, per_row=16, seed=3):
