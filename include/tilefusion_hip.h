@@ -322,6 +322,19 @@ tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, unsigned flag
  * Needs K % 8 == 0, N % 32 == 0 and N <= 256 (TF_EUNSUPPORTED otherwise): it has no workspace to pad into. */
 tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, void *stream);
 
+/* D = A * (B * C), A and B sparse, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  It needs no schedule and calls no hipMalloc / hipFree: the two products run as two
+ * row-kernel passes and the intermediate (B->M x C->N floats) lives in one fixed array of
+ * tf_noalloc_scratch_bytes() bytes (32 MiB) that every GPU the library is loaded on holds until the
+ * process ends; a larger intermediate is rejected with TF_EUNSUPPORTED.  All calls on one GPU
+ * share that array: calls that overlap in time on one GPU (two streams, two threads) race and
+ * give wrong results -- serialise them.  Nothing of an earlier call's contents is read.  Results
+ * equal the reference's fma order exactly (rows of any length are walked in CSR order). */
+tf_status tf_spmm_spmm_noalloc(const tf_csr *A, const tf_csr *B, const tf_dense *C, tf_dense *D,
+                               unsigned flags, void *stream);
+size_t tf_noalloc_scratch_bytes(void);
+
 /* Benchmark aid, no counterpart in the reference (its harness times whole executor calls):
  * when switched on, the executors record events around every kernel launch of a call with this
  * schedule; tf_schedule_get_profile waits for the last call and reports each launch's name and

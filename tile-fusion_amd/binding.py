@@ -110,7 +110,8 @@ SIGNATURES = {
     "tf_schedule_validate_inner": (C.c_int, [_VP, C.c_int, C.c_int, _PI, _PI, _PI, _PI, C.c_int]),
     "tf_schedule_set_profiling": (C.c_int, [_VP, C.c_int]),
     "tf_schedule_get_profile": (C.c_int, [_VP, C.POINTER(Profile)]),
-
+    "tf_spmm_spmm_noalloc": (C.c_int, [_VP, _VP, _VP, _VP, C.c_uint, _VP]),
+    "tf_noalloc_scratch_bytes": (C.c_size_t, []),
     "tf_spmm_spmm": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
     "tf_gemm_spmm": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
     "tf_spmm": (C.c_int, [_VP, _VP, _VP, C.c_uint, _VP]),
@@ -358,6 +359,18 @@ def gemm_spmm(A, B, Cm, D, schedule, NumThreads=1, *, accumulate=False, stream=N
     _check(lib().tf_gemm_spmm(A.to_device().h, B.h, Cm.h, D.h, schedule.h,
                               (ACCUMULATE if accumulate else 0) | (SECOND_STREAM if second_stream else 0),
                               stream.h if stream else None))
+
+
+def spmm_spmm_noalloc(A, B, Cm, D, *, accumulate=False, stream=None):
+    """D = A*(B*C) without a schedule and without any device allocation: the intermediate lives in
+    the library's fixed scratch array (see tf_spmm_spmm_noalloc).  A and B must be on the device."""
+    if A.h is None or B.h is None:
+        raise ValueError("spmm_spmm_noalloc: upload A and B first (to_device allocates)")
+    _check(lib().tf_spmm_spmm_noalloc(A.h, B.h, Cm.h, D.h, ACCUMULATE if accumulate else 0, stream.h if stream else None))
+
+
+def noalloc_scratch_bytes():
+    return int(lib().tf_noalloc_scratch_bytes())
 
 
 def pattern_hash(A):

@@ -290,6 +290,36 @@ static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int
 
 using tf::fail;
 
+// The fixed scratch array of tf_spmm_spmm_noalloc (further down) and its per-device address.
+namespace {
+
+constexpr size_t kScratchFloats = (size_t)8 << 20;  // 32 MiB: e.g. 65,536 intermediate rows of 128 columns
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+constexpr int kMaxDevices = 64;
+float *g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mu;
+
+// The device address of the current device's copy of `scratch`, looked up once per device.
+// (In host code the array's name is only a handle for this lookup, never an address.)
+tf_status scratch_of_current_device(float **out) {
+  int dev = 0;
+  TF_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(TF_EUNSUPPORTED, "device ordinal %d is beyond the %d this library keeps scratch addresses for", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    TF_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(TF_EHIP, "hipGetSymbolAddress returned a null address for the scratch array");
+    g_scratch_ptr[dev] = static_cast<float *>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return TF_OK;
+}
+
+}  // namespace
+
+
 // ---- errors, device, streams -----------------------------------------------------
 
 extern "C" const char *tf_last_error_string(void) { return tf::g_err; }
@@ -304,6 +334,10 @@ extern "C" tf_status tf_device_init(int device, tf_device_info *info) {
   }
   if (device < 0 || device >= count) return fail(TF_EINVAL, "device %d out of range (have %d)", device, count);
   TF_HIP(hipSetDevice(device));
+  {
+    float *unused = nullptr;
+    if (tf_status rc = scratch_of_current_device(&unused)) return rc;
+  }
   if (info) {
     hipDeviceProp_t p;
     TF_HIP(hipGetDeviceProperties(&p, device));
@@ -640,6 +674,36 @@ extern "C" tf_status tf_schedule_get_profile(tf_schedule *s, tf_profile *out) {
     out->name[q] = d->prof_name[q];
   }
   out->n = d->prof_n;
+  return TF_OK;
+}
+
+// ---- an executor that allocates nothing ----------------------------------------------------
+//
+// For callers that cannot call hipMalloc (code under HIP graph capture, serving loops, harnesses
+// that forbid it): D = A*(B*C) as two row-kernel passes with the intermediate in a fixed array in
+// device memory instead of a schedule's workspace.  Every GPU the library runs on holds its own
+// copy of the array from the moment the library is loaded there until the process ends.
+
+extern "C" size_t tf_noalloc_scratch_bytes(void) { return kScratchFloats * sizeof(float); }
+
+extern "C" tf_status tf_spmm_spmm_noalloc(const tf_csr *A, const tf_csr *B, const tf_dense *C, tf_dense *D,
+                                          unsigned flags, void *stream) {
+  if (!A || !B || !C || !D) return fail(TF_EINVAL, "tf_spmm_spmm_noalloc: null argument");
+  if (B->M != A->N) return fail(TF_EINVAL, "tf_spmm_spmm_noalloc: B has %d rows, A has %d columns", B->M, A->N);
+  if (C->M != B->N) return fail(TF_EINVAL, "tf_spmm_spmm_noalloc: C has %d rows, B has %d columns", C->M, B->N);
+  if (D->M != A->M || D->N != C->N)
+    return fail(TF_EINVAL, "tf_spmm_spmm_noalloc: D is %d x %d, A has %d rows and C has %d columns", D->M, D->N, A->M, C->N);
+  const size_t need = (size_t)B->M * C->N;
+  if (need > kScratchFloats)
+    return fail(TF_EUNSUPPORTED, "tf_spmm_spmm_noalloc: the intermediate (%d x %d floats, %zu bytes) exceeds the fixed scratch of %zu bytes; "
+                "use tf_spmm_spmm, whose schedule allocates its workspace", B->M, C->N, need * sizeof(float), kScratchFloats * sizeof(float));
+  float *T = nullptr;
+  if (tf_status rc = scratch_of_current_device(&T)) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // every intermediate row is overwritten (rows without entries with zeros), so nothing of the
+  // previous call's contents is read
+  TF_HIP(tf::launch_spmm_rows(nullptr, B->M, B->p, B->i, B->x, C->d, T, C->N, 0, 0, /*streaming=*/0, st));
+  TF_HIP(tf::launch_spmm_rows(nullptr, A->M, A->p, A->i, A->x, T, D->d, C->N, (flags & TF_ACCUMULATE) ? 1 : 0, 0, /*streaming=*/1, st));
   return TF_OK;
 }
 
