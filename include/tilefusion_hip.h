@@ -202,6 +202,22 @@ typedef struct {
                             executors): built on the first call with a matrix from tf_csr_upload, whose
                             device arrays never change, and on every call with one from
                             tf_csr_wrap_device, whose owner may change them between calls            */
+  /* SpMM-SpMM with an inner pattern, N a multiple of 64, rows of at most 8 entries: marching runs for
+     patterns whose dependences no range of consecutive rows holds (stencils on a 3D grid).  A run is a
+     column of march_tile_x x march_tile_y grid points that one workgroup walks plane by plane, keeping
+     the rows of C and of the intermediate that the coming planes need in LDS and recomputing the
+     intermediate's halo ring -- tiling with redundancy as in the reference's
+     fusion/src/SpMM_SpMM.cpp:984-1057, for rows that are not neighbours in memory.
+     march: 0 = where windowed tiles do not apply and a grid is known, 1 = the same (tf_inspect fails if
+     no marching schedule can be built), -1 = never.  grid_nx/ny/nz: the grid the rows are the points
+     of, x fastest (their product must be the row count); all 0 = found from the pattern when it is a
+     7-point-like stencil (row-to-column distances 1, nx, nx*ny).  The grid only deals rows to runs:
+     what a run loads, recomputes and keeps is derived from the patterns and checked by
+     tf_schedule_validate_inner, so a wrong grid cannot give wrong results.  march_tile_x/y: 0 = the
+     largest column whose rows fit LDS (8 x 8 on a 7-point stencil). */
+  int march;
+  int grid_nx, grid_ny, grid_nz;
+  int march_tile_x, march_tile_y;
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -240,6 +256,9 @@ typedef struct {
   int long_row_hot_cols; /* intermediate rows kept in the XCDs' L2 partitions for the long rows, else 0 */
   long long fused_nnz;   /* stored entries of A in fused rows (getFusedNnzNum)      */
   long long workspace_bytes; /* device memory the executor keeps (intermediate + partials) */
+  int marched;           /* 1 when the tiles are marching runs                       */
+  int march_tile_x, march_tile_y; /* grid points of a run per plane                    */
+  int march_slots;       /* LDS slots (64-column rows) the fullest run uses          */
 } tf_schedule_info;
 
 tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info *info);

@@ -52,6 +52,10 @@ struct DeviceSchedule {
   unsigned long long seg_val_serial = 0;  // the uploaded matrix they were taken from (0: none)
   float *Bpad = nullptr;     // M x K' and K' x N copies of B and C, zero-padded, when K is not a multiple of 8
   float *Cpad = nullptr;
+  // marching runs: the schedule's lists, and the ELL rows with the operands' values filled in
+  int *m_runs = nullptr, *m_row_ptr = nullptr, *m_load_ptr = nullptr, *m_load = nullptr, *m_row_out = nullptr;
+  int *m_ell_off = nullptr, *m_ell_src = nullptr, *m_ell = nullptr;
+  unsigned long long m_serial_a = 0, m_serial_b = 0;  // the uploaded matrices the values were taken from (0: none)
   // A second stream of the same priority for kernels that may run beside the caller's stream (the
   // hot long-row segments beside the rest of the GEMM), with the events that fork it off and join it.
   hipStream_t side = nullptr;
@@ -74,6 +78,9 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *, const int *, int, c
                                            const float *, int, float *, int, int, int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
                             float *, int, int, int, int, hipStream_t);
+hipError_t launch_march_fill(const int *, const int *, const float *, const float *, int *, size_t, hipStream_t);
+hipError_t launch_fused_spmm_spmm_march(const int *, int, const int *, const int *, const int *, const int *, const int *,
+                                        const float *, float *, int, int, int, int, int, int, hipStream_t);
 hipError_t launch_scatter_values(const int *, const int *, const float *, float *, int, hipStream_t);
 hipError_t launch_seg_reduce(const LongRow *, int, const int *, const float *, float *, int, int, hipStream_t);
 hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const int *, const float *,
@@ -130,6 +137,8 @@ void release_device_schedule(DeviceSchedule *d) {
   (void)hipFree(d->seg_ptr); (void)hipFree(d->ent_src); (void)hipFree(d->ent_pos); (void)hipFree(d->seg_col); (void)hipFree(d->lrow_seg); (void)hipFree(d->seg_val);
   (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
   (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad);
+  (void)hipFree(d->m_runs); (void)hipFree(d->m_row_ptr); (void)hipFree(d->m_load_ptr); (void)hipFree(d->m_load);
+  (void)hipFree(d->m_row_out); (void)hipFree(d->m_ell_off); (void)hipFree(d->m_ell_src); (void)hipFree(d->m_ell);
   if (d->side) (void)hipStreamDestroy(d->side);
   if (d->fork) (void)hipEventDestroy(d->fork);
   if (d->join) (void)hipEventDestroy(d->join);
@@ -161,7 +170,24 @@ static tf_status ensure_device(tf_schedule *s) {
   auto *d = new (std::nothrow) DeviceSchedule();
   if (!d) return fail(TF_ENOMEM, "out of host memory");
   d->device = dev;
-  tf_status rc = upload_vec(s->launch_tiles, &d->tiles);
+  tf_status rc = TF_OK;
+  if (s->march) {  // nothing but the run lists is needed on the device
+    rc = upload_vec(s->march_runs, &d->m_runs);
+    if (!rc) rc = upload_vec(s->march_row_ptr, &d->m_row_ptr);
+    if (!rc) rc = upload_vec(s->march_load_ptr, &d->m_load_ptr);
+    if (!rc) rc = upload_vec(s->march_load, &d->m_load);
+    if (!rc) rc = upload_vec(s->march_row_out, &d->m_row_out);
+    if (!rc) rc = upload_vec(s->march_ell_off, &d->m_ell_off);
+    if (!rc) rc = upload_vec(s->march_ell_src, &d->m_ell_src);
+    if (!rc) {
+      hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->m_ell), s->march_ell_off.size() * 2 * sizeof(int));
+      if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(ELL rows)");
+    }
+    if (rc) { release_device_schedule(d); return rc; }
+    s->dev = d;
+    return TF_OK;
+  }
+  rc = upload_vec(s->launch_tiles, &d->tiles);
   if (!rc) rc = upload_vec(s->fused_ids, &d->fused_ids);
   if (!rc) rc = upload_vec(s->win, &d->win);
   if (!rc) rc = upload_vec(s->rem_rows, &d->rem_rows);
@@ -554,6 +580,23 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
   tf::DeviceSchedule *d = s->dev;
   d->prof_n = 0;
   const int n_launch = (int)s->launch_tiles.size();
+  if (s->march) {
+    if (B->nnz != s->inner_nnz || B->N != s->opts.inner_cols || (B->hash && B->hash != s->inner_hash))
+      return fail(TF_ESCHEDULE, "tf_spmm_spmm: the schedule's runs were built on another inner pattern than B's");
+    // The values in the order of the runs' ELL rows (the reference's reordered adjacency,
+    // createReorderedAdj, GCN_Single_Layer_SP_Demo_Utils.h:618-653): filled in on the first call with
+    // uploaded matrices, whose device arrays never change, and on every call with wrapped ones.
+    const bool have = A->serial != 0 && B->serial != 0 && d->m_serial_a == A->serial && d->m_serial_b == B->serial;
+    if (!have)
+      TF_PHASE(s, "march_fill_kernel", st, tf::launch_march_fill(d->m_ell_off, d->m_ell_src, A->x, B->x, d->m_ell, s->march_ell_off.size(), st));
+    d->m_serial_a = A->serial;
+    d->m_serial_b = B->serial;
+    TF_PHASE(s, "fused_spmm_spmm_march_kernel", st,
+             tf::launch_fused_spmm_spmm_march(d->m_runs, (int)s->march_runs.size() / 2, d->m_row_ptr, d->m_load_ptr, d->m_load,
+                                              d->m_row_out, d->m_ell, C->d, D->d, s->opts.N, s->lds_bytes, s->march_tpg,
+                                              s->march_dpg, s->march_lpg, acc, st));
+    return TF_OK;
+  }
   if (s->windowed) {
     if (B->nnz != s->inner_nnz || B->N != s->opts.inner_cols)
       return fail(TF_ESCHEDULE, "tf_spmm_spmm: schedule was built for an inner pattern with %lld entries and %d columns, B has %d and %d",

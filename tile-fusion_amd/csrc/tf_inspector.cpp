@@ -283,6 +283,19 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     S->windowed = windowed;
     if (!windowed) S->opts.strip_cols = 0;
 
+    // ---- marching runs (stencils on 3D grids: no range of consecutive rows holds a row's dependences) ----
+    if (!windowed && have_inner && o.march >= 0) {
+      if (tf::build_march(S, M, Ap, Ai, o.inner_Ap, o.inner_Ai, o, given)) {
+        *out = S;
+        return TF_OK;
+      }
+      if (o.march > 0) {
+        delete S;
+        return tf::fail(TF_EUNSUPPORTED, "tf_inspect: no marching schedule for this pattern (needs a square matrix with at most 8 entries "
+                        "per row in both patterns, N a multiple of 64, a grid given or found, and a column of grid points whose rows fit LDS)");
+      }
+    }
+
     // A row whose own reach (itself plus its columns) exceeds the slab can never fuse.
     auto reach_lo = [&](int i) { return std::min(lo[i], std::min(i, M - 1)); };
     auto reach_hi = [&](int i) { return std::max(hi[i], std::min(i, M - 1) + 1); };
@@ -686,7 +699,12 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   info->strip_cols = s->windowed ? s->opts.strip_cols : 0;
   info->xcd_chunk_rows = s->xcd_chunk_rows;
   info->fused_nnz = s->fused_nnz;
+  info->marched = s->march ? 1 : 0;
+  info->march_tile_x = s->march_tile[0];
+  info->march_tile_y = s->march_tile[1];
+  info->march_slots = s->march_slots;
   long long ws = 0;
+  if (s->march) ws += (long long)s->march_ell_off.size() * 16;  // ELL rows with values, their offsets and sources
   if (s->n_writeback_rows > 0) ws += (long long)s->M * s->opts.N * 4;
   ws += (long long)s->long_chunks.size() * s->opts.N * 4;
   if (s->long_part) ws += ((long long)s->seg_ptr.size() - 1 + (long long)s->seg_groups.size()) * s->opts.N * 4 + (long long)s->seg_src.size() * 4;  // partial sums, regrouped values
@@ -716,6 +734,8 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
   if (L != s->L || M != s->M || Ap[L] != s->nnz)
     return tf::fail(TF_ESCHEDULE, "schedule was built for %d x %d with %lld entries, got %d x %d with %d",
                     s->L, s->M, s->nnz, L, M, Ap[L]);
+  if (s->march)
+    return tf::fail(TF_EINVAL, "tf_schedule_validate: marching runs are checked against both patterns: use tf_schedule_validate_inner");
   const int row_bytes = (s->slab_ld > 0 ? s->slab_ld : s->opts.N) * 4 + (s->gemm_regw ? 16 : 0);
   std::vector<int> owner(M, -1), done(L, 0);
   std::vector<char> stored(M, 0);
@@ -864,6 +884,14 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
 // holds every row its producer rows read, and that window, slab and tables fit the tile's LDS.
 extern "C" tf_status tf_schedule_validate_inner(const tf_schedule *s, int L, int M, const int *Ap, const int *Ai,
                                                 const int *inner_Ap, const int *inner_Ai, int inner_cols) {
+  if (s && s->march) {
+    if (!Ap || !inner_Ap || L != s->L || M != s->M || L != M || Ap[L] != s->nnz)
+      return tf::fail(TF_ESCHEDULE, "tf_schedule_validate_inner: the schedule's runs were built for other patterns");
+    if (inner_cols != s->opts.inner_cols || inner_Ap[M] != s->inner_nnz || tf_pattern_hash(M, inner_Ap, inner_Ai) != s->inner_hash ||
+        tf_pattern_hash(L, Ap, Ai) != s->pattern_hash)
+      return tf::fail(TF_ESCHEDULE, "the schedule's runs were built from another inner pattern");
+    return tf::validate_march(s, M, Ap, Ai, inner_Ap, inner_Ai);
+  }
   if (tf_status rc = tf_schedule_validate(s, L, M, Ap, Ai)) return rc;
   if (!s->windowed) return TF_OK;
   if (!inner_Ap || (!inner_Ai && inner_Ap[M] > 0))

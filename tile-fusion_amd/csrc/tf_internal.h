@@ -39,7 +39,7 @@ struct DeviceSchedule;  // device copies + workspace, defined in tf_api.cpp
 constexpr int kMarchW = 8;               // entries per ELL row (longer rows do not march)
 constexpr int kMarchRowBytes = 256;      // an LDS slot: 64 columns of one row
 constexpr int kMarchTabBytes = 4096;     // per-iteration table of a run, staged at the start of LDS
-constexpr int kMarchMaxIter = kMarchTabBytes / 8 - 2;
+constexpr int kMarchMaxIter = kMarchTabBytes / 16 - 2;  // (16 bytes of table per iteration)
 constexpr int kMarchZeroOff = kMarchTabBytes;                    // a row of zeros, read by padding entries
 constexpr int kMarchSlot0 = kMarchTabBytes + kMarchRowBytes;     // first slot
 constexpr int kMarchSrcA = 1 << 30;      // flag in march_ell_src: the value is one of A's (else of B's)
@@ -103,18 +103,19 @@ struct tf_schedule {
   // Marching runs (SpMM-SpMM on stencil-like patterns whose dependences no contiguous tile holds): a run
   // is one workgroup that walks a sequence of steps (a column of grid points, plane by plane) and keeps
   // the rows of C and of the intermediate that its next rows need in numbered LDS slots of one
-  // 64-column row each.  Iteration i of a run first has the C rows of load list i in LDS, then computes
-  // the ELL rows [row_ptr[i], row_ptr[i+1]): intermediate rows first needed by the run's step i (into
-  // slots; halo rows of neighbouring runs are recomputed), then the second-op rows of step i-1 (to D).
-  // Every entry of an ELL row names the LDS byte offset of the row it reads; the inspector assigns the
-  // slots so that a row stays until its last reader has run.
+  // 64-column row each.  Iteration i of a run has the C rows of load list i in LDS, computes the ELL rows
+  // [row_ptr[2i], row_ptr[2i+1]) -- the intermediate rows first needed by the run's step i, into slots
+  // (halo rows of neighbouring runs are recomputed) -- and, after a barrier, the ELL rows
+  // [row_ptr[2i+1], row_ptr[2i+2]) -- the second-op rows of step i, to D -- while the C rows of list i+1
+  // go to their slots.  Every entry of an ELL row names the LDS byte offset of the row it reads; the
+  // inspector assigns the slots so that a row stays until its last reader has run.
   bool march = false;
   int march_grid[3] = {0, 0, 0};     // the grid the runs were cut from (x fastest)
   int march_tile[2] = {0, 0};        // grid points per run and plane: x, y
   int march_slots = 0;               // LDS slots in use by the fullest run
-  int march_rpg = 0, march_lpg = 0;  // ELL rows / C rows a lane group handles per iteration, at most
+  int march_tpg = 0, march_dpg = 0, march_lpg = 0;  // intermediate rows / second-op rows / C rows a lane group handles per iteration, at most
   std::vector<int> march_runs;       // (first iteration, iterations) per run
-  std::vector<int> march_row_ptr;    // [iterations + 1] into the ELL rows
+  std::vector<int> march_row_ptr;    // [2 * iterations + 1] into the ELL rows
   std::vector<int> march_load_ptr;   // [iterations + 1] into the load list
   std::vector<int> march_load;       // (row of C, LDS byte offset) pairs
   std::vector<int> march_row_out;    // per ELL row: >= 0 row of D, < 0 ~(LDS byte offset) of an intermediate row

@@ -9,6 +9,7 @@
 // group, so the per-element sequence is acc = fma(value, x[column], acc) exactly as in
 // the reference's AVX2 kernels (fusion/src/SpMM_SpMM_vectorized.cpp:892-936).
 #include <hip/hip_runtime.h>
+#include <climits>
 #include <type_traits>
 
 #include "tf_internal.h"
@@ -1488,6 +1489,163 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
 }
 
 // ---------------------------------------------------------------------------------
+// Fused SpMM-SpMM over marching runs (stencils on 3D grids): one workgroup of 64 lane groups
+// walks a run iteration by iteration.  LDS holds numbered slots of one 64-column row each; the
+// schedule has turned every column index into the byte offset of the slot that holds the row
+// at that time, so the kernel knows nothing of grids or stencils:
+//   iteration i   rows of C of load list i are in their slots (fetched during iteration i-1)
+//                 ELL rows [row_ptr[i], row_ptr[i+1]): out < 0 -> an intermediate row, summed from
+//                 slots of C into the slot ~out; out >= 0 -> row `out` of D, summed from slots of
+//                 the intermediate (all written in earlier iterations)
+//                 barrier; the rows of C of list i+1, requested at the start of the iteration and
+//                 held in registers meanwhile, go to their slots (whose last readers have run);
+//                 barrier.
+// An ELL row is 8 (offset, value) pairs, 64 bytes: the lanes of a quad hold two pairs each and
+// pass them on by DPP; padding pairs read a row of zeros with value 0.  Entries are walked in
+// CSR order, so results carry the reference's bits.  The lists of the next iteration (and the
+// load list of the one after) are requested an iteration ahead.
+// ---------------------------------------------------------------------------------
+constexpr int kMarchBlock = kMarchGroups * 16;
+
+template <int G>
+__device__ __forceinline__ fvec<4> march_gather(const char *lane_base, int off) {
+  return *reinterpret_cast<const fvec<4> *>(lane_base + quad_bcast<G>(off));
+}
+
+__device__ __forceinline__ fvec<4> march_row(const int4 e, const char *lane_base) {
+  fvec<4> x[8];
+  x[0] = march_gather<0>(lane_base, e.x); x[1] = march_gather<0>(lane_base, e.z);
+  x[2] = march_gather<1>(lane_base, e.x); x[3] = march_gather<1>(lane_base, e.z);
+  x[4] = march_gather<2>(lane_base, e.x); x[5] = march_gather<2>(lane_base, e.z);
+  x[6] = march_gather<3>(lane_base, e.x); x[7] = march_gather<3>(lane_base, e.z);
+  fvec<4> acc = vzero<4>();
+  quad_fma<0>(e.y, x[0], acc); quad_fma<0>(e.w, x[1], acc);
+  quad_fma<1>(e.y, x[2], acc); quad_fma<1>(e.w, x[3], acc);
+  quad_fma<2>(e.y, x[4], acc); quad_fma<2>(e.w, x[5], acc);
+  quad_fma<3>(e.y, x[6], acc); quad_fma<3>(e.w, x[7], acc);
+  return acc;
+}
+
+template <int TPG, int DPG, int LPG, bool ACC>
+__global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
+    const int2 *__restrict__ runs, int n_runs, int per_xcd, const int *__restrict__ row_ptr,
+    const int *__restrict__ load_ptr, const int2 *__restrict__ load_list, const int *__restrict__ row_out,
+    const int4 *__restrict__ ell, const float *__restrict__ C, float *__restrict__ D, int N) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  char *lds = reinterpret_cast<char *>(smem);
+  const int run = xcd_contiguous(blockIdx.x, per_xcd);
+  if (run >= n_runs) return;
+  const int2 rd = runs[run];
+  const int n_iter = rd.y;
+  // per iteration i = 0..n_iter: [4i] first intermediate row, [4i+1] first second-op row, [4i+2] first load
+  int *tab = reinterpret_cast<int *>(lds);
+  for (int i = threadIdx.x; i <= n_iter; i += kMarchBlock) {
+    const int g = rd.x + i;
+    tab[4 * i] = row_ptr[2 * g];
+    tab[4 * i + 1] = i < n_iter ? row_ptr[2 * g + 1] : 0;
+    tab[4 * i + 2] = load_ptr[g];
+  }
+  if (threadIdx.x < 16) *reinterpret_cast<fvec<4> *>(lds + kMarchZeroOff + threadIdx.x * 16) = vzero<4>();
+  __syncthreads();
+  const int group = threadIdx.x >> 4, glane = threadIdx.x & 15, q = threadIdx.x & 3;
+  char *lane_base = lds + glane * 16;
+  const int4 pad = make_int4(kMarchZeroOff, 0, kMarchZeroOff, 0);
+
+  // list entries [b, e) dealt to the lane groups; a group without one gets row -1 / a row of padding
+  auto fetch_loads = [&](int it, int2 (&l)[LPG]) {
+    const bool in = it < n_iter;
+    const int b = in ? tab[4 * it + 2] : 0, e = in ? tab[4 * it + 6] : 0;
+#pragma unroll
+    for (int u = 0; u < LPG; ++u) {
+      const int x = b + group + kMarchGroups * u;
+      l[u] = x < e ? load_list[x] : make_int2(-1, 0);
+    }
+  };
+  auto fetch_rows = [&](int b, int e, auto &el, auto &out) {
+#pragma unroll
+    for (int u = 0; u < (int)(sizeof(out) / sizeof(out[0])); ++u) {
+      const int x = b + group + kMarchGroups * u;
+      const bool ok = x < e;
+      el[u] = ok ? ell[(size_t)x * 4 + q] : pad;
+      out[u] = ok ? row_out[x] : INT_MIN;  // INT_MIN: no row
+    }
+  };
+  auto fetch_t = [&](int it, int4 (&el)[TPG], int (&out)[TPG]) {
+    const bool in = it < n_iter;
+    fetch_rows(in ? tab[4 * it] : 0, in ? tab[4 * it + 1] : 0, el, out);
+  };
+  auto fetch_d = [&](int it, int4 (&el)[DPG], int (&out)[DPG]) {
+    const bool in = it < n_iter;
+    fetch_rows(in ? tab[4 * it + 1] : 0, in ? tab[4 * it + 4] : 0, el, out);
+  };
+
+  for (int c0 = 0; c0 < N; c0 += 64) {
+    const float *Cl = C + c0 + glane * 4;
+    float *Dl = D + c0 + glane * 4;
+    int2 ll[LPG], ll_n[LPG];
+    int4 elt[TPG], elt_n[TPG], eld[DPG], eld_n[DPG];
+    int outt[TPG], outt_n[TPG], outd[DPG], outd_n[DPG];
+    fvec<4> creg[LPG];
+    // before the first iteration: its rows of C into their slots (a list of any length)
+    fetch_t(0, elt, outt);
+    fetch_d(0, eld, outd);
+    fetch_loads(1, ll);
+    for (int x = tab[2] + group; x < tab[6]; x += kMarchGroups) {
+      const int2 l = load_list[x];
+      *reinterpret_cast<fvec<4> *>(lane_base + l.y) = load_streaming4(Cl + (size_t)l.x * N);
+    }
+    __syncthreads();
+    for (int it = 0; it < n_iter; ++it) {
+      // the rows of C the next iteration needs, and the lists after them
+#pragma unroll
+      for (int u = 0; u < LPG; ++u)
+        if (ll[u].x >= 0) creg[u] = load_streaming4(Cl + (size_t)ll[u].x * N);
+      fetch_loads(it + 2, ll_n);
+      fetch_t(it + 1, elt_n, outt_n);
+      fetch_d(it + 1, eld_n, outd_n);
+      // the intermediate rows this iteration's second-op rows are the first to read
+#pragma unroll
+      for (int u = 0; u < TPG; ++u) {
+        const fvec<4> acc = march_row(elt[u], lane_base);
+        if (outt[u] != INT_MIN) *reinterpret_cast<fvec<4> *>(lane_base + ~outt[u]) = acc;
+      }
+      lds_barrier();
+      // the second-op rows; the next rows of C take the slots of rows no one reads any more
+#pragma unroll
+      for (int u = 0; u < DPG; ++u) {
+        fvec<4> acc = march_row(eld[u], lane_base);
+        if (outd[u] != INT_MIN) {
+          float *dst = Dl + (size_t)outd[u] * N;
+          if (ACC) vadd<4>(*reinterpret_cast<const fvec<4> *>(dst), acc);
+          store_streaming<4>(dst, acc);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < LPG; ++u)
+        if (ll[u].x >= 0) *reinterpret_cast<fvec<4> *>(lane_base + ll[u].y) = creg[u];
+      lds_barrier();
+#pragma unroll
+      for (int u = 0; u < LPG; ++u) ll[u] = ll_n[u];
+#pragma unroll
+      for (int u = 0; u < TPG; ++u) { elt[u] = elt_n[u]; outt[u] = outt_n[u]; }
+#pragma unroll
+      for (int u = 0; u < DPG; ++u) { eld[u] = eld_n[u]; outd[u] = outd_n[u]; }
+    }
+  }
+}
+
+// ell[e] = (LDS offset, value): the value of entry src[e] of B, or of A when kMarchSrcA is set; 0 for padding.
+__global__ void march_fill_kernel(const int *__restrict__ off, const int *__restrict__ src, const float *__restrict__ Ax,
+                                  const float *__restrict__ Bx, int2 *__restrict__ ell, size_t n) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const int sidx = src[i];
+    float v = 0.f;
+    if (sidx >= 0) v = (sidx & kMarchSrcA) ? Ax[sidx & (kMarchSrcA - 1)] : Bx[sidx];
+    ell[i] = make_int2(off[i], __float_as_int(v));
+  }
+}
+
+// ---------------------------------------------------------------------------------
 // Host-side launchers
 // ---------------------------------------------------------------------------------
 namespace {
@@ -1807,6 +1965,39 @@ hipError_t launch_fill(float *p, size_t n, float v, hipStream_t st) {
   const int blocks = (int)std::min<size_t>((n + 255) / 256, 65536);
   hipLaunchKernelGGL(fill_kernel, dim3(blocks), dim3(256), 0, st, p, n, v);
   return hipGetLastError();
+}
+
+hipError_t launch_march_fill(const int *off, const int *src, const float *Ax, const float *Bx, int *ell, size_t n,
+                             hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  const int blocks = (int)std::min<size_t>((n + kBlock - 1) / kBlock, 65536);
+  hipLaunchKernelGGL(march_fill_kernel, dim3(blocks), dim3(kBlock), 0, st, off, src, Ax, Bx, reinterpret_cast<int2 *>(ell), n);
+  return hipGetLastError();
+}
+
+hipError_t launch_fused_spmm_spmm_march(const int *runs, int n_runs, const int *row_ptr, const int *load_ptr,
+                                        const int *load_list, const int *row_out, const int *ell, const float *C,
+                                        float *D, int N, int lds_bytes, int tpg, int dpg, int lpg, int accumulate,
+                                        hipStream_t st) {
+  if (n_runs <= 0) return hipSuccess;
+  if (N % 64 != 0 || tpg < 1 || tpg > 4 || dpg < 1 || dpg > 4 || lpg < 1 || lpg > 4 || lds_bytes > 163840) return hipErrorInvalidValue;
+  const int per = per_xcd_of(n_runs);
+  hipError_t err = hipSuccess;
+#define CALLM3(T_, D_, L_, ACC_)                                                                                  \
+  err = allow_lds(fused_spmm_spmm_march_kernel<T_, D_, L_, ACC_>, lds_bytes);                                     \
+  if (err == hipSuccess)                                                                                          \
+    hipLaunchKernelGGL((fused_spmm_spmm_march_kernel<T_, D_, L_, ACC_>), dim3(grid_of(n_runs)), dim3(kMarchBlock), \
+                       lds_bytes, st, reinterpret_cast<const int2 *>(runs), n_runs, per, row_ptr, load_ptr,       \
+                       reinterpret_cast<const int2 *>(load_list), row_out, reinterpret_cast<const int4 *>(ell), C, D, N)
+#define CALLM2(T_, D_, L_) do { if (accumulate) { CALLM3(T_, D_, L_, true); } else { CALLM3(T_, D_, L_, false); } } while (0)
+  // rows per lane group and iteration (intermediate rows, second-op rows, rows of C), rounded up to the
+  // shapes that are built: 2/1/3 is an 8 x 8 column of a 7-point stencil
+  if (tpg <= 2 && dpg <= 1 && lpg <= 3) CALLM2(2, 1, 3);
+  else if (tpg <= 2 && dpg <= 2 && lpg <= 3) CALLM2(2, 2, 3);
+  else CALLM2(4, 4, 4);
+#undef CALLM2
+#undef CALLM3
+  return err != hipSuccess ? err : hipGetLastError();
 }
 
 }  // namespace tf
