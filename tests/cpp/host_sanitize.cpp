@@ -1,6 +1,6 @@
 // Host-only sanitizer harness: the inspector (every kind of schedule), its validator, the file
 // readers and the reordering, compiled with -fsanitize=address,undefined together with
-// csrc/tf_inspector.cpp, tf_io.cpp and tf_reorder.cpp (no GPU code: the three functions those
+// csrc/tf_inspector.cpp, tf_march.cpp, tf_io.cpp and tf_reorder.cpp (no GPU code: the three functions those
 // files take from the HIP side are stubbed here).  Exits 0 when every schedule validates.
 #include <algorithm>
 #include <cstdarg>
@@ -32,7 +32,7 @@ static int run(const char *name, int M, const std::vector<int> &p, const std::ve
   tf_schedule *s = nullptr;
   tf_status rc = tf_inspect(M, M, p.data(), i.data(), &o, &s);
   if (rc) { printf("%s: inspect %d %s\n", name, rc, tf::g_err); return o.op < 0 ? 0 : 1; }
-  rc = tf_schedule_validate(s, M, M, p.data(), i.data());
+  rc = tf_schedule_validate_inner(s, M, M, p.data(), i.data(), o.inner_Ap, o.inner_Ai, o.inner_cols);
   tf_schedule_info info; tf_schedule_get_info(s, &info);
   tf_schedule_view v; tf_schedule_get_view(s, &v);
   printf("%s: validate %d tiles %d fused %d long %d hot %d wide %d streamed %d ws %lld %s\n", name, rc, info.n_tiles, info.n_fused_rows, info.n_long_rows, info.long_row_hot_cols, info.wide_strips, info.streamed, info.workspace_bytes, rc ? tf::g_err : "");
@@ -46,6 +46,24 @@ int main() {
   { tf_inspect_opts o{}; o.struct_size = sizeof(o); o.op = TF_OP_SPMM_SPMM; o.N = 128; o.inner_Ap = p.data(); o.inner_Ai = i.data(); o.inner_cols = 40000; bad += run("band wide", 40000, p, i, o);
     o.wide_strips = -1; bad += run("band narrow", 40000, p, i, o); o.inner_Ap = nullptr; o.inner_Ai = nullptr; o.wide_strips = 0; bad += run("band general", 40000, p, i, o);
     tf_inspect_opts g{}; g.struct_size = sizeof(g); g.op = TF_OP_GEMM_SPMM; g.N = 128; g.K = 100; bad += run("band gemm stream", 40000, p, i, g); g.N = 64; g.K = 20; g.compute_units = 1024; bad += run("band gemm tiles", 40000, p, i, g); }
+  {  // 7-point stencil on a 21 x 17 x 26 grid: marching runs, found from the pattern and with tiles given
+    const int nx = 21, ny = 17, nz = 26, M = nx * ny * nz;
+    p.assign(1, 0); i.clear();
+    for (int z = 0; z < nz; ++z) for (int y = 0; y < ny; ++y) for (int x = 0; x < nx; ++x) {
+      const int r = (z * ny + y) * nx + x;
+      if (z > 0) i.push_back(r - nx * ny);
+      if (y > 0) i.push_back(r - nx);
+      if (x > 0) i.push_back(r - 1);
+      i.push_back(r);
+      if (x < nx - 1) i.push_back(r + 1);
+      if (y < ny - 1) i.push_back(r + nx);
+      if (z < nz - 1) i.push_back(r + nx * ny);
+      p.push_back((int)i.size());
+    }
+    tf_inspect_opts o{}; o.struct_size = sizeof(o); o.op = TF_OP_SPMM_SPMM; o.N = 64; o.inner_Ap = p.data(); o.inner_Ai = i.data(); o.inner_cols = M; o.march = 1;
+    bad += run("stencil march", M, p, i, o);
+    o.march_tile_x = 5; o.march_tile_y = 3; o.compute_units = 7; bad += run("stencil march 5x3", M, p, i, o);
+    o.march_tile_x = o.march_tile_y = 0; o.grid_nx = ny; o.grid_ny = nx; o.grid_nz = nz; bad += run("stencil march, wrong grid", M, p, i, o); }
   powerlaw(60000, 1500000, 2, p, i);
   { tf_inspect_opts o{}; o.struct_size = sizeof(o); o.op = TF_OP_GEMM_SPMM; o.N = 128; o.K = 128; o.long_row_partition = 1; bad += run("powerlaw part", 60000, p, i, o);
     o.long_row_partition = -1; bad += run("powerlaw chunks", 60000, p, i, o);

@@ -1,7 +1,7 @@
 """The host-side C++ (inspector, validator, file readers, reordering) under AddressSanitizer
 and UBSan: tests/cpp/host_sanitize.cpp builds windowed (wide and lane-group), general,
-streamed and tiled schedules and both kinds of long-row schedules on banded and power-law
-patterns, validates each, runs RCM and a file read.  No GPU code is compiled in."""
+streamed and tiled schedules, both kinds of long-row schedules and marching runs on banded, power-law
+and 3D-stencil patterns, validates each, runs RCM and a file read.  No GPU code is compiled in."""
 import os
 import shutil
 import subprocess
@@ -18,7 +18,7 @@ def test_host_code_under_sanitizers(tmp_path):
     exe = str(tmp_path / "host_sanitize")
     cmd = ["g++", "-O1", "-g", "-std=c++17", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
            "-fno-omit-frame-pointer", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-o", exe,
-           os.path.join(ROOT, "tests", "cpp", "host_sanitize.cpp"), os.path.join(CSRC, "tf_inspector.cpp"),
+           os.path.join(ROOT, "tests", "cpp", "host_sanitize.cpp"), os.path.join(CSRC, "tf_inspector.cpp"), os.path.join(CSRC, "tf_march.cpp"),
            os.path.join(CSRC, "tf_io.cpp"), os.path.join(CSRC, "tf_reorder.cpp")]
     b = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
     assert b.returncode == 0, b.stderr[-2000:]

@@ -55,6 +55,7 @@ struct DeviceSchedule {
   // marching runs: the schedule's lists, and the ELL rows with the operands' values filled in
   int *m_runs = nullptr, *m_row_ptr = nullptr, *m_load_ptr = nullptr, *m_load = nullptr, *m_row_out = nullptr;
   int *m_ell_off = nullptr, *m_ell_src = nullptr, *m_ell = nullptr;
+  float *m_trash = nullptr;  // a row in global memory that takes the stores of lane groups without a row
   unsigned long long m_serial_a = 0, m_serial_b = 0;  // the uploaded matrices the values were taken from (0: none)
   // A second stream of the same priority for kernels that may run beside the caller's stream (the
   // hot long-row segments beside the rest of the GEMM), with the events that fork it off and join it.
@@ -80,7 +81,7 @@ hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const fl
                             float *, int, int, int, int, hipStream_t);
 hipError_t launch_march_fill(const int *, const int *, const float *, const float *, int *, size_t, hipStream_t);
 hipError_t launch_fused_spmm_spmm_march(const int *, int, const int *, const int *, const int *, const int *, const int *,
-                                        const float *, float *, int, int, int, int, int, int, hipStream_t);
+                                        const float *, float *, float *, int, int, int, int, int, int, hipStream_t);
 hipError_t launch_scatter_values(const int *, const int *, const float *, float *, int, hipStream_t);
 hipError_t launch_seg_reduce(const LongRow *, int, const int *, const float *, float *, int, int, hipStream_t);
 hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const int *, const float *,
@@ -138,7 +139,7 @@ void release_device_schedule(DeviceSchedule *d) {
   (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
   (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad);
   (void)hipFree(d->m_runs); (void)hipFree(d->m_row_ptr); (void)hipFree(d->m_load_ptr); (void)hipFree(d->m_load);
-  (void)hipFree(d->m_row_out); (void)hipFree(d->m_ell_off); (void)hipFree(d->m_ell_src); (void)hipFree(d->m_ell);
+  (void)hipFree(d->m_row_out); (void)hipFree(d->m_ell_off); (void)hipFree(d->m_ell_src); (void)hipFree(d->m_ell); (void)hipFree(d->m_trash);
   if (d->side) (void)hipStreamDestroy(d->side);
   if (d->fork) (void)hipEventDestroy(d->fork);
   if (d->join) (void)hipEventDestroy(d->join);
@@ -181,6 +182,8 @@ static tf_status ensure_device(tf_schedule *s) {
     if (!rc) rc = upload_vec(s->march_ell_src, &d->m_ell_src);
     if (!rc) {
       hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->m_ell), s->march_ell_off.size() * 2 * sizeof(int));
+      if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&d->m_trash), 64 * sizeof(float));
+      if (e == hipSuccess) e = hipMemset(d->m_trash, 0, 64 * sizeof(float));
       if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(ELL rows)");
     }
     if (rc) { release_device_schedule(d); return rc; }
@@ -593,7 +596,7 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
     d->m_serial_b = B->serial;
     TF_PHASE(s, "fused_spmm_spmm_march_kernel", st,
              tf::launch_fused_spmm_spmm_march(d->m_runs, (int)s->march_runs.size() / 2, d->m_row_ptr, d->m_load_ptr, d->m_load,
-                                              d->m_row_out, d->m_ell, C->d, D->d, s->opts.N, s->lds_bytes, s->march_tpg,
+                                              d->m_row_out, d->m_ell, C->d, D->d, d->m_trash, s->opts.N, s->lds_bytes, s->march_tpg,
                                               s->march_dpg, s->march_lpg, acc, st));
     return TF_OK;
   }

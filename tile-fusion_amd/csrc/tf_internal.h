@@ -41,9 +41,13 @@ constexpr int kMarchRowBytes = 256;      // an LDS slot: 64 columns of one row
 constexpr int kMarchTabBytes = 4096;     // per-iteration table of a run, staged at the start of LDS
 constexpr int kMarchMaxIter = kMarchTabBytes / 16 - 2;  // (16 bytes of table per iteration)
 constexpr int kMarchZeroOff = kMarchTabBytes;                    // a row of zeros, read by padding entries
-constexpr int kMarchSlot0 = kMarchTabBytes + kMarchRowBytes;     // first slot
+constexpr int kMarchTrashOff = kMarchTabBytes + kMarchRowBytes;  // a row that takes what lane groups without work write
+constexpr int kMarchSlot0 = kMarchTabBytes + 2 * kMarchRowBytes; // first slot
 constexpr int kMarchSrcA = 1 << 30;      // flag in march_ell_src: the value is one of A's (else of B's)
-constexpr int kMarchGroups = 64;         // lane groups (of 16 lanes) per workgroup
+constexpr int kMarchGroups = 32;         // lane groups (of 16 lanes) per workgroup
+// rows one lane group takes per iteration, at most (the kernel's register sets): intermediate rows,
+// second-op rows, rows of C
+constexpr int kMarchTpg = 3, kMarchDpg = 2, kMarchLpg = 5;
 
 }  // namespace tf
 

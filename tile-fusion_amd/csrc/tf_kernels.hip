@@ -1489,23 +1489,36 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
 }
 
 // ---------------------------------------------------------------------------------
-// Fused SpMM-SpMM over marching runs (stencils on 3D grids): one workgroup of 64 lane groups
+// Fused SpMM-SpMM over marching runs (stencils on 3D grids): one workgroup of 32 lane groups
 // walks a run iteration by iteration.  LDS holds numbered slots of one 64-column row each; the
 // schedule has turned every column index into the byte offset of the slot that holds the row
 // at that time, so the kernel knows nothing of grids or stencils:
-//   iteration i   rows of C of load list i are in their slots (fetched during iteration i-1)
-//                 ELL rows [row_ptr[i], row_ptr[i+1]): out < 0 -> an intermediate row, summed from
-//                 slots of C into the slot ~out; out >= 0 -> row `out` of D, summed from slots of
-//                 the intermediate (all written in earlier iterations)
-//                 barrier; the rows of C of list i+1, requested at the start of the iteration and
-//                 held in registers meanwhile, go to their slots (whose last readers have run);
-//                 barrier.
+//   iteration i   rows of C of load list i are in their slots
+//                 ELL rows [row_ptr[2i], row_ptr[2i+1]): intermediate rows, summed from slots of C
+//                 into the slot ~out; barrier;
+//                 ELL rows [row_ptr[2i+1], row_ptr[2i+2]): rows `out` of D, summed from slots of
+//                 the intermediate; the rows of C of list i+1, held in registers meanwhile, go to
+//                 their slots (whose last readers have run); barrier.
 // An ELL row is 8 (offset, value) pairs, 64 bytes: the lanes of a quad hold two pairs each and
 // pass them on by DPP; padding pairs read a row of zeros with value 0.  Entries are walked in
-// CSR order, so results carry the reference's bits.  The lists of the next iteration (and the
-// load list of the one after) are requested an iteration ahead.
+// CSR order, so results carry the reference's bits.
+// Memory latency is what such a loop has to hide: a run is one workgroup per compute unit, in
+// step with all others.  The lists of an iteration (its ELL rows and the load list two lists
+// on) are requested two iterations ahead and the rows of C two lists ahead, into register
+// sets used in turn -- which is why the workgroup has 512 threads: eight wavefronts have 256
+// registers each.  Loads return in the order they were issued, so within an iteration what is
+// needed first is requested first.
 // ---------------------------------------------------------------------------------
 constexpr int kMarchBlock = kMarchGroups * 16;
+
+// -1 / 0 for true / false, in a form the compiler cannot see through: a value that was loaded and is
+// blended with such a mask stays a load that is always issued.  (Written as a select, the load moves
+// under the condition, and a load under a condition is waited for at once.)
+__device__ __forceinline__ int opaque_mask(bool c) {
+  int m = c ? -1 : 0;
+  asm volatile("" : "+v"(m));
+  return m;
+}
 
 template <int G>
 __device__ __forceinline__ fvec<4> march_gather(const char *lane_base, int off) {
@@ -1526,11 +1539,25 @@ __device__ __forceinline__ fvec<4> march_row(const int4 e, const char *lane_base
   return acc;
 }
 
-template <int TPG, int DPG, int LPG, bool ACC>
+// What a lane keeps of one iteration's lists: its pairs of the ELL rows of its lane group (up to
+// kMarchTpg intermediate rows, kMarchDpg second-op rows), where they go, and the group's share
+// of the load list two lists on.
+struct MarchLists {
+  int4 et[kMarchTpg], ed[kMarchDpg];
+  int ot[kMarchTpg], od[kMarchDpg];
+  int2 ll[kMarchLpg];
+};
+// Rows of C on their way: the group's share of one load list and the rows themselves.
+struct MarchStage {
+  int2 ll[kMarchLpg];
+  fvec<4> c[kMarchLpg];
+};
+
+template <bool ACC>
 __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
     const int2 *__restrict__ runs, int n_runs, int per_xcd, const int *__restrict__ row_ptr,
     const int *__restrict__ load_ptr, const int2 *__restrict__ load_list, const int *__restrict__ row_out,
-    const int4 *__restrict__ ell, const float *__restrict__ C, float *__restrict__ D, int N) {
+    const int4 *__restrict__ ell, const float *__restrict__ C, float *__restrict__ D, float *__restrict__ trash, int N) {
   extern __shared__ __align__(16) unsigned char smem[];
   char *lds = reinterpret_cast<char *>(smem);
   const int run = xcd_contiguous(blockIdx.x, per_xcd);
@@ -1549,87 +1576,101 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
   __syncthreads();
   const int group = threadIdx.x >> 4, glane = threadIdx.x & 15, q = threadIdx.x & 3;
   char *lane_base = lds + glane * 16;
-  const int4 pad = make_int4(kMarchZeroOff, 0, kMarchZeroOff, 0);
-
-  // list entries [b, e) dealt to the lane groups; a group without one gets row -1 / a row of padding
-  auto fetch_loads = [&](int it, int2 (&l)[LPG]) {
-    const bool in = it < n_iter;
-    const int b = in ? tab[4 * it + 2] : 0, e = in ? tab[4 * it + 6] : 0;
+  // List entries [b, e) dealt to the lane groups.  Nothing in the loop is under a condition: a lane
+  // group without an entry loads row 0 of C into the trash row, computes a row of padding into the
+  // trash row, stores it to the trash row in global memory.  A wait for an older load can then leave
+  // all younger ones in flight, which loads and stores under conditions do not allow.
+  auto fetch_loads = [&](int list, int2 (&l)[kMarchLpg]) {
+    const bool in = list < n_iter;
+    const int b = in ? tab[4 * list + 2] : 0, e = in ? tab[4 * list + 6] : 0;
 #pragma unroll
-    for (int u = 0; u < LPG; ++u) {
+    for (int u = 0; u < kMarchLpg; ++u) {
       const int x = b + group + kMarchGroups * u;
-      l[u] = x < e ? load_list[x] : make_int2(-1, 0);
+      const int2 v = load_list[max(min(x, e - 1), 0)];
+      const int m = opaque_mask(x < e);
+      l[u] = make_int2(v.x, (v.y & m) | (kMarchTrashOff & ~m));  // a group without an entry re-reads another's row into the trash row
     }
   };
-  auto fetch_rows = [&](int b, int e, auto &el, auto &out) {
+  auto fetch_lists = [&](int it, MarchLists &L) {
+    const bool in = it < n_iter;
+    const int b0 = in ? tab[4 * it] : 0, b1 = in ? tab[4 * it + 1] : 0, b2 = in ? tab[4 * it + 4] : 0;
 #pragma unroll
-    for (int u = 0; u < (int)(sizeof(out) / sizeof(out[0])); ++u) {
-      const int x = b + group + kMarchGroups * u;
-      const bool ok = x < e;
-      el[u] = ok ? ell[(size_t)x * 4 + q] : pad;
-      out[u] = ok ? row_out[x] : INT_MIN;  // INT_MIN: no row
+    for (int u = 0; u < kMarchTpg; ++u) {
+      const int x = b0 + group + kMarchGroups * u, xc = max(min(x, b1 - 1), 0);
+      const bool ok = x < b1;
+      const int o = row_out[xc], m = opaque_mask(ok);
+      L.et[u] = ell[(size_t)xc * 4 + q];  // a group without a row recomputes another's, into the trash row
+      L.ot[u] = (o & m) | (~kMarchTrashOff & ~m);
     }
-  };
-  auto fetch_t = [&](int it, int4 (&el)[TPG], int (&out)[TPG]) {
-    const bool in = it < n_iter;
-    fetch_rows(in ? tab[4 * it] : 0, in ? tab[4 * it + 1] : 0, el, out);
-  };
-  auto fetch_d = [&](int it, int4 (&el)[DPG], int (&out)[DPG]) {
-    const bool in = it < n_iter;
-    fetch_rows(in ? tab[4 * it + 1] : 0, in ? tab[4 * it + 4] : 0, el, out);
+#pragma unroll
+    for (int u = 0; u < kMarchDpg; ++u) {
+      const int x = b1 + group + kMarchGroups * u, xc = max(min(x, b2 - 1), 0);
+      const bool ok = x < b2;
+      const int o = row_out[xc], m = opaque_mask(ok);
+      L.ed[u] = ell[(size_t)xc * 4 + q];
+      L.od[u] = o | ~m;  // -1: no row
+    }
+    fetch_loads(it + 2, L.ll);
   };
 
   for (int c0 = 0; c0 < N; c0 += 64) {
     const float *Cl = C + c0 + glane * 4;
     float *Dl = D + c0 + glane * 4;
-    int2 ll[LPG], ll_n[LPG];
-    int4 elt[TPG], elt_n[TPG], eld[DPG], eld_n[DPG];
-    int outt[TPG], outt_n[TPG], outd[DPG], outd_n[DPG];
-    fvec<4> creg[LPG];
-    // before the first iteration: its rows of C into their slots (a list of any length)
-    fetch_t(0, elt, outt);
-    fetch_d(0, eld, outd);
-    fetch_loads(1, ll);
-    for (int x = tab[2] + group; x < tab[6]; x += kMarchGroups) {
-      const int2 l = load_list[x];
-      *reinterpret_cast<fvec<4> *>(lane_base + l.y) = load_streaming4(Cl + (size_t)l.x * N);
-    }
-    __syncthreads();
-    for (int it = 0; it < n_iter; ++it) {
-      // the rows of C the next iteration needs, and the lists after them
+    float *Tl = trash + glane * 4;
+    auto issue = [&](MarchStage &S) {
 #pragma unroll
-      for (int u = 0; u < LPG; ++u)
-        if (ll[u].x >= 0) creg[u] = load_streaming4(Cl + (size_t)ll[u].x * N);
-      fetch_loads(it + 2, ll_n);
-      fetch_t(it + 1, elt_n, outt_n);
-      fetch_d(it + 1, eld_n, outd_n);
+      for (int u = 0; u < kMarchLpg; ++u) S.c[u] = load_streaming4(Cl + (size_t)S.ll[u].x * N);
+    };
+    // One iteration.  `cur` holds its lists; `fut` is free and takes those of iteration it + 2.  Stage
+    // X is free (its rows went to LDS an iteration ago) and takes list it + 2, whose entries came with
+    // `cur`; stage Y holds list it + 1, which goes to LDS in the second half.
+    auto step = [&](int it, const MarchLists &cur, MarchLists &fut, MarchStage &X, const MarchStage &Y) {
+#pragma unroll
+      for (int u = 0; u < kMarchLpg; ++u) X.ll[u] = cur.ll[u];
+      issue(X);
+      fetch_lists(it + 2, fut);
       // the intermediate rows this iteration's second-op rows are the first to read
 #pragma unroll
-      for (int u = 0; u < TPG; ++u) {
-        const fvec<4> acc = march_row(elt[u], lane_base);
-        if (outt[u] != INT_MIN) *reinterpret_cast<fvec<4> *>(lane_base + ~outt[u]) = acc;
+      for (int u = 0; u < kMarchTpg; ++u) {
+        const fvec<4> acc = march_row(cur.et[u], lane_base);
+        *reinterpret_cast<fvec<4> *>(lane_base + ~cur.ot[u]) = acc;
       }
       lds_barrier();
       // the second-op rows; the next rows of C take the slots of rows no one reads any more
 #pragma unroll
-      for (int u = 0; u < DPG; ++u) {
-        fvec<4> acc = march_row(eld[u], lane_base);
-        if (outd[u] != INT_MIN) {
-          float *dst = Dl + (size_t)outd[u] * N;
-          if (ACC) vadd<4>(*reinterpret_cast<const fvec<4> *>(dst), acc);
-          store_streaming<4>(dst, acc);
-        }
+      for (int u = 0; u < kMarchDpg; ++u) {
+        fvec<4> acc = march_row(cur.ed[u], lane_base);
+        float *dst = cur.od[u] >= 0 ? Dl + (size_t)cur.od[u] * N : Tl;
+        if (ACC) vadd<4>(*reinterpret_cast<const fvec<4> *>(dst), acc);
+        store_streaming<4>(dst, acc);
       }
 #pragma unroll
-      for (int u = 0; u < LPG; ++u)
-        if (ll[u].x >= 0) *reinterpret_cast<fvec<4> *>(lane_base + ll[u].y) = creg[u];
+      for (int u = 0; u < kMarchLpg; ++u) *reinterpret_cast<fvec<4> *>(lane_base + Y.ll[u].y) = Y.c[u];
       lds_barrier();
-#pragma unroll
-      for (int u = 0; u < LPG; ++u) ll[u] = ll_n[u];
-#pragma unroll
-      for (int u = 0; u < TPG; ++u) { elt[u] = elt_n[u]; outt[u] = outt_n[u]; }
-#pragma unroll
-      for (int u = 0; u < DPG; ++u) { eld[u] = eld_n[u]; outd[u] = outd_n[u]; }
+    };
+    MarchLists E0, E1, E2;
+    MarchStage S0, S1;
+    // before the first iteration: its rows of C into their slots (a list of any length), list 1 on its
+    // way, the lists of the first two iterations
+    fetch_lists(0, E0);
+    fetch_loads(1, S1.ll);
+    fetch_lists(1, E1);
+    for (int x = tab[2] + group; x < tab[6]; x += kMarchGroups) {
+      const int2 l = load_list[x];
+      *reinterpret_cast<fvec<4> *>(lane_base + l.y) = load_streaming4(Cl + (size_t)l.x * N);
+    }
+    issue(S1);
+    __syncthreads();
+    // (six steps, the period of the register sets, without a way out in between: iterations past the
+    // run's last find empty lists and work on the trash rows.  A path that skips steps would make
+    // the waits for loads assume that nothing younger is in flight.)
+    for (int it = 0; it < n_iter; it += 6) {
+      step(it, E0, E2, S0, S1);
+      step(it + 1, E1, E0, S1, S0);
+      step(it + 2, E2, E1, S0, S1);
+      step(it + 3, E0, E2, S1, S0);
+      step(it + 4, E1, E0, S0, S1);
+      step(it + 5, E2, E1, S1, S0);
     }
   }
 }
@@ -1977,26 +2018,22 @@ hipError_t launch_march_fill(const int *off, const int *src, const float *Ax, co
 
 hipError_t launch_fused_spmm_spmm_march(const int *runs, int n_runs, const int *row_ptr, const int *load_ptr,
                                         const int *load_list, const int *row_out, const int *ell, const float *C,
-                                        float *D, int N, int lds_bytes, int tpg, int dpg, int lpg, int accumulate,
-                                        hipStream_t st) {
+                                        float *D, float *trash, int N, int lds_bytes, int tpg, int dpg, int lpg,
+                                        int accumulate, hipStream_t st) {
   if (n_runs <= 0) return hipSuccess;
-  if (N % 64 != 0 || tpg < 1 || tpg > 4 || dpg < 1 || dpg > 4 || lpg < 1 || lpg > 4 || lds_bytes > 163840) return hipErrorInvalidValue;
+  // (rows per lane group and iteration beyond what the kernel's register sets hold would be skipped silently)
+  if (N % 64 != 0 || tpg < 1 || tpg > kMarchTpg || dpg < 1 || dpg > kMarchDpg || lpg < 1 || lpg > kMarchLpg || lds_bytes > 163840)
+    return hipErrorInvalidValue;
   const int per = per_xcd_of(n_runs);
   hipError_t err = hipSuccess;
-#define CALLM3(T_, D_, L_, ACC_)                                                                                  \
-  err = allow_lds(fused_spmm_spmm_march_kernel<T_, D_, L_, ACC_>, lds_bytes);                                     \
+#define CALLM(ACC_)                                                                                               \
+  err = allow_lds(fused_spmm_spmm_march_kernel<ACC_>, lds_bytes);                                                 \
   if (err == hipSuccess)                                                                                          \
-    hipLaunchKernelGGL((fused_spmm_spmm_march_kernel<T_, D_, L_, ACC_>), dim3(grid_of(n_runs)), dim3(kMarchBlock), \
+    hipLaunchKernelGGL((fused_spmm_spmm_march_kernel<ACC_>), dim3(grid_of(n_runs)), dim3(kMarchBlock),            \
                        lds_bytes, st, reinterpret_cast<const int2 *>(runs), n_runs, per, row_ptr, load_ptr,       \
-                       reinterpret_cast<const int2 *>(load_list), row_out, reinterpret_cast<const int4 *>(ell), C, D, N)
-#define CALLM2(T_, D_, L_) do { if (accumulate) { CALLM3(T_, D_, L_, true); } else { CALLM3(T_, D_, L_, false); } } while (0)
-  // rows per lane group and iteration (intermediate rows, second-op rows, rows of C), rounded up to the
-  // shapes that are built: 2/1/3 is an 8 x 8 column of a 7-point stencil
-  if (tpg <= 2 && dpg <= 1 && lpg <= 3) CALLM2(2, 1, 3);
-  else if (tpg <= 2 && dpg <= 2 && lpg <= 3) CALLM2(2, 2, 3);
-  else CALLM2(4, 4, 4);
-#undef CALLM2
-#undef CALLM3
+                       reinterpret_cast<const int2 *>(load_list), row_out, reinterpret_cast<const int4 *>(ell), C, D, trash, N)
+  if (accumulate) { CALLM(true); } else { CALLM(false); }
+#undef CALLM
   return err != hipSuccess ? err : hipGetLastError();
 }
 

@@ -16,8 +16,6 @@
 // schedule slow or impossible, never wrong.
 #include <algorithm>
 #include <climits>
-#include <cstdio>
-#include <cstdlib>
 #include <cstring>
 #include <map>
 
@@ -28,7 +26,6 @@ namespace tf {
 namespace {
 
 constexpr int kMaxLds = 163840;
-constexpr int kMaxPerGroup = 4;  // ELL rows / C rows one lane group takes per iteration, at most
 
 // The grid a pattern was generated on, from the distances between a row and its columns: a
 // 7-point-like stencil on nx x ny x nz points, x fastest, has the distances 1, nx and nx*ny.
@@ -116,7 +113,7 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
           // whole rounds of the lane groups.
           size_t steady_t = 1;
           for (int s = 1; s < steps; ++s) steady_t = std::max(steady_t, tgroup[s].size());
-          const size_t cap_t = kMarchGroups * std::min<size_t>(kMaxPerGroup, (steady_t + kMarchGroups - 1) / kMarchGroups);
+          const size_t cap_t = kMarchGroups * std::min<size_t>(kMarchTpg, (steady_t + kMarchGroups - 1) / kMarchGroups);
           const int warm = tgroup[0].size() > cap_t ? (int)((tgroup[0].size() + cap_t - 1) / cap_t) - 1 : 0;
           const int n_iter = steps + warm;
           if (n_iter > kMarchMaxIter) return false;
@@ -153,7 +150,7 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
           {
             size_t steady_c = 1;
             for (int g = warm + 2; g < n_iter; ++g) steady_c = std::max(steady_c, cgroup[g].size());
-            const size_t cap_c = kMarchGroups * std::min<size_t>(kMaxPerGroup, (steady_c + kMarchGroups - 1) / kMarchGroups);
+            const size_t cap_c = kMarchGroups * std::min<size_t>(kMarchLpg, (steady_c + kMarchGroups - 1) / kMarchGroups);
             for (int g = n_iter - 1; g >= 1; --g) {
               std::sort(cgroup[g].begin(), cgroup[g].end());
               while (cgroup[g].size() > cap_c) { cgroup[g - 1].push_back(cgroup[g].back()); cgroup[g].pop_back(); }
@@ -224,7 +221,7 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
               produced += (long long)tgroup[it].size();
               max_t = std::max(max_t, (int)tgroup[it].size());
             }
-            if (next_slot > slot_budget) { if (getenv("TF_MARCH_DEBUG")) fprintf(stderr, "march %dx%d: run %d phase %d needs %d slots (budget %d), T %zu C %zu\n", bx, by, run, ph, next_slot, slot_budget, tgroup[std::max(ph,0)/2].size(), cgroup[std::min((ph+1)/2, n_iter-1)].size()); return false; }
+            if (next_slot > slot_budget) return false;
           }
           max_slots = std::max(max_slots, next_slot);
           td.cons_end = (int)ids.size();
@@ -233,8 +230,8 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
           tiles.push_back(td);
         }
     }
-    if ((long long)row_out.size() * kMarchW > INT_MAX || max_t > kMaxPerGroup * kMarchGroups || max_d > kMaxPerGroup * kMarchGroups ||
-        max_loads > kMaxPerGroup * kMarchGroups || (int)ids.size() != M)
+    if ((long long)row_out.size() * kMarchW > INT_MAX || max_t > kMarchTpg * kMarchGroups || max_d > kMarchDpg * kMarchGroups ||
+        max_loads > kMarchLpg * kMarchGroups || (int)ids.size() != M)
       return false;
     S->march = true;
     S->march_grid[0] = nx; S->march_grid[1] = ny; S->march_grid[2] = nz;
@@ -313,7 +310,7 @@ tf_status validate_march(const tf_schedule *s, int M, const int *Ap, const int *
       s->march_row_ptr.empty() || s->march_row_ptr.back() != (int)n_rows || s->march_row_ptr.size() != 2 * s->march_load_ptr.size() - 1 ||
       s->march_load_ptr.back() * 2 != (int)s->march_load.size())
     return fail(TF_ESCHEDULE, "marching schedule: tables do not match");
-  if (s->march_tpg < 1 || s->march_tpg > kMaxPerGroup || s->march_dpg < 1 || s->march_dpg > kMaxPerGroup || s->march_lpg < 1 || s->march_lpg > kMaxPerGroup)
+  if (s->march_tpg < 1 || s->march_tpg > kMarchTpg || s->march_dpg < 1 || s->march_dpg > kMarchDpg || s->march_lpg < 1 || s->march_lpg > kMarchLpg)
     return fail(TF_ESCHEDULE, "marching schedule: rows per lane group out of range");
   const int n_iters = (int)s->march_load_ptr.size() - 1;
   std::vector<int> done(M, 0);
