@@ -187,7 +187,8 @@ def kernel_names(info, op_is_gemm, unfused):
     if unfused:
         return "gemm_rows_kernel + spmm_rows_kernel"
     if not op_is_gemm:
-        return ("fused_spmm_spmm_window64_kernel" if info["wide_strips"] else
+        return ("fused_spmm_spmm_march_kernel" if info["marched"] else
+                "fused_spmm_spmm_window64_kernel" if info["wide_strips"] else
                 "fused_spmm_spmm_window_kernel" if info["windowed"] else
                 "fused_spmm_spmm_kernel" if info["n_fused_rows"] else "spmm_rows_kernel (twice)")
     if info["n_fused_rows"] == 0:
@@ -206,7 +207,8 @@ def run_config(tf, cfg, idx, steps, warmup, args):
     inner = Ah if (not gemm and cfg["B"] is A and not args.no_window) else None
     S = tf.inspector(Ah, 1, op=op, N=N, K=K, lds_budget_bytes=args.lds, tile_rows=args.tile_rows,
                      max_redundancy=args.max_redundancy, inner=inner, strip_cols=args.strip, wide_strips=args.wide,
-                     long_row_nnz=args.long_row, xcd_chunk_rows=args.xcd_chunk, long_row_partition=args.long_part)
+                     long_row_nnz=args.long_row, xcd_chunk_rows=args.xcd_chunk, long_row_partition=args.long_part,
+                     march=args.march, reorder_adjacency=args.reorder_adj)
     inspect_s = time.perf_counter() - t0
     S.validate()
     info = S.info()
@@ -274,7 +276,7 @@ def run_config(tf, cfg, idx, steps, warmup, args):
         "rel_err_vs_f64": err, "rows_checked": rows_checked,
         "kernels": kernels, "kernel": kernel_names(info, gemm, args.unfused),
         "schedule": {"lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "wide_strips": bool(info["wide_strips"]),
-                     "streamed": bool(info["streamed"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
+                     "streamed": bool(info["streamed"]), "marched": bool(info["marched"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
                      "remainder_rows": info["n_remainder_rows"], "long_rows": info["n_long_rows"],
                      "long_row_hot_cols": info["long_row_hot_cols"],
                      "recomputed_rows": info["n_producer_rows"] - A.shape[1], "writeback_rows": info["n_writeback_rows"],
@@ -310,6 +312,9 @@ def main():
     ap.add_argument("--long-row", type=int, default=0, help="rows with more entries than this are chunked")
     ap.add_argument("--long-part", type=int, default=0, choices=[-1, 0, 1],
                     help="long rows: 1 = regrouped by the XCD partition of their columns, -1 = chunks of consecutive entries, 0 = library's choice")
+    ap.add_argument("--march", type=int, default=0, choices=[-1, 0, 1], help="marching runs for stencils on 3D grids: -1 = never, 1 = must")
+    ap.add_argument("--reorder-adj", type=int, default=0, choices=[-1, 0, 1],
+                    help="remainder rows: -1 = read from A's arrays through the row list, 0/1 = stored in list order (reordered adjacency)")
     ap.add_argument("--second-stream", action="store_true", help="hot long-row segments on the executor's second stream, beside the GEMM (TF_SECOND_STREAM)")
     ap.add_argument("--matrix", default=None, help="run on a .mtx / .smtx file instead of a synthetic configuration "
                     "(square; symmetric files are expanded), with --op, --N and --K")

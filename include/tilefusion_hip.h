@@ -218,6 +218,14 @@ typedef struct {
   int march;
   int grid_nx, grid_ny, grid_nz;
   int march_tile_x, march_tile_y;
+  /* Remainder rows (second-op rows served from the intermediate in HBM) are worked on in the order of
+     a list (by length class).  0 / 1 = when that order is not simply all rows in order, the schedule
+     also keeps those rows' columns -- and the executor their values -- side by side in list order,
+     which is what the reference's reordered adjacency is to its executors (createReorderedAdj,
+     fusion/gcn/SingleLayer/GCN_Single_Layer_SP_Demo_Utils.h:618-653, read by
+     forwardForOneLayerFusedParallelSeparatedReorderedAdjVectorizedSP, GCN_Layer_MKL_Forward_Utils.h:294-373);
+     -1 = the rows are read from A's arrays in place through the list. */
+  int reorder_adjacency;
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -308,13 +316,14 @@ tf_status tf_schedule_validate_inner(const tf_schedule *s, int L, int M, const i
 enum {
   TF_ACCUMULATE = 1u,   /* D += A*(B*C), the reference's convention (its callers zero D
                            first); without it D is overwritten and need not be initialised */
-  TF_SECOND_STREAM = 2u /* GeMM-SpMM with column-partitioned long rows: run the hot long-row segments
+  TF_SECOND_STREAM = 2u, /* GeMM-SpMM with column-partitioned long rows: run the hot long-row segments
                            on a second stream of the schedule's own (same priority), forked from and
                            joined to the given one with events, beside the GEMM of the other rows.
                            Without it every kernel of a call runs on the given stream, one after
                            another -- which measured as fast on the R-MAT configuration (2.32 ms
                            against 2.35 ms: the gathers and the GEMM's operand traffic meet in the
                            same memory system), so it is not the default */
+  TF_RELU = 4u           /* tf_gcn_two_layers: ReLU between the layers */
 };
 
 /* D = A * (B * C), A and B sparse.  Stands in for
@@ -333,6 +342,21 @@ tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_dense *C, tf_d
  * K x N (Weight, not transposed), D is L x N.  The tile GEMM runs on fp32 MFMA. */
 tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf_dense *D,
                        tf_schedule *schedule, unsigned flags, void *stream);
+
+/* Two GCN layers in one call:  D = A * (act(A * (X * W1)) * W2),  act = ReLU with TF_RELU, else
+ * the identity.  Stands in for fusedGCN (binding-project/src/Functions.cpp:228-290) and for what the
+ * reference's end-to-end model runs (binding-project/gcn-e2e-training/FusedGCNModule.py:7-18: two fused
+ * layers with a ReLU between).  A is square (M x M), X is M x K, W1 is K x H, W2 is H x N (weights not
+ * transposed, as in tf_gemm_spmm), D is M x N.  s1 must come from tf_inspect on A's pattern for
+ * (TF_OP_GEMM_SPMM, K, H), s2 for (TF_OP_GEMM_SPMM, H, N); they may be one schedule when K = H = N.
+ * The hidden layer stays on the device: in `hidden` (M x H) when given -- training keeps it for the
+ * backward pass -- else in a buffer that s2 owns.  Each layer runs as tf_gemm_spmm does, so rows fuse
+ * inside a layer; no tile carries a row through both layers (a row of the second layer needs the whole
+ * neighbourhood of its neighbours from the first).  The reference's fusedGCN reads its second GEMM's input
+ * from the first GEMM's output instead of from the first layer's (imRes1 at :262) and has no activation;
+ * this entry point computes the composition its callers mean. */
+tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const tf_dense *W1, const tf_dense *W2, tf_dense *D,
+                            tf_schedule *s1, tf_schedule *s2, tf_dense *hidden, unsigned flags, void *stream);
 
 /* Unfused building blocks, the reference's in-process baselines:
  * Y = A * X   (swiftware::sparse::spmmCsrParallel<float>, fusion/src/SpMM_SpMM.cpp:37-55) */

@@ -143,3 +143,79 @@ def test_launch_times_and_second_stream(gpu, tf, orc):
     for _ in range(3):                                       # replays keep giving the same bits
         tf.gemm_spmm(Ah, Bd, Wd, D2, S)
         assert np.array_equal(D2.to_numpy(), a)
+
+
+def test_two_gcn_layers_in_one_call(gpu, tf, orc):
+    """tf_gcn_two_layers against the oracle's executor composed twice (ReLU between, on the host), with
+    and without the activation, with the hidden layer handed back, and with one schedule for both
+    layers when the widths agree."""
+    say("tf_gcn_two_layers")
+    cfg = tf.workloads.make_config(3, 0.03)
+    A = cfg["A"]
+    M = A.shape[0]
+    Ah = tf.CsrMatrix.from_scipy(A)
+    for K, H, N in ((256, 128, 64), (64, 64, 64), (40, 96, 32)):
+        X = tf.workloads.uniform((M, K), 101, 0.0, 1.0)
+        W1, W2 = tf.workloads.glorot(K, H, 102), tf.workloads.glorot(H, N, 103)
+        s1 = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=H, K=K)
+        s2 = s1 if (K, H) == (H, N) else tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=N, K=H)
+        sch = orc.unfused_schedule(M)
+        h_lin, _ = orc.gemm_spmm(A, X, W1, sch, nthreads=8)
+        for relu in (True, False):
+            h = np.maximum(h_lin, 0.0) if relu else h_lin
+            want, _ = orc.gemm_spmm(A, h, W2, sch, nthreads=8)
+            D = tf.DenseMatrix(M, N); D.fill(float("nan"))
+            hid = tf.DenseMatrix(M, H); hid.fill(float("nan"))
+            tf.gcn_two_layers(Ah, tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W1), tf.DenseMatrix.from_numpy(W2), D,
+                              s1, s2, relu=relu, hidden=hid)
+            assert orc.rel_err(hid.to_numpy(), h) <= TOL and orc.rel_err(D.to_numpy(), want) <= TOL, (K, H, N, relu)
+            D2 = tf.DenseMatrix(M, N); D2.fill(float("nan"))
+            tf.gcn_two_layers(Ah, tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W1), tf.DenseMatrix.from_numpy(W2), D2,
+                              s1, s2, relu=relu)          # hidden layer in the schedule's own buffer
+            assert np.array_equal(D2.to_numpy(), D.to_numpy())
+    with pytest.raises(tf.TileFusionError) as e:               # schedules in the wrong order
+        tf.gcn_two_layers(Ah, tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W1), tf.DenseMatrix.from_numpy(W2), D, s2, s1)
+    assert e.value.status == -4
+
+
+def test_remainder_rows_in_list_order(gpu, tf, orc):
+    """Reordered adjacency: remainder rows stored side by side in the order of the row list give the same
+    bits as the same rows read from A's arrays in place, for both executors, for an uploaded matrix (values
+    copied once) and after its values changed in a new upload (copied again)."""
+    say("reordered adjacency for remainder rows")
+    cfg = tf.workloads.make_config(3, 0.05)
+    A, B, W = cfg["A"], cfg["B"], cfg["C"]
+    M = A.shape[0]
+    Bd, Wd = tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W)
+    want, _ = orc.gemm_spmm(A, B, W, orc.unfused_schedule(M), nthreads=8)
+    outs = []
+    for ra in (0, -1):
+        Ah = tf.CsrMatrix.from_scipy(A)
+        S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=cfg["N"], K=cfg["K"], reorder_adjacency=ra)
+        S.validate()
+        assert S.info()["n_remainder_rows"] == M
+        D = tf.DenseMatrix(M, cfg["N"]); D.fill(float("nan"))
+        tf.gemm_spmm(Ah, Bd, Wd, D, S)
+        tf.gemm_spmm(Ah, Bd, Wd, D, S)                       # second call: values already in list order
+        outs.append(D.to_numpy())
+        assert orc.rel_err(outs[-1], want) <= TOL
+        A2 = A.copy(); A2.data = A.data * np.float32(0.5)    # same pattern, other values, new upload
+        Ah2 = tf.CsrMatrix.from_scipy(A2)
+        tf.gemm_spmm(Ah2, Bd, Wd, D, S)
+        assert orc.rel_err(D.to_numpy(), 0.5 * want) <= TOL
+    assert np.array_equal(outs[0], outs[1])
+    # SpMM-SpMM on a scrambled band: nothing fuses, every row is a remainder row in length-class order
+    Sm = tf.workloads.banded_random(20000, 32, 16, seed=3)
+    p = np.random.default_rng(4).permutation(20000)
+    Sm = sp.csr_matrix(Sm[p, :][:, p]); Sm.sort_indices()
+    Sm = sp.csr_matrix((Sm.data.astype(np.float32), Sm.indices.astype(np.int32), Sm.indptr.astype(np.int32)), shape=Sm.shape)
+    Cd = tf.workloads.uniform((20000, 64), 5)
+    Sh = tf.CsrMatrix.from_scipy(Sm)
+    got = []
+    for ra in (0, -1):
+        S = tf.inspector(Sh, 1, op=tf.OP_SPMM_SPMM, N=64, reorder_adjacency=ra)
+        S.validate()
+        D = tf.DenseMatrix(20000, 64)
+        tf.spmm_spmm(Sh, Sh, tf.DenseMatrix.from_numpy(Cd), D, S)
+        got.append(D.to_numpy())
+    assert np.array_equal(got[0], got[1]) and np.array_equal(got[0], oracle_spmm_spmm(orc, Sm, Sm, Cd))

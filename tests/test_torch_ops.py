@@ -149,3 +149,30 @@ def test_layer_written_like_the_reference(gpu, tf):
         opt.step()
         losses.append(float(loss.detach()))
     assert losses[-1] < losses[0]
+
+
+@pytest.mark.gpu
+def test_two_layer_forward_op(gpu, tf):
+    """sw_gcn.fusedGCN: both layers in one call with the hidden layer kept on the device, against
+    float64; and with gradients wanted, against dense autograd."""
+    print("sw_gcn fusedGCN", flush=True)
+    n = 3000
+    A = tf.workloads.erdos_renyi_gcn(n, 8.0, seed=29)
+    adj = csr_tensor(A, "cuda")
+    g = torch.Generator().manual_seed(7)
+    for in_dim, hid, out_dim in ((64, 64, 32), (50, 40, 7), (128, 128, 128)):
+        x0 = torch.rand(n, in_dim, generator=g)
+        w1 = torch.rand(hid, in_dim, generator=g) - 0.5
+        w2 = torch.rand(out_dim, hid, generator=g) - 0.5
+        Ad = A.astype(np.float64)
+        want = Ad @ (np.maximum(Ad @ (x0.double().numpy() @ w1.double().numpy().T), 0.0) @ w2.double().numpy().T)
+        with torch.no_grad():
+            got = torch.ops.sw_gcn.fusedGCN(adj, x0.cuda(), w1.cuda(), w2.cuda(), 8)
+        assert got.shape == (n, out_dim) and rel_err(got, want) <= TOL, (in_dim, hid, out_dim)
+    xd, w1d, w2d = x0.double().requires_grad_(), w1.double().requires_grad_(), w2.double().requires_grad_()
+    Adt = torch.tensor(A.toarray(), dtype=torch.float64)
+    go = torch.rand(n, out_dim, generator=g) - 0.5
+    (Adt @ ((Adt @ (xd @ w1d.t())).relu() @ w2d.t())).backward(go.double())
+    x, a1, a2 = x0.cuda().requires_grad_(), w1.cuda().requires_grad_(), w2.cuda().requires_grad_()
+    torch.ops.sw_gcn.fusedGCN(adj, x, a1, a2, 8).backward(go.cuda())
+    assert rel_err(x.grad, xd.grad.numpy()) <= TOL and rel_err(a1.grad, w1d.grad.numpy()) <= TOL and rel_err(a2.grad, w2d.grad.numpy()) <= TOL

@@ -13,6 +13,7 @@ OP_SPMM_SPMM = 0
 OP_GEMM_SPMM = 1
 ACCUMULATE = 1
 SECOND_STREAM = 2
+RELU = 4
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -39,7 +40,7 @@ class InspectOpts(C.Structure):
                 ("compute_units", C.c_int), ("inner_Ap", C.POINTER(C.c_int)), ("inner_Ai", C.POINTER(C.c_int)),
                 ("inner_cols", C.c_int), ("strip_cols", C.c_int), ("xcd_chunk_rows", C.c_int), ("wide_strips", C.c_int), ("long_row_partition", C.c_int),
                 ("march", C.c_int), ("grid_nx", C.c_int), ("grid_ny", C.c_int), ("grid_nz", C.c_int),
-                ("march_tile_x", C.c_int), ("march_tile_y", C.c_int)]
+                ("march_tile_x", C.c_int), ("march_tile_y", C.c_int), ("reorder_adjacency", C.c_int)]
 
 
 class ScheduleInfo(C.Structure):
@@ -117,6 +118,7 @@ SIGNATURES = {
     "tf_noalloc_scratch_bytes": (C.c_size_t, []),
     "tf_spmm_spmm": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
     "tf_gemm_spmm": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
+    "tf_gcn_two_layers": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
     "tf_spmm": (C.c_int, [_VP, _VP, _VP, C.c_uint, _VP]),
     "tf_gemm": (C.c_int, [_VP, _VP, _VP, _VP]),
 }
@@ -333,7 +335,7 @@ class FusedSchedule:
 
 def inspector(A, NumThreads=1, *, op, N, K=0, lds_budget_bytes=0, tile_rows=0, max_redundancy=0.0,
               long_row_nnz=0, compute_units=0, inner=None, strip_cols=0, xcd_chunk_rows=0, wide_strips=0, long_row_partition=0,
-              march=0, grid=None, march_tile=None):
+              march=0, grid=None, march_tile=None, reorder_adjacency=0):
     """swiftware::fusion::inspector(A, NumThreads) (README.md:25).  NumThreads is accepted
     for signature parity and unused: the schedule is sized by the GPU, not by a CPU
     thread count.  The extra keywords are the parameters the reference passes to its
@@ -344,7 +346,7 @@ def inspector(A, NumThreads=1, *, op, N, K=0, lds_budget_bytes=0, tile_rows=0, m
     o = InspectOpts(C.sizeof(InspectOpts), op, N, K, lds_budget_bytes, tile_rows, max_redundancy, long_row_nnz, compute_units,
                     inner._pp if inner is not None else None, inner._pi if inner is not None else None,
                     inner.N if inner is not None else 0, strip_cols, xcd_chunk_rows, wide_strips, long_row_partition,
-                    march, *(grid or (0, 0, 0)), *(march_tile or (0, 0)))
+                    march, *(grid or (0, 0, 0)), *(march_tile or (0, 0)), reorder_adjacency)
     h = _VP()
     _check(lib().tf_inspect(A.M, A.N, A._pp, A._pi, C.byref(o), C.byref(h)))
     return FusedSchedule(h, A, inner)
@@ -364,6 +366,13 @@ def gemm_spmm(A, B, Cm, D, schedule, NumThreads=1, *, accumulate=False, stream=N
     _check(lib().tf_gemm_spmm(A.to_device().h, B.h, Cm.h, D.h, schedule.h,
                               (ACCUMULATE if accumulate else 0) | (SECOND_STREAM if second_stream else 0),
                               stream.h if stream else None))
+
+
+def gcn_two_layers(A, X, W1, W2, D, s1, s2, *, relu=True, hidden=None, accumulate=False, stream=None):
+    """D = A * (act(A * (X * W1)) * W2), the two-layer forward of the reference's end-to-end model
+    (binding-project/gcn-e2e-training/FusedGCNModule.py:14-18); the hidden layer stays on the device."""
+    _check(lib().tf_gcn_two_layers(A.to_device().h, X.h, W1.h, W2.h, D.h, s1.h, s2.h, hidden.h if hidden is not None else None,
+                                   (RELU if relu else 0) | (ACCUMULATE if accumulate else 0), stream.h if stream else None))
 
 
 def spmm_spmm_noalloc(A, B, Cm, D, *, accumulate=False, stream=None):

@@ -50,6 +50,12 @@ struct DeviceSchedule {
   int *seg_ptr = nullptr, *ent_src = nullptr, *ent_pos = nullptr, *seg_col = nullptr, *lrow_seg = nullptr;  // column-partitioned long rows
   float *seg_val = nullptr;  // A's values in the order of the regrouped entries
   unsigned long long seg_val_serial = 0;  // the uploaded matrix they were taken from (0: none)
+  // the short remainder rows stored in the order of the row list: row pointers, columns, where each
+  // value comes from in A's array, and the values themselves (of the uploaded matrix rem_val_serial)
+  int *rem_ptr = nullptr, *rem_col = nullptr, *rem_src = nullptr;
+  float *rem_val = nullptr;
+  unsigned long long rem_val_serial = 0;
+  float *hidden = nullptr;   // tf_gcn_two_layers: the first layer's output, L x K of this (second-layer) schedule
   float *Bpad = nullptr;     // M x K' and K' x N copies of B and C, zero-padded, when K is not a multiple of 8
   float *Cpad = nullptr;
   // marching runs: the schedule's lists, and the ELL rows with the operands' values filled in
@@ -78,7 +84,8 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *, const int *, int, c
                                            const float *, int, const float *, const int *, const int *,
                                            const float *, int, float *, int, int, int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
-                            float *, int, int, int, int, hipStream_t);
+                            float *, int, int, int, int, hipStream_t, int compact = 0);
+hipError_t launch_gather_values(const int *, const float *, float *, int, hipStream_t);
 hipError_t launch_march_fill(const int *, const int *, const float *, const float *, int *, size_t, hipStream_t);
 hipError_t launch_fused_spmm_spmm_march(const int *, int, const int *, const int *, const int *, const int *, const int *,
                                         const float *, float *, float *, int, int, int, int, int, int, hipStream_t);
@@ -95,6 +102,7 @@ hipError_t launch_fused_gemm_spmm_stream(const TileDesc *, int, const int *, con
 hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t);
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 hipError_t launch_pad(const float *, int, int, float *, int, int, hipStream_t);
+hipError_t launch_relu(float *, size_t, hipStream_t);
 
 // An intermediate larger than the 256 MB last-level cache is gone from it before its readers
 // come: such rows leave through streaming stores.
@@ -137,7 +145,8 @@ void release_device_schedule(DeviceSchedule *d) {
   (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows); (void)hipFree(d->seg_groups);
   (void)hipFree(d->seg_ptr); (void)hipFree(d->ent_src); (void)hipFree(d->ent_pos); (void)hipFree(d->seg_col); (void)hipFree(d->lrow_seg); (void)hipFree(d->seg_val);
   (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
-  (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad);
+  (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad); (void)hipFree(d->hidden);
+  (void)hipFree(d->rem_ptr); (void)hipFree(d->rem_col); (void)hipFree(d->rem_src); (void)hipFree(d->rem_val);
   (void)hipFree(d->m_runs); (void)hipFree(d->m_row_ptr); (void)hipFree(d->m_load_ptr); (void)hipFree(d->m_load);
   (void)hipFree(d->m_row_out); (void)hipFree(d->m_ell_off); (void)hipFree(d->m_ell_src); (void)hipFree(d->m_ell); (void)hipFree(d->m_trash);
   if (d->side) (void)hipStreamDestroy(d->side);
@@ -198,6 +207,15 @@ static tf_status ensure_device(tf_schedule *s) {
   if (!rc) rc = upload_vec(s->launch_step, &d->step_begin);
   if (!rc) rc = upload_vec(s->step_ptr, &d->step_ptr);
   if (!rc) rc = upload_vec(s->fused_rec, &d->fused_rec);
+  if (!rc && !s->rem_ptr.empty()) {
+    rc = upload_vec(s->rem_ptr, &d->rem_ptr);
+    if (!rc) rc = upload_vec(s->rem_col, &d->rem_col);
+    if (!rc) rc = upload_vec(s->rem_src, &d->rem_src);
+    if (!rc) {
+      hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->rem_val), std::max<size_t>(s->rem_src.size(), 1) * sizeof(float));
+      if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(reordered rows)");
+    }
+  }
   if (!rc) rc = upload_vec(s->long_chunks, &d->long_chunks);
   if (!rc) rc = upload_vec(s->long_rows, &d->long_rows);
   if (!rc && s->long_part) {
@@ -286,7 +304,18 @@ static tf_status run_hot_segments(const tf_csr *A, tf_schedule *s, hipStream_t s
 static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int accumulate, bool hot_on_side, hipStream_t st) {
   DeviceSchedule *d = s->dev;
   const int N = s->opts.N;
-  if (!s->rem_rows.empty()) {
+  if (!s->rem_rows.empty() && !s->rem_ptr.empty()) {
+    // The rows in the order of the list, entries side by side -- the reference's reordered adjacency
+    // (createReorderedAdj, GCN_Single_Layer_SP_Demo_Utils.h:618-653; executor at
+    // GCN_Layer_MKL_Forward_Utils.h:294-373).  The values are copied on the first call with an uploaded
+    // matrix, whose device arrays never change, and on every call with a wrapped one.
+    if (!(A->serial != 0 && d->rem_val_serial == A->serial))
+      TF_PHASE(s, "gather_values_kernel", st, launch_gather_values(d->rem_src, A->x, d->rem_val, (int)s->rem_src.size(), st));
+    d->rem_val_serial = A->serial;
+    TF_PHASE(s, "spmm_rows_kernel (short remainder rows)", st,
+             launch_spmm_rows(d->rem_rows, (int)s->rem_rows.size(), d->rem_ptr, d->rem_col, d->rem_val, d->inter, D->d, N, accumulate,
+                              s->xcd_chunk_rows, /*streaming=*/1, st, /*compact=*/1));
+  } else if (!s->rem_rows.empty()) {
     // identity list: no indirection needed
     TF_PHASE(s, "spmm_rows_kernel (short remainder rows)", st,
              launch_spmm_rows(s->rem_identity ? nullptr : d->rem_rows, (int)s->rem_rows.size(), A->p, A->i,
@@ -699,6 +728,30 @@ extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_d
     }
   }
   return tf::run_remainder(A, D, s, acc, overlap && !s->plain_rows.empty(), st);
+}
+
+extern "C" tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const tf_dense *W1, const tf_dense *W2, tf_dense *D,
+                                       tf_schedule *s1, tf_schedule *s2, tf_dense *hidden, unsigned flags, void *stream) {
+  if (!A || !X || !W1 || !W2 || !D || !s1 || !s2) return fail(TF_EINVAL, "tf_gcn_two_layers: null argument");
+  if (A->M != A->N) return fail(TF_EINVAL, "tf_gcn_two_layers: A must be square (it is %d x %d)", A->M, A->N);
+  const int H = W1->N;
+  if (W2->M != H) return fail(TF_EINVAL, "tf_gcn_two_layers: W1 has %d columns, W2 has %d rows", H, W2->M);
+  if (hidden && (hidden->M != A->M || hidden->N != H))
+    return fail(TF_EINVAL, "tf_gcn_two_layers: hidden is %d x %d, expected %d x %d", hidden->M, hidden->N, A->M, H);
+  tf_dense h;
+  h.M = A->M; h.N = H; h.owns = false;
+  if (hidden) {
+    h.d = hidden->d;
+  } else {
+    if (tf_status rc = tf::ensure_device(s2)) return rc;
+    if (!s2->dev->hidden) TF_HIP(hipMalloc(reinterpret_cast<void **>(&s2->dev->hidden), (size_t)A->M * H * sizeof(float)));
+    h.d = s2->dev->hidden;
+  }
+  if (s2->user_K != H) return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule was built for K = %d, the hidden layer has %d columns", s2->user_K, H);
+  // first layer (its schedule is checked against X and W1 there), activation, second layer
+  if (tf_status rc = tf_gemm_spmm(A, X, W1, &h, s1, flags & TF_SECOND_STREAM, stream)) return rc;
+  if (flags & TF_RELU) TF_HIP(tf::launch_relu(h.d, (size_t)h.M * h.N, static_cast<hipStream_t>(stream)));
+  return tf_gemm_spmm(A, &h, W2, D, s2, flags & (TF_ACCUMULATE | TF_SECOND_STREAM), stream);
 }
 
 // ---- benchmark aid: per-launch times of the last executor call -------------------------

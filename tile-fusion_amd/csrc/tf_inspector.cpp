@@ -580,6 +580,17 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       for (auto &v : byc) S->rem_rows.insert(S->rem_rows.end(), v.begin(), v.end());
       S->rem_identity = (int)S->rem_rows.size() == L;
       for (int q = 0; q < L && S->rem_identity; ++q) S->rem_identity = (S->rem_rows[q] == q);
+      // Reordered adjacency (createReorderedAdj, GCN_Single_Layer_SP_Demo_Utils.h:618-653): a list that is
+      // not simply all rows in order gets its rows stored side by side in list order, so that a
+      // workgroup reads one stretch of columns and values instead of one stretch per row.
+      if (!S->rem_identity && !S->rem_rows.empty() && o.reorder_adjacency >= 0) {
+        S->rem_ptr.reserve(S->rem_rows.size() + 1);
+        S->rem_ptr.push_back(0);
+        for (int i : S->rem_rows) {
+          for (int k = Ap[i]; k < Ap[i + 1]; ++k) { S->rem_col.push_back(Ai[k]); S->rem_src.push_back(k); }
+          S->rem_ptr.push_back((int)S->rem_col.size());
+        }
+      }
     }
 
     // Row kernels: workgroup ids go to the XCDs round-robin, which keeps all eight of them in the
@@ -709,6 +720,7 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   ws += (long long)s->long_chunks.size() * s->opts.N * 4;
   if (s->long_part) ws += ((long long)s->seg_ptr.size() - 1 + (long long)s->seg_groups.size()) * s->opts.N * 4 + (long long)s->seg_src.size() * 4;  // partial sums, regrouped values
   if (s->user_K != s->opts.K) ws += ((long long)s->M + s->opts.N) * s->opts.K * 4;  // padded copies of B and C
+  ws += (long long)s->rem_ptr.size() * 4 + (long long)s->rem_col.size() * 12;       // remainder rows in list order
   info->workspace_bytes = ws;
   return TF_OK;
 }
@@ -802,6 +814,17 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
         return tf::fail(TF_ESCHEDULE, "remainder row %d reads intermediate row %d that no tile stores", i, Ai[k]);
     return TF_OK;
   };
+  if (!s->rem_ptr.empty()) {  // the rows of the list stored in list order must be A's rows, entry for entry
+    if (s->rem_ptr.size() != s->rem_rows.size() + 1 || s->rem_ptr[0] != 0 || s->rem_ptr.back() != (int)s->rem_col.size() || s->rem_src.size() != s->rem_col.size())
+      return tf::fail(TF_ESCHEDULE, "remainder rows in list order: bad tables");
+    for (size_t q = 0; q < s->rem_rows.size(); ++q) {
+      const int i = s->rem_rows[q];
+      if (i < 0 || i >= L || s->rem_ptr[q + 1] - s->rem_ptr[q] != Ap[i + 1] - Ap[i])
+        return tf::fail(TF_ESCHEDULE, "remainder rows in list order: row %d has another length than in A", i);
+      for (int k = Ap[i], e = s->rem_ptr[q]; k < Ap[i + 1]; ++k, ++e)
+        if (s->rem_src[e] != k || s->rem_col[e] != Ai[k]) return tf::fail(TF_ESCHEDULE, "remainder rows in list order: row %d differs from A's", i);
+    }
+  }
   for (int i : s->rem_rows) {
     if (done[i]++) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled twice", i);
     if (Ap[i + 1] - Ap[i] > s->opts.long_row_nnz)

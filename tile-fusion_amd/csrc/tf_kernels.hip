@@ -631,7 +631,7 @@ template <int V, int LPR>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
     const int *__restrict__ rows, int n_rows, int n_blocks, int per_xcd, const int *__restrict__ Ap,
     const int *__restrict__ Ai, const float *__restrict__ Ax, const float *__restrict__ X, int ldx,
-    float *__restrict__ Y, int N, int accumulate, int streaming) {
+    float *__restrict__ Y, int N, int accumulate, int streaming, int compact) {
   constexpr int G = kBlock / LPR;
   const int group = threadIdx.x / LPR, glane = threadIdx.x % LPR;
   const int b = xcd_contiguous(blockIdx.x, per_xcd);
@@ -639,7 +639,10 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
   const int q = b * G + group;
   if (q >= n_rows) return;  // whole lane groups leave together
   const int i = rows ? rows[q] : q;
-  const int kb = Ap[i], ke = Ap[i + 1];
+  // compact: the CSR arrays hold the listed rows only, in the order of the list (the reference's
+  // reordered adjacency: consumer rows stored in schedule order), so row q of them is row rows[q] of Y
+  const int r = compact ? q : i;
+  const int kb = Ap[r], ke = Ap[r + 1];
   for (int c0 = 0; c0 < N; c0 += LPR * V) {
     const int coff = c0 + glane * V;
     const bool ok = coff < N;
@@ -698,6 +701,11 @@ __global__ __launch_bounds__(kBlock) void long_row_reduce_kernel(const LongRow *
   }
 }
 
+// out[i] = val[src[i]]: the values of the rows of a list, in the order of the list.
+__global__ void gather_values_kernel(const int *__restrict__ src, const float *__restrict__ val, float *__restrict__ out, int n) {
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) out[i] = val[src[i]];
+}
+
 // Column-partitioned long rows: out[pos[i]] = val[src[i]] puts the values of A into the order of
 // the regrouped entries (src ascending: the reads walk A's array once, the writes fall into
 // nine ascending streams), and Y[row] (+)= the row's segment sums, added in the order of its list.
@@ -743,6 +751,16 @@ __global__ void pad_kernel(const float *__restrict__ src, int src_rows, int ld_s
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
     const int r = (int)(i / ld_dst), c = (int)(i % ld_dst);
     dst[i] = (r < src_rows && c < ld_src) ? src[(size_t)r * ld_src + c] : 0.f;
+  }
+}
+
+// p = max(p, 0), four values per thread (n is a multiple of 4: the kernels' N is).
+__global__ void relu_kernel(float *__restrict__ p, size_t n4) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
+    fvec<4> v = *reinterpret_cast<const fvec<4> *>(p + 4 * i);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v.v[c] = fmaxf(v.v[c], 0.f);
+    *reinterpret_cast<fvec<4> *>(p + 4 * i) = v;
   }
 }
 
@@ -1813,7 +1831,7 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *tiles, const int *win
 
 hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const int *Ai, const float *Ax,
                             const float *X, float *Y, int N, int accumulate, int xcd_chunk_rows,
-                            int streaming, hipStream_t st) {
+                            int streaming, hipStream_t st, int compact) {
   if (n_rows <= 0) return hipSuccess;
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
@@ -1822,7 +1840,7 @@ hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const in
   const int bpc = xcd_chunk_rows == 0 ? 0 : chunk_bpc(n_blocks, xcd_chunk_rows > 0 ? std::max(1, xcd_chunk_rows / G) : 0);
 #define CALL(V_, L_)                                                                                   \
   hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(grid_chunked(n_blocks, bpc)), dim3(kBlock), 0, st, \
-                     rows, n_rows, n_blocks, bpc, Ap, Ai, Ax, X, N, Y, N, accumulate, streaming)
+                     rows, n_rows, n_blocks, bpc, Ap, Ai, Ax, X, N, Y, N, accumulate, streaming, compact)
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
 #undef CALL
   return hipGetLastError();
@@ -1853,6 +1871,13 @@ hipError_t launch_scatter_values(const int *ent_src, const int *ent_pos, const f
   if (n_entries <= 0) return hipSuccess;
   const int blocks = std::min((n_entries + kBlock - 1) / kBlock, 65536);
   hipLaunchKernelGGL(scatter_values_kernel, dim3(blocks), dim3(kBlock), 0, st, ent_src, ent_pos, Ax, seg_val, n_entries);
+  return hipGetLastError();
+}
+
+hipError_t launch_gather_values(const int *src, const float *Ax, float *out, int n, hipStream_t st) {
+  if (n <= 0) return hipSuccess;
+  const int blocks = std::min((n + kBlock - 1) / kBlock, 65536);
+  hipLaunchKernelGGL(gather_values_kernel, dim3(blocks), dim3(kBlock), 0, st, src, Ax, out, n);
   return hipGetLastError();
 }
 
@@ -1998,6 +2023,14 @@ hipError_t launch_pad(const float *src, int src_rows, int ld_src, float *dst, in
   if (n == 0) return hipSuccess;
   const int blocks = (int)std::min<size_t>((n + kBlock - 1) / kBlock, 65536);
   hipLaunchKernelGGL(pad_kernel, dim3(blocks), dim3(kBlock), 0, st, src, src_rows, ld_src, dst, rows, ld_dst);
+  return hipGetLastError();
+}
+
+hipError_t launch_relu(float *p, size_t n, hipStream_t st) {
+  if (n == 0) return hipSuccess;
+  if (n % 4 != 0) return hipErrorInvalidValue;
+  const int blocks = (int)std::min<size_t>((n / 4 + 255) / 256, 65536);
+  hipLaunchKernelGGL(relu_kernel, dim3(blocks), dim3(256), 0, st, p, n / 4);
   return hipGetLastError();
 }
 

@@ -303,6 +303,40 @@ def unfused_gcn_forward(Adj, Feature, Weight, NumThreads):
     return _Unfused.apply(Adj, Feature, Weight)
 
 
+def _two_layers(ctx, X, W1kn, W2kn, relu):
+    """ctx.A @ (act(ctx.A @ (X @ W1kn)) @ W2kn) through tf_gcn_two_layers; the hidden layer never leaves the device."""
+    _require_gpu(X, W1kn, W2kn)
+    M, K = X.shape
+    H, N = W1kn.shape[1], W2kn.shape[1]
+    if ctx.shape[0] != ctx.shape[1] or ctx.shape[1] != M or W1kn.shape[0] != K or W2kn.shape[0] != H:
+        raise RuntimeError(f"sw_gcn: shapes do not chain: Adj {ctx.shape}, Feature {tuple(X.shape)}, weights {tuple(W1kn.shape)}, {tuple(W2kn.shape)}")
+    Hp, Np = _pad_to(H, 32), _pad_to(N, 32)
+    if Hp > _MAX_N or Np > _MAX_N:  # wider layers go through the single-layer path, which splits columns
+        h = _gemm_spmm(ctx, X, W1kn)
+        return _gemm_spmm(ctx, h.relu_() if relu else h, W2kn)
+    X = X.to(torch.float32).contiguous()
+    # zero columns of W1 give zero hidden columns (also after ReLU), which meet zero rows of W2
+    W1p = torch.nn.functional.pad(W1kn.to(torch.float32), (0, Hp - H)).contiguous()
+    W2p = torch.nn.functional.pad(W2kn.to(torch.float32), (0, Np - N, 0, Hp - H)).contiguous()
+    out = torch.empty((M, Np), dtype=torch.float32, device=X.device)
+    s1, s2 = ctx.schedule(K, Hp), ctx.schedule(Hp, Np)
+    with _Dense(X) as xb, _Dense(W1p) as w1, _Dense(W2p) as w2, _Dense(out) as ob:
+        _b._check(_b.lib().tf_gcn_two_layers(ctx.h, xb, w1, w2, ob, s1.h, s2.h, None, _b.RELU if relu else 0, _stream()))
+    return out if Np == N else out[:, :N].contiguous()
+
+
+def fusedGCN(Adj, Feature, Weight1, Weight2, NumThreads):
+    """Two layers with a ReLU between, Adj @ (relu(Adj @ (Feature @ Weight1^T)) @ Weight2^T), weights [out, in]:
+    the forward of the reference's end-to-end model (gcn-e2e-training/FusedGCNModule.py:14-18) and the
+    composition its unregistered fusedGCN (binding-project/src/Functions.cpp:228-290) stands for.  When a
+    gradient is wanted the two layers run as two fusedGeMMSpMM calls, whose backward passes exist."""
+    del NumThreads
+    _require_gpu(Adj, Feature, Weight1, Weight2)
+    if torch.is_grad_enabled() and (Feature.requires_grad or Weight1.requires_grad or Weight2.requires_grad):
+        return _FusedGeMMSpMM.apply(Adj, _FusedGeMMSpMM.apply(Adj, Feature, Weight1).relu(), Weight2)
+    return _two_layers(_ctx(Adj), Feature, Weight1.t(), Weight2.t(), True)
+
+
 SCHEMAS = {
     "inspect": "(Tensor Adj, int MTileSize) -> Tensor[]",
     "inspect_vt_ro": "(Tensor Adj, int InDim, int OutDim, int CacheSize, int NumThreads) -> Tensor[]",
@@ -312,6 +346,7 @@ SCHEMAS = {
     "geMMSpMM_f_bw": "(Tensor Adj, Tensor Feature, Tensor Weight, Tensor[] Schedule, int NumThreads) -> Tensor",
     "cachedSpMMGeMM": "(Tensor AF, Tensor Weight, int NumThreads) -> Tensor",
     "unfused_gcn_forward": "(Tensor Adj, Tensor Feature, Tensor Weight, int NumThreads) -> Tensor",
+    "fusedGCN": "(Tensor Adj, Tensor Feature, Tensor Weight1, Tensor Weight2, int NumThreads) -> Tensor",
 }
 
 _library = torch.library.Library("sw_gcn", "DEF")
