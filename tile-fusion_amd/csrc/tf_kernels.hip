@@ -983,8 +983,40 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
   // every wavefront walks one contiguous run of row blocks; run lengths differ by at most one
   // and the longer runs are spread evenly over the compute units
   const int gw = blockIdx.x * (kGemmBlock / 64) + wave;
-  const int run0 = (int)((long long)gw * nrb / total_waves);
-  const int run_end = (int)((long long)(gw + 1) * nrb / total_waves);
+  // When the blocks do not divide among the wavefronts, the odd ones are cut into their NB column blocks
+  // and those are dealt out instead: a wavefront with one more whole block than the others would set
+  // the kernel's time (200,000 rows are 6,250 blocks for 2,048 wavefronts: four blocks against three
+  // and a quarter).  Not when the odd blocks are so many that a wavefront would get all columns anyway.
+  const int whole = nrb / total_waves, odd = nrb - whole * total_waves;
+  const int tail_per_wave = (odd * NB + total_waves - 1) / total_waves;
+  const bool split_tail = odd > 0 && tail_per_wave < NB;
+  const int run0 = split_tail ? gw * whole : (int)((long long)gw * nrb / total_waves);
+  const int run_end = split_tail ? run0 + whole : (int)((long long)(gw + 1) * nrb / total_waves);
+  if (split_tail) {
+    const int n_tail = odd * NB;
+    for (int t = gw * tail_per_wave; t < min(n_tail, (gw + 1) * tail_per_wave); ++t) {
+      const int rb = whole * total_waves + t / NB, nb = t % NB;
+      const int pos = min(rb * 32 + j, n_rows - 1);
+      const float *p = X + (size_t)(LIST ? rows[pos] : pos) * K + 4 * h;
+      v16f acc1;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc1[r] = 0.f;
+      const float *wt = wlds + ((4 * h) * 32 + j) * NB + nb;  // element (k, nb*32 + j) sits at (k*32 + j)*NB + nb
+      fvec<4> a = *reinterpret_cast<const fvec<4> *>(p);
+      for (int st = 0; st < steps; ++st) {
+        const fvec<4> an = *reinterpret_cast<const fvec<4> *>(p + 8 * min(st + 1, steps - 1));
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[u], wt[(size_t)(8 * st + u) * 32 * NB], acc1, 0, 0, 0);
+        a = an;
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int x = rb * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+        if (x < n_rows) Y[(size_t)(LIST ? rows[x] : x) * N + nb * 32 + j] = acc1[r];
+      }
+    }
+  }
   for (int rb0 = run0; rb0 < run_end; rb0 += kGemmSeg) {
     const int rb_end = min(run_end, rb0 + kGemmSeg);
     if constexpr (LIST) {
@@ -1538,6 +1570,13 @@ __device__ __forceinline__ int opaque_mask(bool c) {
   return m;
 }
 
+// The lists are read once: streaming loads, so that they do not push the rows of C out of L2.
+__device__ __forceinline__ int4 load_streaming_i4(const int4 *p) {
+  typedef int i4 __attribute__((ext_vector_type(4)));
+  const i4 v = __builtin_nontemporal_load(reinterpret_cast<const i4 *>(p));
+  return make_int4(v[0], v[1], v[2], v[3]);
+}
+
 template <int G>
 __device__ __forceinline__ fvec<4> march_gather(const char *lane_base, int off) {
   return *reinterpret_cast<const fvec<4> *>(lane_base + quad_bcast<G>(off));
@@ -1617,7 +1656,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
       const int x = b0 + group + kMarchGroups * u, xc = max(min(x, b1 - 1), 0);
       const bool ok = x < b1;
       const int o = row_out[xc], m = opaque_mask(ok);
-      L.et[u] = ell[(size_t)xc * 4 + q];  // a group without a row recomputes another's, into the trash row
+      L.et[u] = load_streaming_i4(ell + (size_t)xc * 4 + q);  // a group without a row recomputes another's, into the trash row
       L.ot[u] = (o & m) | (~kMarchTrashOff & ~m);
     }
 #pragma unroll
@@ -1625,7 +1664,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
       const int x = b1 + group + kMarchGroups * u, xc = max(min(x, b2 - 1), 0);
       const bool ok = x < b2;
       const int o = row_out[xc], m = opaque_mask(ok);
-      L.ed[u] = ell[(size_t)xc * 4 + q];
+      L.ed[u] = load_streaming_i4(ell + (size_t)xc * 4 + q);
       L.od[u] = o | ~m;  // -1: no row
     }
     fetch_loads(it + 2, L.ll);
@@ -1637,6 +1676,8 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
     float *Tl = trash + glane * 4;
     auto issue = [&](MarchStage &S) {
 #pragma unroll
+      // (streaming loads measured faster than plain ones, 0.46 against 0.57 ms on the 128^3 grid, although a
+      // run's rows of C are its neighbours' halo rows an iteration or two later)
       for (int u = 0; u < kMarchLpg; ++u) S.c[u] = load_streaming4(Cl + (size_t)S.ll[u].x * N);
     };
     // One iteration.  `cur` holds its lists; `fut` is free and takes those of iteration it + 2.  Stage
