@@ -398,7 +398,8 @@ def main():
                    **head["schedule"], "kernels_per_step": len(head["kernels"]) or None,
                    "working_set_vs_llc": head["working_set_vs_llc"],
                    **({"reorder_s": round(reorder_s, 4)} if reorder_s is not None else {}),
-                   "rel_err_vs_f64": head["rel_err_vs_f64"], "rows_checked": head["rows_checked"], "device": dev["arch"]},
+                   "rel_err_vs_f64": head["rel_err_vs_f64"], "rows_checked": head["rows_checked"], "device": dev["arch"],
+                   "xcd_round_robin_verified": dev["xcd_round_robin"]},
     }
     dev_s = head["kernel_ms"] * 1e-3
     hbm = {"achieved": round(head["algorithmic_bytes"] / dev_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head["hbm_frac"]}

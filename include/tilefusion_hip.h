@@ -51,6 +51,10 @@ typedef struct {
   int clock_khz;
   size_t hbm_bytes;
   char arch[64];           /* "gfx950..."                                         */
+  int xcd_round_robin;     /* 1: a probe launch found workgroup b on the XCD of workgroup b mod xcds and
+                              those xcds distinct -- what the kernels that pin work to an XCD's L2 rely on
+                              (column-partitioned long rows, runs of neighbouring tiles); 0: it did not
+                              (results stay right, that locality is lost); -1: the probe could not run  */
 } tf_device_info;
 
 /* Selects the device for the calling thread and reports its properties.  Optional:
@@ -226,6 +230,10 @@ typedef struct {
      forwardForOneLayerFusedParallelSeparatedReorderedAdjVectorizedSP, GCN_Layer_MKL_Forward_Utils.h:294-373);
      -1 = the rows are read from A's arrays in place through the list. */
   int reorder_adjacency;
+  /* Column-partitioned long rows (long_row_partition): bytes of most-read intermediate rows dealt to each of
+     the 8 XCD partitions; default 12 MB, three times an XCD's L2 (the reads inside a partition are skewed
+     too, and its hottest rows are what stays). */
+  int hot_partition_bytes;
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;

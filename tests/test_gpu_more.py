@@ -219,3 +219,9 @@ def test_remainder_rows_in_list_order(gpu, tf, orc):
         tf.spmm_spmm(Sh, Sh, tf.DenseMatrix.from_numpy(Cd), D, S)
         got.append(D.to_numpy())
     assert np.array_equal(got[0], got[1]) and np.array_equal(got[0], oracle_spmm_spmm(orc, Sm, Sm, Cd))
+
+
+def test_device_reports_the_workgroup_to_xcd_mapping(gpu):
+    """tf_device_init probes what the XCD-pinned kernels rely on: workgroup b runs on XCD b mod 8."""
+    assert gpu["xcds"] == 8 and gpu["compute_units"] == 256 and gpu["wavefront"] == 64
+    assert gpu["xcd_round_robin"] == 1, gpu

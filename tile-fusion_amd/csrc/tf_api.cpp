@@ -103,6 +103,7 @@ hipError_t launch_gemm(const float *, const float *, float *, const int *, int, 
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 hipError_t launch_pad(const float *, int, int, float *, int, int, hipStream_t);
 hipError_t launch_relu(float *, size_t, hipStream_t);
+hipError_t launch_xcd_probe(int *, int, hipStream_t);
 
 // An intermediate larger than the 256 MB last-level cache is gone from it before its readers
 // come: such rows leave through streaming stores.
@@ -412,6 +413,21 @@ extern "C" tf_status tf_device_init(int device, tf_device_info *info) {
     info->clock_khz = p.clockRate;
     info->hbm_bytes = p.totalGlobalMem;
     std::snprintf(info->arch, sizeof(info->arch), "%s", p.gcnArchName);
+    // Workgroup b of a launch is expected on XCD b mod 8: checked once here, on 64 workgroups.
+    info->xcd_round_robin = -1;
+    int *probe = nullptr, host[64];
+    if (hipMalloc(reinterpret_cast<void **>(&probe), sizeof(host)) == hipSuccess) {
+      if (tf::launch_xcd_probe(probe, 64, nullptr) == hipSuccess &&
+          hipMemcpy(host, probe, sizeof(host), hipMemcpyDeviceToHost) == hipSuccess) {
+        bool ok = true;
+        for (int b = 0; b < 64 && ok; ++b) ok = host[b] == host[b % info->xcds];
+        for (int a = 0; a < info->xcds && ok; ++a)
+          for (int b = a + 1; b < info->xcds && ok; ++b) ok = host[a] != host[b];
+        info->xcd_round_robin = ok ? 1 : 0;
+      }
+      (void)hipFree(probe);
+    }
+    (void)hipGetLastError();
   }
   return TF_OK;
 }

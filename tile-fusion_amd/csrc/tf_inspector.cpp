@@ -463,7 +463,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
                         (o.long_row_partition == 0 && long_nnz >= (1 << 20) && (long long)M * o.N * 4 > (64LL << 20));
       // (three times an L2's 4 MB measured best on the R-MAT graph: 2.68 ms per step with 4 MB, 2.54 with 12 or
       // 16 MB, 2.60 with 32 MB -- the reads inside a partition are skewed too, and its hottest rows are what stays)
-      const int part_rows = std::max(64, (12 << 20) / (o.N * 4));
+      const int part_rows = std::max(64, (o.hot_partition_bytes > 0 ? o.hot_partition_bytes : (12 << 20)) / (o.N * 4));
       if (want && !S->long_rows.empty() && long_nnz < INT_MAX) {
         constexpr int kParts = 8, kSegMax = 64, kPad = 256, kMinGroup = 4;
         std::vector<int> reads(M, 0);

@@ -764,6 +764,11 @@ __global__ void relu_kernel(float *__restrict__ p, size_t n4) {
   }
 }
 
+// out[workgroup] = the XCD it runs on (hardware register XCC_ID, bits 3:0).
+__global__ void xcd_probe_kernel(int *__restrict__ out) {
+  if (threadIdx.x == 0) out[blockIdx.x] = (int)__builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11));
+}
+
 __global__ void fill_kernel(float *__restrict__ p, size_t n, float v) {
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
 }
@@ -2072,6 +2077,11 @@ hipError_t launch_relu(float *p, size_t n, hipStream_t st) {
   if (n % 4 != 0) return hipErrorInvalidValue;
   const int blocks = (int)std::min<size_t>((n / 4 + 255) / 256, 65536);
   hipLaunchKernelGGL(relu_kernel, dim3(blocks), dim3(256), 0, st, p, n / 4);
+  return hipGetLastError();
+}
+
+hipError_t launch_xcd_probe(int *out, int n, hipStream_t st) {
+  hipLaunchKernelGGL(xcd_probe_kernel, dim3(n), dim3(64), 0, st, out);
   return hipGetLastError();
 }
 
