@@ -58,6 +58,16 @@ __device__ __forceinline__ fvec<4> load_streaming4(const float *src) {
   return r;
 }
 
+// A plain load of four floats as one value (assigning *(fvec<4> *) to a member of a struct in registers
+// can stay a copy through private memory).
+__device__ __forceinline__ fvec<4> load4(const float *src) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const f4 x = *reinterpret_cast<const f4 *>(src);
+  fvec<4> r;
+  r.v[0] = x[0]; r.v[1] = x[1]; r.v[2] = x[2]; r.v[3] = x[3];
+  return r;
+}
+
 // Consecutive workgroup ids land on different XCDs (each with its own 4 MB L2).  Work items
 // are cut into chunks of `bpc` consecutive items and chunk c goes to XCD c % 8, so that an
 // XCD walks whole chunks in order.  With bpc = all items / 8 every XCD gets one contiguous
@@ -1587,18 +1597,28 @@ __device__ __forceinline__ fvec<4> march_gather(const char *lane_base, int off) 
   return *reinterpret_cast<const fvec<4> *>(lane_base + quad_bcast<G>(off));
 }
 
+// One ELL row: the lanes of a quad hold two (LDS offset, value) pairs each.  Four gathers are in
+// flight at a time (eight measured no faster and cost sixteen registers).
 __device__ __forceinline__ fvec<4> march_row(const int4 e, const char *lane_base) {
-  fvec<4> x[8];
+  fvec<4> x[4];
   x[0] = march_gather<0>(lane_base, e.x); x[1] = march_gather<0>(lane_base, e.z);
   x[2] = march_gather<1>(lane_base, e.x); x[3] = march_gather<1>(lane_base, e.z);
-  x[4] = march_gather<2>(lane_base, e.x); x[5] = march_gather<2>(lane_base, e.z);
-  x[6] = march_gather<3>(lane_base, e.x); x[7] = march_gather<3>(lane_base, e.z);
   fvec<4> acc = vzero<4>();
   quad_fma<0>(e.y, x[0], acc); quad_fma<0>(e.w, x[1], acc);
+  x[0] = march_gather<2>(lane_base, e.x); x[1] = march_gather<2>(lane_base, e.z);
   quad_fma<1>(e.y, x[2], acc); quad_fma<1>(e.w, x[3], acc);
-  quad_fma<2>(e.y, x[4], acc); quad_fma<2>(e.w, x[5], acc);
-  quad_fma<3>(e.y, x[6], acc); quad_fma<3>(e.w, x[7], acc);
+  x[2] = march_gather<3>(lane_base, e.x); x[3] = march_gather<3>(lane_base, e.z);
+  quad_fma<2>(e.y, x[0], acc); quad_fma<2>(e.w, x[1], acc);
+  quad_fma<3>(e.y, x[2], acc); quad_fma<3>(e.w, x[3], acc);
   return acc;
+}
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
 }
 
 // What a lane keeps of one iteration's lists: its pairs of the ELL rows of its lane group (up to
@@ -1679,35 +1699,62 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
     const float *Cl = C + c0 + glane * 4;
     float *Dl = D + c0 + glane * 4;
     float *Tl = trash + glane * 4;
+    // (plain loads: a run's rows of C are its neighbours' halo rows an iteration or two later, and
+    // after a streaming load they were gone from L2 by then -- 1.36 GB fetched per launch on the 128^3
+    // grid against 1.05 GB)
     auto issue = [&](MarchStage &S) {
 #pragma unroll
-      // (streaming loads measured faster than plain ones, 0.46 against 0.57 ms on the 128^3 grid, although a
-      // run's rows of C are its neighbours' halo rows an iteration or two later)
-      for (int u = 0; u < kMarchLpg; ++u) S.c[u] = load_streaming4(Cl + (size_t)S.ll[u].x * N);
+      for (int u = 0; u < kMarchLpg; ++u) S.c[u] = load4(Cl + (size_t)S.ll[u].x * N);
     };
     // One iteration.  `cur` holds its lists; `fut` is free and takes those of iteration it + 2.  Stage
     // X is free (its rows went to LDS an iteration ago) and takes list it + 2, whose entries came with
-    // `cur`; stage Y holds list it + 1, which goes to LDS in the second half.
-    auto step = [&](int it, const MarchLists &cur, MarchLists &fut, MarchStage &X, const MarchStage &Y) {
-#pragma unroll
-      for (int u = 0; u < kMarchLpg; ++u) X.ll[u] = cur.ll[u];
-      issue(X);
-      fetch_lists(it + 2, fut);
+    // `cur`; stage Y holds list it + 1, which goes to LDS in the second half.  The requests to memory
+    // are dealt out over the rows, one share before each row: all at once at the top of the iteration
+    // they queue at the memory pipeline while the LDS and the ALUs have nothing to do.
+    auto step = [&](int it, const MarchLists &cur, MarchLists &fut, MarchStage &X, const MarchStage &Y) __attribute__((always_inline)) {
+      static_assert(kMarchLpg == kMarchTpg + kMarchDpg, "one share of the requests per row");
+      const int nx = it + 2, nl = it + 4;
+      const bool in = nx < n_iter, inl = nl < n_iter;
+      const int b0 = in ? tab[4 * nx] : 0, b1 = in ? tab[4 * nx + 1] : 0, b2 = in ? tab[4 * nx + 4] : 0;
+      const int lb = inl ? tab[4 * nl + 2] : 0, le = inl ? tab[4 * nl + 6] : 0;
+      auto share = [&](auto vc) __attribute__((always_inline)) {
+        constexpr int v = decltype(vc)::value;
+        X.ll[v] = cur.ll[v];
+        X.c[v] = load4(Cl + (size_t)X.ll[v].x * N);
+        if constexpr (v < kMarchTpg) {
+          const int x = b0 + group + kMarchGroups * v, xc = max(min(x, b1 - 1), 0);
+          const int o = row_out[xc], m = opaque_mask(x < b1);
+          fut.et[v] = load_streaming_i4(ell + (size_t)xc * 4 + q);  // a group without a row recomputes another's, into the trash row
+          fut.ot[v] = (o & m) | (~kMarchTrashOff & ~m);
+        } else {
+          constexpr int u = v - kMarchTpg;
+          const int x = b1 + group + kMarchGroups * u, xc = max(min(x, b2 - 1), 0);
+          const int o = row_out[xc], m = opaque_mask(x < b2);
+          fut.ed[u] = load_streaming_i4(ell + (size_t)xc * 4 + q);
+          fut.od[u] = o | ~m;  // -1: no row
+        }
+        const int x = lb + group + kMarchGroups * v;
+        const int2 l = load_list[max(min(x, le - 1), 0)];
+        const int m = opaque_mask(x < le);
+        fut.ll[v] = make_int2(l.x, (l.y & m) | (kMarchTrashOff & ~m));  // a group without an entry re-reads another's row into the trash row
+      };
       // the intermediate rows this iteration's second-op rows are the first to read
-#pragma unroll
-      for (int u = 0; u < kMarchTpg; ++u) {
+      static_for<0, kMarchTpg>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        share(uc);
         const fvec<4> acc = march_row(cur.et[u], lane_base);
         *reinterpret_cast<fvec<4> *>(lane_base + ~cur.ot[u]) = acc;
-      }
+      });
       lds_barrier();
       // the second-op rows; the next rows of C take the slots of rows no one reads any more
-#pragma unroll
-      for (int u = 0; u < kMarchDpg; ++u) {
+      static_for<0, kMarchDpg>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        share(std::integral_constant<int, kMarchTpg + u>{});
         fvec<4> acc = march_row(cur.ed[u], lane_base);
         float *dst = cur.od[u] >= 0 ? Dl + (size_t)cur.od[u] * N : Tl;
         if (ACC) vadd<4>(*reinterpret_cast<const fvec<4> *>(dst), acc);
         store_streaming<4>(dst, acc);
-      }
+      });
 #pragma unroll
       for (int u = 0; u < kMarchLpg; ++u) *reinterpret_cast<fvec<4> *>(lane_base + Y.ll[u].y) = Y.c[u];
       lds_barrier();
@@ -1721,7 +1768,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
     fetch_lists(1, E1);
     for (int x = tab[2] + group; x < tab[6]; x += kMarchGroups) {
       const int2 l = load_list[x];
-      *reinterpret_cast<fvec<4> *>(lane_base + l.y) = load_streaming4(Cl + (size_t)l.x * N);
+      *reinterpret_cast<fvec<4> *>(lane_base + l.y) = load4(Cl + (size_t)l.x * N);
     }
     issue(S1);
     __syncthreads();
