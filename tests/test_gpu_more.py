@@ -221,6 +221,37 @@ def test_remainder_rows_in_list_order(gpu, tf, orc):
     assert np.array_equal(got[0], got[1]) and np.array_equal(got[0], oracle_spmm_spmm(orc, Sm, Sm, Cd))
 
 
+def test_many_rows_without_entries(gpu, tf, orc):
+    """Second-op rows without entries, when they are many, are cleared by a fill kernel of their own instead of
+    taking a lane group each: every such row of D is zero afterwards (D starts as NaN), rows with entries match
+    the oracle bit for bit, and with accumulate the empty rows keep what D held."""
+    say("many empty rows")
+    rng = np.random.default_rng(21)
+    M = 40000
+    A = sp.random(M, M, density=6.0 / M, format="csr", random_state=21, dtype=np.float32)
+    keep = rng.random(M) < 0.4                      # 60 % of the rows lose their entries
+    A = sp.diags(keep.astype(np.float32)) @ A
+    A.eliminate_zeros(); A.sort_indices()
+    A = sp.csr_matrix((A.data.astype(np.float32), A.indices.astype(np.int32), A.indptr.astype(np.int32)), shape=A.shape)
+    empty = np.diff(A.indptr) == 0
+    assert empty.sum() > 20000
+    Cd = tf.workloads.uniform((M, 64), 6)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64)
+    S.validate()
+    assert S.info()["n_remainder_rows"] + S.info()["n_fused_rows"] == M
+    D = tf.DenseMatrix(M, 64); D.fill(float("nan"))
+    tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(Cd), D, S)
+    got = D.to_numpy()
+    want = oracle_spmm_spmm(orc, A, A, Cd)
+    assert np.array_equal(got, want) and not got[empty].any()
+    D.fill(1.5)
+    tf.spmm_spmm(Ah, Ah, tf.DenseMatrix.from_numpy(Cd), D, S, accumulate=True)
+    acc = D.to_numpy()
+    assert np.array_equal(acc[empty], np.full_like(acc[empty], 1.5))
+    assert np.allclose(acc[~empty], want[~empty] + 1.5, rtol=1e-6, atol=1e-6)
+
+
 def test_device_reports_the_workgroup_to_xcd_mapping(gpu):
     """tf_device_init probes what the XCD-pinned kernels rely on: workgroup b runs on XCD b mod 8."""
     assert gpu["xcds"] == 8 and gpu["compute_units"] == 256 and gpu["wavefront"] == 64

@@ -38,6 +38,7 @@ struct DeviceSchedule {
   int *fused_ids = nullptr;
   int *win = nullptr;
   int *rem_rows = nullptr;
+  int *zero_rows = nullptr;
   int *plain_rows = nullptr;
   int *step_begin = nullptr;  // streamed GeMM-SpMM: per launched tile, first entry in step_ptr
   int *step_ptr = nullptr;
@@ -84,7 +85,7 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *, const int *, int, c
                                            const float *, int, const float *, const int *, const int *,
                                            const float *, int, float *, int, int, int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
-                            float *, int, int, int, int, hipStream_t, int compact = 0);
+                            float *, int, int, int, int, hipStream_t, int compact = 0, int coalesced_pairs = 0);
 hipError_t launch_gather_values(const int *, const float *, float *, int, hipStream_t);
 hipError_t launch_march_fill(const int *, const int *, const float *, const float *, int *, size_t, hipStream_t);
 hipError_t launch_fused_spmm_spmm_march(const int *, int, const int *, const int *, const int *, const int *, const int *,
@@ -103,6 +104,7 @@ hipError_t launch_gemm(const float *, const float *, float *, const int *, int, 
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 hipError_t launch_pad(const float *, int, int, float *, int, int, hipStream_t);
 hipError_t launch_relu(float *, size_t, hipStream_t);
+hipError_t launch_zero_rows(const int *, int, float *, int, hipStream_t);
 hipError_t launch_xcd_probe(int *, int, hipStream_t);
 
 // An intermediate larger than the 256 MB last-level cache is gone from it before its readers
@@ -142,7 +144,7 @@ int default_compute_units() {
 
 void release_device_schedule(DeviceSchedule *d) {
   if (!d) return;
-  (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows); (void)hipFree(d->plain_rows);
+  (void)hipFree(d->tiles); (void)hipFree(d->fused_ids); (void)hipFree(d->win); (void)hipFree(d->rem_rows); (void)hipFree(d->zero_rows); (void)hipFree(d->plain_rows);
   (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows); (void)hipFree(d->seg_groups);
   (void)hipFree(d->seg_ptr); (void)hipFree(d->ent_src); (void)hipFree(d->ent_pos); (void)hipFree(d->seg_col); (void)hipFree(d->lrow_seg); (void)hipFree(d->seg_val);
   (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
@@ -204,6 +206,7 @@ static tf_status ensure_device(tf_schedule *s) {
   if (!rc) rc = upload_vec(s->fused_ids, &d->fused_ids);
   if (!rc) rc = upload_vec(s->win, &d->win);
   if (!rc) rc = upload_vec(s->rem_rows, &d->rem_rows);
+  if (!rc) rc = upload_vec(s->zero_rows, &d->zero_rows);
   if (!rc) rc = upload_vec(s->plain_rows, &d->plain_rows);
   if (!rc) rc = upload_vec(s->launch_step, &d->step_begin);
   if (!rc) rc = upload_vec(s->step_ptr, &d->step_ptr);
@@ -296,7 +299,7 @@ static tf_status run_hot_segments(const tf_csr *A, tf_schedule *s, hipStream_t s
     TF_PHASE(s, "scatter_values_kernel", st, launch_scatter_values(d->ent_src, d->ent_pos, A->x, d->seg_val, (int)s->seg_src.size(), st));
   d->seg_val_serial = A->serial;
   TF_PHASE(s, "spmm_rows_kernel (hot long-row segments)", st,
-           launch_spmm_rows(nullptr, 8 * s->seg_per_xcd, d->seg_ptr, d->seg_col, d->seg_val, d->inter, d->partial, s->opts.N, 0, -1, 1, st));
+           launch_spmm_rows(nullptr, 8 * s->seg_per_xcd, d->seg_ptr, d->seg_col, d->seg_val, d->inter, d->partial, s->opts.N, 0, -1, 1, st, /*compact=*/0, /*coalesced_pairs=*/1));
   return TF_OK;
 }
 
@@ -305,6 +308,8 @@ static tf_status run_hot_segments(const tf_csr *A, tf_schedule *s, hipStream_t s
 static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int accumulate, bool hot_on_side, hipStream_t st) {
   DeviceSchedule *d = s->dev;
   const int N = s->opts.N;
+  if (!s->zero_rows.empty() && !accumulate)  // (D += 0 needs nothing)
+    TF_PHASE(s, "zero_rows_kernel (rows without entries)", st, launch_zero_rows(d->zero_rows, (int)s->zero_rows.size(), D->d, N, st));
   if (!s->rem_rows.empty() && !s->rem_ptr.empty()) {
     // The rows in the order of the list, entries side by side -- the reference's reordered adjacency
     // (createReorderedAdj, GCN_Single_Layer_SP_Demo_Utils.h:618-653; executor at

@@ -575,6 +575,20 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         return len <= 8 ? 0 : len <= 32 ? 1 : len <= 128 ? 2 : len <= 512 ? 3 : 4;
       };
       std::vector<int> byc[5];
+      // Rows without entries, when they are many (half of the nodes of an R-MAT graph are isolated): a row
+      // of zeros needs no lane group, no row pointers and no place in a round of the row kernel, whose
+      // time is rounds times the latency of a row's chain of loads.
+      {
+        size_t n_empty = 0;
+        for (int i : S->rem_rows) n_empty += Ap[i + 1] == Ap[i];
+        if (n_empty >= 4096 && n_empty * 8 >= S->rem_rows.size()) {
+          std::vector<int> keep;
+          keep.reserve(S->rem_rows.size() - n_empty);
+          S->zero_rows.reserve(n_empty);
+          for (int i : S->rem_rows) (Ap[i + 1] == Ap[i] ? S->zero_rows : keep).push_back(i);
+          S->rem_rows.swap(keep);
+        }
+      }
       for (int i : S->rem_rows) byc[cls(i)].push_back(i);
       S->rem_rows.clear();
       for (auto &v : byc) S->rem_rows.insert(S->rem_rows.end(), v.begin(), v.end());
@@ -695,7 +709,7 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   info->rows = s->L; info->inter_rows = s->M;
   info->n_tiles = (int)s->tiles.size();
   info->n_fused_rows = (int)s->fused_ids.size();
-  info->n_remainder_rows = (int)(s->rem_rows.size() + s->long_rows.size());
+  info->n_remainder_rows = (int)(s->rem_rows.size() + s->zero_rows.size() + s->long_rows.size());
   info->n_long_rows = (int)s->long_rows.size();
   info->n_long_chunks = s->long_part ? (int)s->seg_ptr.size() - 1 : (int)s->long_chunks.size();
   info->long_row_hot_cols = s->long_part ? s->hot_cols : 0;
@@ -825,7 +839,13 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
         if (s->rem_src[e] != k || s->rem_col[e] != Ai[k]) return tf::fail(TF_ESCHEDULE, "remainder rows in list order: row %d differs from A's", i);
     }
   }
+  for (int i : s->zero_rows) {
+    if (i < 0 || i >= L) return tf::fail(TF_ESCHEDULE, "empty row %d out of range", i);
+    if (done[i]++) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled twice", i);
+    if (Ap[i + 1] != Ap[i]) return tf::fail(TF_ESCHEDULE, "row %d is listed as empty and has entries", i);
+  }
   for (int i : s->rem_rows) {
+    if (i < 0 || i >= L) return tf::fail(TF_ESCHEDULE, "remainder row %d out of range", i);
     if (done[i]++) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled twice", i);
     if (Ap[i + 1] - Ap[i] > s->opts.long_row_nnz)
       return tf::fail(TF_ESCHEDULE, "remainder row %d is long but not chunked", i);

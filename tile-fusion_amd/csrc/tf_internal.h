@@ -86,6 +86,8 @@ struct tf_schedule {
   std::vector<int> rem_rows;        // remainder rows handled one row per lane group, ordered by
                                     // length class so that a workgroup's rows cost about the same
   bool rem_identity = false;        // rem_rows is 0..L-1 in order
+  std::vector<int> zero_rows;       // second-op rows without entries, when many: their rows of D are cleared by a
+                                    // fill kernel instead of taking a lane group each in the row kernel
   // When the list is not the identity, its rows are also kept as a CSR of their own in list order
   // (row q of it is row rem_rows[q] of A): rem_ptr [n + 1], rem_col, and rem_src = where each entry
   // sits in A's arrays (the executor copies the values from there).

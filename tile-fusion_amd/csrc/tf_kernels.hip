@@ -160,6 +160,10 @@ __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float
 // The same sum with every lane reading the row's (column, value) pairs itself: the lanes of a
 // group read the same address, which costs one request per group and no cross-lane traffic.
 // Eight pairs, then their eight gathers, then the fmas; slots past the row's end load nothing.
+// (Requesting the next eight pairs behind the current gathers, so that they arrive together, takes
+// 112 registers instead of 60 and halves the wavefronts in flight: the R-MAT step went from 2.24 to
+// 2.88 ms.  What bounds a launch of many short rows or segments is rounds of lane groups times the
+// length of a row's chain of dependent loads; rows in flight are worth more than a shorter chain.)
 template <int V, int LPR, class Src>
 __device__ __forceinline__ void row_dot_direct(const int *__restrict__ idx, const float *__restrict__ val,
                                                int kb, int ke, bool col_ok, const Src &src, fvec<V> &acc) {
@@ -637,7 +641,7 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
 // that no tile fuses, and tf_spmm.  One lane group per row and small, short-lived
 // workgroups: what hides the gather latency is the number of rows in flight.
 // ---------------------------------------------------------------------------------
-template <int V, int LPR>
+template <int V, int LPR, bool COAL>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
     const int *__restrict__ rows, int n_rows, int n_blocks, int per_xcd, const int *__restrict__ Ap,
     const int *__restrict__ Ai, const float *__restrict__ Ax, const float *__restrict__ X, int ldx,
@@ -659,7 +663,13 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
     const GlobalRows<V> src{X, ldx, ok ? coff : 0};
     fvec<V> acc = vzero<V>();
     if (accumulate && ok) acc = *reinterpret_cast<const fvec<V> *>(Y + (size_t)i * N + coff);
-    row_dot_direct<V, LPR>(Ai, Ax, kb, ke, ok, src, acc);
+    // COAL: the group's lanes load the pairs of up to LPR entries with one coalesced request and hand
+    // them round by shuffles -- one round trip for the pairs of a long row or segment instead of one
+    // per eight entries (hot long-row segments of the R-MAT step, 22 entries on average: 0.86 -> 0.74
+    // ms).  Rows of a few entries, and segments whose gathers all miss L2, are served as well or
+    // better by every lane reading the pairs itself (cold segments 0.27 -> 0.29 ms).
+    if constexpr (COAL) row_dot<V, LPR>(Ai, Ax, kb, ke, glane, ok, src, acc);
+    else row_dot_direct<V, LPR>(Ai, Ax, kb, ke, ok, src, acc);
     if (ok) {
       if (streaming) store_streaming<V>(Y + (size_t)i * N + coff, acc);
       else *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
@@ -765,6 +775,17 @@ __global__ void pad_kernel(const float *__restrict__ src, int src_rows, int ld_s
 }
 
 // p = max(p, 0), four values per thread (n is a multiple of 4: the kernels' N is).
+// Rows of zeros: Y[rows[q], :] = 0 (second-op rows without entries), V floats per thread.
+template <int V>
+__global__ void zero_rows_kernel(const int *__restrict__ rows, size_t units, float *__restrict__ Y, int N) {
+  const int per_row = N / V;
+  for (size_t u = blockIdx.x * (size_t)blockDim.x + threadIdx.x; u < units; u += (size_t)gridDim.x * blockDim.x) {
+    const size_t q = u / per_row;
+    const int c = (int)(u - q * per_row) * V;
+    store_streaming<V>(Y + (size_t)rows[q] * N + c, vzero<V>());  // (plain stores: this launch 5 % faster, the next one 5 % slower)
+  }
+}
+
 __global__ void relu_kernel(float *__restrict__ p, size_t n4) {
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
     fvec<4> v = *reinterpret_cast<const fvec<4> *>(p + 4 * i);
@@ -1924,18 +1945,20 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *tiles, const int *win
 
 hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const int *Ai, const float *Ax,
                             const float *X, float *Y, int N, int accumulate, int xcd_chunk_rows,
-                            int streaming, hipStream_t st, int compact) {
+                            int streaming, hipStream_t st, int compact, int coalesced_pairs) {
   if (n_rows <= 0) return hipSuccess;
   const Shape s = pick_shape(N);
   const int G = kBlock / s.LPR;
   const int n_blocks = (n_rows + G - 1) / G;
   // 0: workgroup b takes block b; > 0: chunks of rows per XCD turn; < 0: one contiguous run per XCD
   const int bpc = xcd_chunk_rows == 0 ? 0 : chunk_bpc(n_blocks, xcd_chunk_rows > 0 ? std::max(1, xcd_chunk_rows / G) : 0);
-#define CALL(V_, L_)                                                                                   \
-  hipLaunchKernelGGL((spmm_rows_kernel<V_, L_>), dim3(grid_chunked(n_blocks, bpc)), dim3(kBlock), 0, st, \
+#define CALL2(V_, L_, COAL_)                                                                                   \
+  hipLaunchKernelGGL((spmm_rows_kernel<V_, L_, COAL_>), dim3(grid_chunked(n_blocks, bpc)), dim3(kBlock), 0, st, \
                      rows, n_rows, n_blocks, bpc, Ap, Ai, Ax, X, N, Y, N, accumulate, streaming, compact)
+#define CALL(V_, L_) do { if (coalesced_pairs) { CALL2(V_, L_, true); } else { CALL2(V_, L_, false); } } while (0)
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
 #undef CALL
+#undef CALL2
   return hipGetLastError();
 }
 
@@ -2116,6 +2139,15 @@ hipError_t launch_pad(const float *src, int src_rows, int ld_src, float *dst, in
   if (n == 0) return hipSuccess;
   const int blocks = (int)std::min<size_t>((n + kBlock - 1) / kBlock, 65536);
   hipLaunchKernelGGL(pad_kernel, dim3(blocks), dim3(kBlock), 0, st, src, src_rows, ld_src, dst, rows, ld_dst);
+  return hipGetLastError();
+}
+
+hipError_t launch_zero_rows(const int *rows, int n_rows, float *Y, int N, hipStream_t st) {
+  if (n_rows <= 0) return hipSuccess;
+  const size_t units = (size_t)n_rows * (N % 4 == 0 ? N / 4 : N);
+  const unsigned blocks = (unsigned)std::min<size_t>((units + 255) / 256, 1u << 20);
+  if (N % 4 == 0) hipLaunchKernelGGL((zero_rows_kernel<4>), dim3(blocks), dim3(256), 0, st, rows, units, Y, N);
+  else hipLaunchKernelGGL((zero_rows_kernel<1>), dim3(blocks), dim3(256), 0, st, rows, units, Y, N);
   return hipGetLastError();
 }
 
