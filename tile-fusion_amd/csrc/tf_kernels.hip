@@ -953,10 +953,12 @@ constexpr int kGemmBlock = 512;
 
 template <int NB> struct alignas((NB == 1 || NB == 2 || NB == 4) ? 4 * NB : (NB == 8 ? 16 : 4)) wvec { float v[NB]; };
 
-// W in LDS is interleaved so that the NB values a lane feeds to the NB column blocks of one
-// k step are adjacent: element (k, nb*32 + j) sits at (k*32 + j)*NB + nb.  One LDS read per
-// k step then serves all NB MFMAs (16 bytes when NB = 4), and the reads for the next eight
-// values of k are issued before the MFMAs of the current eight.
+// Column block nb of a wavefront's 32 x (32 NB) output tile holds the columns NB j + nb, j = 0 .. 31 (not
+// 32 nb + j): W then sits in LDS as it is in memory, row-major, the NB values a lane feeds to the NB MFMAs of
+// one k step are adjacent (one LDS read of 4 NB bytes per k step), and a lane ends up with NB consecutive
+// columns of each of its output rows, which leave with one store (16 bytes when NB = 4; a row of the tile
+// is 32 such stores side by side).  The reads for the next eight values of k are issued before the MFMAs
+// of the current eight.
 template <int NB>
 __device__ __forceinline__ void mfma_step8(const fvec<4> &a, const wvec<NB> (&bw)[4], v16f (&acc)[NB]) {
 #pragma unroll
@@ -966,13 +968,13 @@ __device__ __forceinline__ void mfma_step8(const fvec<4> &a, const wvec<NB> (&bw
       acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[t], bw[t].v[nb], acc[nb], 0, 0, 0);
 }
 
-// Copies W (K x N, row-major) into LDS in the interleaved layout described above:
-// 16 bytes per load, eight loads in flight per thread, then the scatter into LDS.
+// Copies W (K x N, row-major) into LDS as it is: 16 bytes per load, eight loads in flight per thread.
 template <int NB>
-__device__ __forceinline__ void stage_weights_interleaved(const float *__restrict__ W, int K, float *wlds) {
+__device__ __forceinline__ void stage_weights(const float *__restrict__ W, int K, float *wlds) {
   constexpr int N = NB * 32;
   const int n4 = K * N / 4;
   const fvec<4> *src = reinterpret_cast<const fvec<4> *>(W);
+  fvec<4> *dst = reinterpret_cast<fvec<4> *>(wlds);
   for (int i0 = threadIdx.x; i0 < n4; i0 += 8 * kGemmBlock) {
     fvec<4> v[8];
 #pragma unroll
@@ -983,12 +985,7 @@ __device__ __forceinline__ void stage_weights_interleaved(const float *__restric
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int i = i0 + u * kGemmBlock;
-      if (i < n4) {
-        const int e = i * 4, k = e / N, n = e % N;  // four consecutive columns of one column block
-        float *dst = wlds + (k * 32 + (n % 32)) * NB + n / 32;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) dst[c * NB] = v[u].v[c];
-      }
+      if (i < n4) dst[i] = v[u];
     }
   }
 }
@@ -1003,7 +1000,7 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
                                                                int K) {
   extern __shared__ __align__(16) float wlds[];
   constexpr int N = NB * 32;
-  stage_weights_interleaved<NB>(W, K, wlds);
+  stage_weights<NB>(W, K, wlds);
   __syncthreads();
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int h = lane / 32, j = lane % 32;
@@ -1037,7 +1034,7 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
       v16f acc1;
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc1[r] = 0.f;
-      const float *wt = wlds + ((4 * h) * 32 + j) * NB + nb;  // element (k, nb*32 + j) sits at (k*32 + j)*NB + nb
+      const float *wt = wlds + ((4 * h) * 32 + j) * NB + nb;  // W[k][NB j + nb] sits at (k*32 + j)*NB + nb
       fvec<4> a = *reinterpret_cast<const fvec<4> *>(p);
       for (int st = 0; st < steps; ++st) {
         const fvec<4> an = *reinterpret_cast<const fvec<4> *>(p + 8 * min(st + 1, steps - 1));
@@ -1049,7 +1046,7 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int x = rb * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-        if (x < n_rows) Y[(size_t)(LIST ? rows[x] : x) * N + nb * 32 + j] = acc1[r];
+        if (x < n_rows) Y[(size_t)(LIST ? rows[x] : x) * N + NB * j + nb] = acc1[r];
       }
     }
   }
@@ -1112,9 +1109,10 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
         for (int r = 0; r < 16; ++r) {
           const int x = blk * 32 + 8 * (r / 4) + 4 * h + (r % 4);
           if (rb0 * 32 + x < n_rows) {
-            float *dst = Y + (size_t)row_at(x) * N + j;
+            wvec<NB> out;
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) dst[nb * 32] = acc[nb][r];
+            for (int nb = 0; nb < NB; ++nb) out.v[nb] = acc[nb][r];
+            *reinterpret_cast<wvec<NB> *>(Y + (size_t)row_at(x) * N + NB * j) = out;
           }
         }
       }
