@@ -1104,7 +1104,7 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
       }
       if (s0 + 3 < steps) mfma_step8<NB>(c[3], bn, acc);
       if (g == G4 - 1) {
-        // accumulator register r of lane (h, j) holds output row 8*(r/4) + 4*h + r%4, column j
+        // accumulator register r of column block nb of lane (h, j) holds output row 8*(r/4) + 4*h + r%4, column NB j + nb
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int x = blk * 32 + 8 * (r / 4) + 4 * h + (r % 4);
