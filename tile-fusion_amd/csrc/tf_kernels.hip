@@ -162,8 +162,8 @@ __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float
 // Eight pairs, then their eight gathers, then the fmas; slots past the row's end load nothing.
 // (Requesting the next eight pairs behind the current gathers, so that they arrive together, takes
 // 112 registers instead of 60 and halves the wavefronts in flight: the R-MAT step went from 2.24 to
-// 2.88 ms.  What bounds a launch of many short rows or segments is rounds of lane groups times the
-// length of a row's chain of dependent loads; rows in flight are worth more than a shorter chain.)
+// 2.88 ms.  Wavefronts in flight are worth more to these launches than a shorter chain of dependent
+// loads per row.)
 template <int V, int LPR, class Src>
 __device__ __forceinline__ void row_dot_direct(const int *__restrict__ idx, const float *__restrict__ val,
                                                int kb, int ke, bool col_ok, const Src &src, fvec<V> &acc) {
