@@ -64,6 +64,29 @@ int main() {
     bad += run("stencil march", M, p, i, o);
     o.march_tile_x = 5; o.march_tile_y = 3; o.compute_units = 7; bad += run("stencil march 5x3", M, p, i, o);
     o.march_tile_x = o.march_tile_y = 0; o.grid_nx = ny; o.grid_ny = nx; o.grid_nz = nz; bad += run("stencil march, wrong grid", M, p, i, o); }
+  {  // 5-point stencil on a 300 x 90 grid (runs along the grid's lines) and a tall 7-point grid (more planes
+     // than a run's table holds: cut into several runs along z)
+    auto stencil = [&](int nx, int ny, int nz) {
+      p.assign(1, 0); i.clear();
+      for (int z = 0; z < nz; ++z) for (int y = 0; y < ny; ++y) for (int x = 0; x < nx; ++x) {
+        const int r = (z * ny + y) * nx + x;
+        if (z > 0) i.push_back(r - nx * ny);
+        if (y > 0) i.push_back(r - nx);
+        if (x > 0) i.push_back(r - 1);
+        i.push_back(r);
+        if (x < nx - 1) i.push_back(r + 1);
+        if (y < ny - 1) i.push_back(r + nx);
+        if (z < nz - 1) i.push_back(r + nx * ny);
+        p.push_back((int)i.size());
+      }
+      return nx * ny * nz;
+    };
+    int M = stencil(300, 1, 90);
+    tf_inspect_opts o{}; o.struct_size = sizeof(o); o.op = TF_OP_SPMM_SPMM; o.N = 64; o.inner_Ap = p.data(); o.inner_Ai = i.data(); o.inner_cols = M; o.march = 1;
+    bad += run("flat stencil march", M, p, i, o);
+    M = stencil(10, 9, 700);
+    o.inner_Ap = p.data(); o.inner_Ai = i.data(); o.inner_cols = M; o.compute_units = 4;
+    bad += run("tall stencil march", M, p, i, o); }
   powerlaw(60000, 1500000, 2, p, i);
   { tf_inspect_opts o{}; o.struct_size = sizeof(o); o.op = TF_OP_GEMM_SPMM; o.N = 128; o.K = 128; o.long_row_partition = 1; bad += run("powerlaw part", 60000, p, i, o);
     o.long_row_partition = -1; bad += run("powerlaw chunks", 60000, p, i, o);

@@ -54,6 +54,26 @@ def test_march_bit_exact(gpu, tf, orc, dims, N):
     assert np.array_equal(got, want), (dims, N, info)
 
 
+@pytest.mark.parametrize("dims,N", [((300, 1, 90), 64), ((128, 1, 128), 128), ((10, 9, 700), 64)])
+def test_march_flat_and_tall_grids(gpu, tf, orc, dims, N):
+    """A 5-point stencil on a 2D grid (found from its two distances; the runs walk the grid's lines, 64 points of
+    a line at a time) and a grid with more planes than a run's table of iterations holds (cut into several runs
+    along z): the same bits as the oracle."""
+    say(f"march {dims} N={N}")
+    nx, ny, nz = dims
+    A = stencil_3d(nx, ny, nz, seed=17)
+    Cd = tf.workloads.uniform((A.shape[0], N), 18)
+    want = oracle_spmm_spmm(orc, A, A, Cd)
+    got, info = march(tf, A, A, Cd)
+    assert np.array_equal(got, want), (dims, N, info)
+    if ny == 1:
+        assert info["march_tile_y"] == 1 and info["march_tile_x"] > 8, info
+    if nz > 254:
+        got, info = march(tf, A, A, Cd, compute_units=4)   # few compute units: the cut comes from the table's size
+        assert np.array_equal(got, want), (dims, N, info)
+        assert info["n_tiles"] > 4, info
+
+
 def test_march_tiles_hints_and_operands(gpu, tf, orc):
     say("march: tile sizes, grid hints, B != A, accumulate")
     nx, ny, nz = 24, 18, 30

@@ -17,6 +17,7 @@
 #include <algorithm>
 #include <climits>
 #include <cstring>
+#include <iterator>
 #include <map>
 
 #include "tf_internal.h"
@@ -28,7 +29,9 @@ namespace {
 constexpr int kMaxLds = 163840;
 
 // The grid a pattern was generated on, from the distances between a row and its columns: a
-// 7-point-like stencil on nx x ny x nz points, x fastest, has the distances 1, nx and nx*ny.
+// 7-point-like stencil on nx x ny x nz points, x fastest, has the distances 1, nx and nx*ny; a
+// 5-point-like stencil on nx x n points the distances 1 and nx (a grid of nx x 1 x n: the runs then
+// walk the grid's lines, a stretch of a line at a time).
 bool detect_grid(int M, const int *Ap, const int *Ai, int grid[3]) {
   std::map<int, long long> dist;
   for (int i = 0; i < M; ++i)
@@ -38,6 +41,12 @@ bool detect_grid(int M, const int *Ap, const int *Ai, int grid[3]) {
       if (dist.size() > 3 && !dist.count(d)) return false;
       ++dist[d];
     }
+  if (dist.size() == 2) {
+    const int d1 = dist.begin()->first, d2 = std::next(dist.begin())->first;
+    if (d1 != 1 || d2 < 16 || M % d2 != 0 || M / d2 < 2) return false;
+    grid[0] = d2; grid[1] = 1; grid[2] = M / d2;
+    return true;
+  }
   if (dist.size() != 3) return false;
   auto it = dist.begin();
   const int d1 = it->first; ++it;
@@ -72,6 +81,14 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
     const int per_plane = tx * ty;
     int nzc = std::max(1, (o.compute_units + per_plane - 1) / per_plane);
     nzc = std::min(nzc, std::max(1, nz / 8));  // a run of a few planes is mostly start-up
+    // (a run's table of iterations has kMarchMaxIter places: taller grids are cut further, into a whole
+    // number of turns of the compute units where that is near)
+    const int nzc_min = (nz + kMarchMaxIter - 9) / (kMarchMaxIter - 8);
+    if (nzc < nzc_min) {
+      nzc = nzc_min;
+      for (int c = nzc_min; c <= 2 * nzc_min; ++c)
+        if ((long long)per_plane * c % o.compute_units == 0) { nzc = c; break; }
+    }
     const int zlen = (nz + nzc - 1) / nzc;
 
     std::vector<int> runs, row_ptr, load_ptr, load, row_out, row_id, ell_off, ell_src, ids;
@@ -265,9 +282,16 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
     ok = attempt(given.march_tile_x, given.march_tile_y);
   } else {
     // the largest column that fits: the halo ring costs less the larger the column is
-    const int cand[][2] = {{8, 8}, {8, 7}, {8, 6}, {8, 5}, {8, 4}, {4, 4}};
-    for (const auto &c : cand)
-      if ((ok = attempt(c[0], c[1]))) break;
+    if (ny >= 8) {
+      const int cand[][2] = {{8, 8}, {8, 7}, {8, 6}, {8, 5}, {8, 4}, {4, 4}};
+      for (const auto &c : cand)
+        if ((ok = attempt(c[0], c[1]))) break;
+    } else {  // a flat grid: the column takes all of y and as much of x as gives it the same number of points
+      for (const int points : {64, 56, 48, 40, 32, 16}) {
+        const int bx = std::min(nx, points / ny);
+        if (bx >= 1 && (ok = attempt(bx, ny))) break;
+      }
+    }
   }
   if (!ok) return false;
 
