@@ -36,6 +36,33 @@ def test_operators_are_registered_with_the_reference_signatures():
     assert args == ["Adj", "Weight", "Feature", "LevelPtr", "MixPtr", "Partition", "NumThreads"]
 
 
+def test_load_library_like_the_reference(tmp_path):
+    """torch.ops.load_library("…/libsw_gcn.so"), the line the reference's Python layers start with
+    (binding-project/gcn-e2e-training/FusedGCNLayer.py:3), in a fresh interpreter and from another directory:
+    loading the library registers torch.ops.sw_gcn.* (it imports torch_ops.py), an inspector runs on CPU tensors."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = os.path.join(root, "tile-fusion_amd", "lib", "libsw_gcn.so")
+    if not os.path.exists(lib):
+        pytest.skip("libsw_gcn.so is not built")
+    code = f"""
+import torch
+torch.ops.load_library({lib!r})
+names = ["inspect", "inspect_vt_ro", "executeFusedGeMMSpMM", "fusedGeMMSpMM", "fusedGeMMSpMM_vt_ro", "geMMSpMM_f_bw",
+         "cachedSpMMGeMM", "unfused_gcn_forward"]
+assert all(hasattr(torch.ops.sw_gcn, n) for n in names)
+crow = torch.arange(0, 9, dtype=torch.int32); col = torch.arange(0, 8, dtype=torch.int32)
+adj = torch.sparse_csr_tensor(crow, col, torch.ones(8), size=(8, 8))
+sched = torch.ops.sw_gcn.inspect_vt_ro(adj, 32, 32, 500000, 1)
+assert len(sched) == 3
+print("ok")
+"""
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600, cwd=str(tmp_path))
+    assert r.returncode == 0 and "ok" in r.stdout, (r.stdout[-500:], r.stderr[-2000:])
+
+
 def test_inspect_returns_the_binding_layout(tf):
     A = tf.workloads.banded_random(3000, 32, 16, seed=9)
     adj = csr_tensor(A)
