@@ -283,25 +283,6 @@ __device__ __forceinline__ fvec<4> lds_row_dot(const int2 *__restrict__ ent, int
   return acc;
 }
 
-// The same with eight entries in flight: all entry reads of a batch are issued, then all
-// gathers, then the fmas -- two LDS round trips per eight entries.  For callers whose row is
-// alone on its lane group's critical path.
-__device__ __forceinline__ fvec<4> lds_row_dot8(const int2 *__restrict__ ent, int kb, int ke,
-                                                const char *base, fvec<4> acc) {
-  int k = kb;
-  for (; k + 8 <= ke; k += 8) {
-    int2 e[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) e[u] = ent[k + u];
-    fvec<4> x[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) x[u] = *reinterpret_cast<const fvec<4> *>(base + e[u].x);
-#pragma unroll
-    for (int u = 0; u < 8; ++u) vfma<4>(__int_as_float(e[u].y), x[u], acc);
-  }
-  return lds_row_dot(ent, k, ke, base, acc);
-}
-
 // The value lane G of the caller's quad holds (a DPP quad_perm broadcast, folded into the
 // consuming instruction: no LDS traffic and no instruction of its own).
 template <int G> __device__ __forceinline__ int quad_bcast(int v) {
@@ -1502,7 +1483,7 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
       const int cnt = min(LPR, rec.z - rec.y - u * LPR);
       if (u == 0 || cnt > 0) {
         scratch[glane] = make_int2(((c[u] - t.prod_begin) & ring_mask) * (ld * 4), __float_as_int(a[u]));
-        acc = lds_row_dot8(scratch, 0, cnt, rbase, acc);
+        acc = lds_row_dot_quad(scratch, 0, cnt, rbase, glane & 3, acc);  // (reads up to 3 pairs past the row's: never used)
       }
     }
     if (ok) store_streaming<4>(dst, acc);
