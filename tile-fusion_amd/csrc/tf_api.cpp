@@ -89,7 +89,7 @@ hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const fl
 hipError_t launch_gather_values(const int *, const float *, float *, int, hipStream_t);
 hipError_t launch_march_fill(const int *, const int *, const float *, const float *, int *, size_t, hipStream_t);
 hipError_t launch_fused_spmm_spmm_march(const int *, int, const int *, const int *, const int *, const int *, const int *,
-                                        const float *, float *, float *, int, int, int, int, int, int, hipStream_t);
+                                        const float *, float *, float *, int, int, int, int, int, int, int, hipStream_t);
 hipError_t launch_scatter_values(const int *, const int *, const float *, float *, int, hipStream_t);
 hipError_t launch_seg_reduce(const LongRow *, int, const int *, const float *, float *, int, int, hipStream_t);
 hipError_t launch_long_rows(const LongChunk *, int, const LongRow *, int, const int *, const float *,
@@ -647,7 +647,7 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
     TF_PHASE(s, "fused_spmm_spmm_march_kernel", st,
              tf::launch_fused_spmm_spmm_march(d->m_runs, (int)s->march_runs.size() / 2, d->m_row_ptr, d->m_load_ptr, d->m_load,
                                               d->m_row_out, d->m_ell, C->d, D->d, d->m_trash, s->opts.N, s->lds_bytes, s->march_tpg,
-                                              s->march_dpg, s->march_lpg, acc, st));
+                                              s->march_dpg, s->march_lpg, s->march_width, acc, st));
     return TF_OK;
   }
   if (s->windowed) {

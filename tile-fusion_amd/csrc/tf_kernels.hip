@@ -1599,6 +1599,9 @@ __device__ __forceinline__ fvec<4> march_gather(const char *lane_base, int off) 
 
 // One ELL row: the lanes of a quad hold two (LDS offset, value) pairs each.  Four gathers are in
 // flight at a time (eight measured no faster and cost sixteen registers).
+// W: the longest row of either pattern (8, or 7 and less: a 7-point stencil's rows never fill the eighth
+// pair, which then is neither gathered nor multiplied).
+template <int W>
 __device__ __forceinline__ fvec<4> march_row(const int4 e, const char *lane_base) {
   fvec<4> x[4];
   x[0] = march_gather<0>(lane_base, e.x); x[1] = march_gather<0>(lane_base, e.z);
@@ -1607,9 +1610,11 @@ __device__ __forceinline__ fvec<4> march_row(const int4 e, const char *lane_base
   quad_fma<0>(e.y, x[0], acc); quad_fma<0>(e.w, x[1], acc);
   x[0] = march_gather<2>(lane_base, e.x); x[1] = march_gather<2>(lane_base, e.z);
   quad_fma<1>(e.y, x[2], acc); quad_fma<1>(e.w, x[3], acc);
-  x[2] = march_gather<3>(lane_base, e.x); x[3] = march_gather<3>(lane_base, e.z);
+  x[2] = march_gather<3>(lane_base, e.x);
+  if constexpr (W > 7) x[3] = march_gather<3>(lane_base, e.z);
   quad_fma<2>(e.y, x[0], acc); quad_fma<2>(e.w, x[1], acc);
-  quad_fma<3>(e.y, x[2], acc); quad_fma<3>(e.w, x[3], acc);
+  quad_fma<3>(e.y, x[2], acc);
+  if constexpr (W > 7) quad_fma<3>(e.w, x[3], acc);
   return acc;
 }
 
@@ -1635,7 +1640,7 @@ struct MarchStage {
   fvec<4> c[kMarchLpg];
 };
 
-template <bool ACC>
+template <bool ACC, int W>
 __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
     const int2 *__restrict__ runs, int n_runs, int per_xcd, const int *__restrict__ row_ptr,
     const int *__restrict__ load_ptr, const int2 *__restrict__ load_list, const int *__restrict__ row_out,
@@ -1742,7 +1747,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
       static_for<0, kMarchTpg>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
         share(uc);
-        const fvec<4> acc = march_row(cur.et[u], lane_base);
+        const fvec<4> acc = march_row<W>(cur.et[u], lane_base);
         *reinterpret_cast<fvec<4> *>(lane_base + ~cur.ot[u]) = acc;
       });
       lds_barrier();
@@ -1750,7 +1755,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
       static_for<0, kMarchDpg>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
         share(std::integral_constant<int, kMarchTpg + u>{});
-        fvec<4> acc = march_row(cur.ed[u], lane_base);
+        fvec<4> acc = march_row<W>(cur.ed[u], lane_base);
         float *dst = cur.od[u] >= 0 ? Dl + (size_t)cur.od[u] * N : Tl;
         if (ACC) vadd<4>(*reinterpret_cast<const fvec<4> *>(dst), acc);
         store_streaming<4>(dst, acc);
@@ -2161,20 +2166,25 @@ hipError_t launch_march_fill(const int *off, const int *src, const float *Ax, co
 hipError_t launch_fused_spmm_spmm_march(const int *runs, int n_runs, const int *row_ptr, const int *load_ptr,
                                         const int *load_list, const int *row_out, const int *ell, const float *C,
                                         float *D, float *trash, int N, int lds_bytes, int tpg, int dpg, int lpg,
-                                        int accumulate, hipStream_t st) {
+                                        int width, int accumulate, hipStream_t st) {
   if (n_runs <= 0) return hipSuccess;
   // (rows per lane group and iteration beyond what the kernel's register sets hold would be skipped silently)
-  if (N % 64 != 0 || tpg < 1 || tpg > kMarchTpg || dpg < 1 || dpg > kMarchDpg || lpg < 1 || lpg > kMarchLpg || lds_bytes > 163840)
+  if (N % 64 != 0 || tpg < 1 || tpg > kMarchTpg || dpg < 1 || dpg > kMarchDpg || lpg < 1 || lpg > kMarchLpg || lds_bytes > 163840 ||
+      width < 0 || width > kMarchW)
     return hipErrorInvalidValue;
   const int per = per_xcd_of(n_runs);
   hipError_t err = hipSuccess;
-#define CALLM(ACC_)                                                                                               \
-  err = allow_lds(fused_spmm_spmm_march_kernel<ACC_>, lds_bytes);                                                 \
+#define CALLM(ACC_, W_)                                                                                           \
+  err = allow_lds(fused_spmm_spmm_march_kernel<ACC_, W_>, lds_bytes);                                             \
   if (err == hipSuccess)                                                                                          \
-    hipLaunchKernelGGL((fused_spmm_spmm_march_kernel<ACC_>), dim3(grid_of(n_runs)), dim3(kMarchBlock),            \
+    hipLaunchKernelGGL((fused_spmm_spmm_march_kernel<ACC_, W_>), dim3(grid_of(n_runs)), dim3(kMarchBlock),        \
                        lds_bytes, st, reinterpret_cast<const int2 *>(runs), n_runs, per, row_ptr, load_ptr,       \
                        reinterpret_cast<const int2 *>(load_list), row_out, reinterpret_cast<const int4 *>(ell), C, D, trash, N)
-  if (accumulate) { CALLM(true); } else { CALLM(false); }
+  if (width <= 7) {
+    if (accumulate) { CALLM(true, 7); } else { CALLM(false, 7); }
+  } else {
+    if (accumulate) { CALLM(true, 8); } else { CALLM(false, 8); }
+  }
 #undef CALLM
   return err != hipSuccess ? err : hipGetLastError();
 }

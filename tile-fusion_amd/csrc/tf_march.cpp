@@ -64,8 +64,11 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
   if (S->L != M || o.inner_cols != M || o.N % 64 != 0) return false;
   const long long nnzA = Ap[M], nnzB = Bp[M];
   if (nnzA >= kMarchSrcA || nnzB >= kMarchSrcA) return false;
-  for (int i = 0; i < M; ++i)
+  int width = 0;
+  for (int i = 0; i < M; ++i) {
     if (Ap[i + 1] - Ap[i] > kMarchW || Bp[i + 1] - Bp[i] > kMarchW) return false;
+    width = std::max(width, std::max(Ap[i + 1] - Ap[i], Bp[i + 1] - Bp[i]));
+  }
   int grid[3] = {given.grid_nx, given.grid_ny, given.grid_nz};
   if (grid[0] > 0 || grid[1] > 0 || grid[2] > 0) {
     if (grid[0] <= 0 || grid[1] <= 0 || grid[2] <= 0 || (long long)grid[0] * grid[1] * grid[2] != M) return false;
@@ -254,6 +257,7 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
     S->march_grid[0] = nx; S->march_grid[1] = ny; S->march_grid[2] = nz;
     S->march_tile[0] = bx; S->march_tile[1] = by;
     S->march_slots = max_slots;
+    S->march_width = width;
     S->march_tpg = std::max(1, (max_t + kMarchGroups - 1) / kMarchGroups);
     S->march_dpg = std::max(1, (max_d + kMarchGroups - 1) / kMarchGroups);
     S->march_lpg = std::max(1, (max_loads + kMarchGroups - 1) / kMarchGroups);
@@ -336,6 +340,10 @@ tf_status validate_march(const tf_schedule *s, int M, const int *Ap, const int *
     return fail(TF_ESCHEDULE, "marching schedule: tables do not match");
   if (s->march_tpg < 1 || s->march_tpg > kMarchTpg || s->march_dpg < 1 || s->march_dpg > kMarchDpg || s->march_lpg < 1 || s->march_lpg > kMarchLpg)
     return fail(TF_ESCHEDULE, "marching schedule: rows per lane group out of range");
+  // the kernel leaves out the eighth pair of every row when no row has more than seven entries
+  for (int i = 0; i < M; ++i)
+    if (Ap[i + 1] - Ap[i] > s->march_width || Bp[i + 1] - Bp[i] > s->march_width)
+      return fail(TF_ESCHEDULE, "marching schedule: row %d has more than the %d entries the schedule says is the most", i, s->march_width);
   const int n_iters = (int)s->march_load_ptr.size() - 1;
   std::vector<int> done(M, 0);
   // slot contents: kind 0 nothing, 1 a row of C, 2 an intermediate row; rstamp/wstamp: the phase (counted
