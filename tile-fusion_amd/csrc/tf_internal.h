@@ -123,7 +123,7 @@ struct tf_schedule {
   int march_grid[3] = {0, 0, 0};     // the grid the runs were cut from (x fastest)
   int march_tile[2] = {0, 0};        // grid points per run and plane: x, y
   int march_slots = 0;               // LDS slots in use by the fullest run
-  int march_width = tf::kMarchW;         // entries of the longest row of either pattern (the kernel skips the eighth pair when <= 7)
+  int march_width = tf::kMarchW;         // entries of the longest row of either pattern (the kernel takes only that many pairs of a row, five at least)
   int march_tpg = 0, march_dpg = 0, march_lpg = 0;  // intermediate rows / second-op rows / C rows a lane group handles per iteration, at most
   std::vector<int> march_runs;       // (first iteration, iterations) per run
   std::vector<int> march_row_ptr;    // [2 * iterations + 1] into the ELL rows

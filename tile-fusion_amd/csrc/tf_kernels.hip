@@ -1599,21 +1599,24 @@ __device__ __forceinline__ fvec<4> march_gather(const char *lane_base, int off) 
 
 // One ELL row: the lanes of a quad hold two (LDS offset, value) pairs each.  Four gathers are in
 // flight at a time (eight measured no faster and cost sixteen registers).
-// W: the longest row of either pattern (8, or 7 and less: a 7-point stencil's rows never fill the eighth
-// pair, which then is neither gathered nor multiplied).
+// W: the longest row of either pattern, 5 .. 8: a 7-point stencil's rows never fill the eighth pair, a
+// 5-point stencil's not the last three, which then are neither gathered nor multiplied.
 template <int W>
 __device__ __forceinline__ fvec<4> march_row(const int4 e, const char *lane_base) {
+  static_assert(W >= 5 && W <= 8, "pairs 0 .. 4 are always taken");
   fvec<4> x[4];
   x[0] = march_gather<0>(lane_base, e.x); x[1] = march_gather<0>(lane_base, e.z);
   x[2] = march_gather<1>(lane_base, e.x); x[3] = march_gather<1>(lane_base, e.z);
   fvec<4> acc = vzero<4>();
   quad_fma<0>(e.y, x[0], acc); quad_fma<0>(e.w, x[1], acc);
-  x[0] = march_gather<2>(lane_base, e.x); x[1] = march_gather<2>(lane_base, e.z);
+  x[0] = march_gather<2>(lane_base, e.x);
+  if constexpr (W > 5) x[1] = march_gather<2>(lane_base, e.z);
   quad_fma<1>(e.y, x[2], acc); quad_fma<1>(e.w, x[3], acc);
-  x[2] = march_gather<3>(lane_base, e.x);
+  if constexpr (W > 6) x[2] = march_gather<3>(lane_base, e.x);
   if constexpr (W > 7) x[3] = march_gather<3>(lane_base, e.z);
-  quad_fma<2>(e.y, x[0], acc); quad_fma<2>(e.w, x[1], acc);
-  quad_fma<3>(e.y, x[2], acc);
+  quad_fma<2>(e.y, x[0], acc);
+  if constexpr (W > 5) quad_fma<2>(e.w, x[1], acc);
+  if constexpr (W > 6) quad_fma<3>(e.y, x[2], acc);
   if constexpr (W > 7) quad_fma<3>(e.w, x[3], acc);
   return acc;
 }
@@ -2180,10 +2183,11 @@ hipError_t launch_fused_spmm_spmm_march(const int *runs, int n_runs, const int *
     hipLaunchKernelGGL((fused_spmm_spmm_march_kernel<ACC_, W_>), dim3(grid_of(n_runs)), dim3(kMarchBlock),        \
                        lds_bytes, st, reinterpret_cast<const int2 *>(runs), n_runs, per, row_ptr, load_ptr,       \
                        reinterpret_cast<const int2 *>(load_list), row_out, reinterpret_cast<const int4 *>(ell), C, D, trash, N)
-  if (width <= 7) {
-    if (accumulate) { CALLM(true, 7); } else { CALLM(false, 7); }
-  } else {
-    if (accumulate) { CALLM(true, 8); } else { CALLM(false, 8); }
+  switch (width <= 5 ? 5 : width) {
+    case 5: if (accumulate) { CALLM(true, 5); } else { CALLM(false, 5); } break;
+    case 6: if (accumulate) { CALLM(true, 6); } else { CALLM(false, 6); } break;
+    case 7: if (accumulate) { CALLM(true, 7); } else { CALLM(false, 7); } break;
+    default: if (accumulate) { CALLM(true, 8); } else { CALLM(false, 8); } break;
   }
 #undef CALLM
   return err != hipSuccess ? err : hipGetLastError();

@@ -340,7 +340,7 @@ tf_status validate_march(const tf_schedule *s, int M, const int *Ap, const int *
     return fail(TF_ESCHEDULE, "marching schedule: tables do not match");
   if (s->march_tpg < 1 || s->march_tpg > kMarchTpg || s->march_dpg < 1 || s->march_dpg > kMarchDpg || s->march_lpg < 1 || s->march_lpg > kMarchLpg)
     return fail(TF_ESCHEDULE, "marching schedule: rows per lane group out of range");
-  // the kernel leaves out the eighth pair of every row when no row has more than seven entries
+  // the kernel takes only the first march_width pairs of every row
   for (int i = 0; i < M; ++i)
     if (Ap[i + 1] - Ap[i] > s->march_width || Bp[i + 1] - Bp[i] > s->march_width)
       return fail(TF_ESCHEDULE, "marching schedule: row %d has more than the %d entries the schedule says is the most", i, s->march_width);
