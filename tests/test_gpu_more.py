@@ -252,6 +252,38 @@ def test_many_rows_without_entries(gpu, tf, orc):
     assert np.allclose(acc[~empty], want[~empty] + 1.5, rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("N", [32, 64, 96, 128, 160, 192, 224, 256])
+def test_gemm_every_output_width(gpu, tf, N):
+    """tf_gemm (the row GEMM on fp32 MFMA, a lane stores N/32 consecutive columns of each of its rows) for every
+    width it takes, row counts that are no multiple of the 32-row block, K that is no multiple of 8, and the same
+    kernel behind a row list inside tf_gemm_spmm -- against float64, to 1e-5 / 1e-4."""
+    say(f"gemm N={N}")
+    rng = np.random.default_rng(3)
+    for K in (8, 40, 200):
+        for M in (1, 31, 4097):
+            X = rng.standard_normal((M, K)).astype(np.float32)
+            W = rng.standard_normal((K, N)).astype(np.float32)
+            Y = tf.DenseMatrix(M, N); Y.fill(float("nan"))
+            tf.gemm(tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W), Y)
+            want = X.astype(np.float64) @ W.astype(np.float64)
+            assert np.abs(Y.to_numpy() - want).max() <= 1e-5 * max(np.abs(want).max(), 1e-30), (M, K, N)
+    A = tf.workloads.make_config(3, 0.02)["A"].tolil()
+    A[:, ::3] = 0                                   # a third of the intermediate rows is never read: a row list
+    A = A.tocsr(); A.eliminate_zeros(); A.sort_indices()
+    A = sp.csr_matrix((A.data.astype(np.float32), A.indices.astype(np.int32), A.indptr.astype(np.int32)), shape=A.shape)
+    n = A.shape[0]
+    B = rng.standard_normal((n, 64)).astype(np.float32)
+    W = rng.standard_normal((64, N)).astype(np.float32)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=N, K=64)
+    S.validate()
+    assert 0 < S.info()["n_writeback_rows"] < n
+    D = tf.DenseMatrix(n, N)
+    tf.gemm_spmm(Ah, tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W), D, S)
+    want = A.astype(np.float64) @ (B.astype(np.float64) @ W.astype(np.float64))
+    assert np.abs(D.to_numpy() - want).max() <= TOL * np.abs(want).max()
+
+
 def test_device_reports_the_workgroup_to_xcd_mapping(gpu):
     """tf_device_init probes what the XCD-pinned kernels rely on: workgroup b runs on XCD b mod 8."""
     assert gpu["xcds"] == 8 and gpu["compute_units"] == 256 and gpu["wavefront"] == 64
