@@ -259,8 +259,8 @@ def test_gemm_every_output_width(gpu, tf, N):
     kernel behind a row list inside tf_gemm_spmm -- against float64, to 1e-5 / 1e-4."""
     say(f"gemm N={N}")
     rng = np.random.default_rng(3)
-    for K in (8, 40, 200):
-        for M in (1, 31, 4097):
+    for K in (8, 40, 128, 200, 256):                # 128 and 256 have kernels with K built in (N <= 128)
+        for M in (1, 31, 4097, 70000):              # 70,000 rows: more than one block per wavefront
             X = rng.standard_normal((M, K)).astype(np.float32)
             W = rng.standard_normal((K, N)).astype(np.float32)
             Y = tf.DenseMatrix(M, N); Y.fill(float("nan"))
@@ -272,16 +272,17 @@ def test_gemm_every_output_width(gpu, tf, N):
     A = A.tocsr(); A.eliminate_zeros(); A.sort_indices()
     A = sp.csr_matrix((A.data.astype(np.float32), A.indices.astype(np.int32), A.indptr.astype(np.int32)), shape=A.shape)
     n = A.shape[0]
-    B = rng.standard_normal((n, 64)).astype(np.float32)
-    W = rng.standard_normal((64, N)).astype(np.float32)
     Ah = tf.CsrMatrix.from_scipy(A)
-    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=N, K=64)
-    S.validate()
-    assert 0 < S.info()["n_writeback_rows"] < n
-    D = tf.DenseMatrix(n, N)
-    tf.gemm_spmm(Ah, tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W), D, S)
-    want = A.astype(np.float64) @ (B.astype(np.float64) @ W.astype(np.float64))
-    assert np.abs(D.to_numpy() - want).max() <= TOL * np.abs(want).max()
+    for K in (64, 128):
+        B = rng.standard_normal((n, K)).astype(np.float32)
+        W = rng.standard_normal((K, N)).astype(np.float32)
+        S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=N, K=K)
+        S.validate()
+        assert 0 < S.info()["n_writeback_rows"] < n
+        D = tf.DenseMatrix(n, N)
+        tf.gemm_spmm(Ah, tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W), D, S)
+        want = A.astype(np.float64) @ (B.astype(np.float64) @ W.astype(np.float64))
+        assert np.abs(D.to_numpy() - want).max() <= TOL * np.abs(want).max(), (K, N)
 
 
 def test_device_reports_the_workgroup_to_xcd_mapping(gpu):

@@ -973,7 +973,12 @@ __device__ __forceinline__ void stage_weights(const float *__restrict__ W, int K
 
 constexpr int kGemmSeg = 16;  // row blocks whose row numbers a wavefront keeps in LDS at a time
 
-template <int NB, bool LIST>
+// G4C > 0: K = 32 G4C is known when the kernel is built, and a block's MFMAs, the requests for the operands
+// three groups ahead and the reads of W one step ahead are one stretch of code without a branch: a wavefront
+// issues in order, so address arithmetic, a wait for a row number or a branch between two MFMAs leaves the
+// pipe without work from this wavefront (39,000 -> 33,500 cycles per block and wavefront for K = 128, of
+// which the block's 256 MFMAs of the two wavefronts of a SIMD take 32,800).
+template <int NB, bool LIST, int G4C>
 __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__restrict__ X,
                                                                const float *__restrict__ W,
                                                                float *__restrict__ Y,
@@ -1039,6 +1044,62 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
     const int total_groups = (rb_end - rb0) * G4;
     // row (of X and Y) behind position x of this segment
     auto row_at = [&](int x) { return LIST ? ridx[x] : min(rb0 * 32 + x, n_rows - 1); };
+    if constexpr (G4C > 0) {
+      static_assert(G4C >= 4 && G4C % 4 == 0, "four operand sets in turn, a block starts with the first");
+      const int nblk = rb_end - rb0;
+      auto operand_row = [&](int b) { return X + (size_t)row_at(min(b, nblk - 1) * 32 + j) * K + 4 * h; };
+      const float *pc = operand_row(0);
+      fvec<4> set[4][4];
+#pragma unroll
+      for (int q = 0; q < 3; ++q)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) set[q][u] = load4(pc + q * 32 + 8 * u);
+      wvec<NB> bw[4], bn[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) bw[t] = wl[t * 32];
+      // accumulator register r of block b, all NB column blocks, into its row of Y
+      auto store_row = [&](const v16f (&acc)[NB], int b, int r) __attribute__((always_inline)) {
+        wvec<NB> out;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) out.v[nb] = acc[nb][r];
+        *reinterpret_cast<wvec<NB> *>(Y + (size_t)row_at(b * 32 + 8 * (r / 4) + 4 * h + (r % 4)) * N + NB * j) = out;
+      };
+      for (int b = 0; b < nblk; ++b) {
+        const float *pn = operand_row(b + 1);
+        v16f acc[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
+#pragma unroll
+        for (int g = 0; g < G4C; ++g) {
+          const float *src = g + 3 < G4C ? pc + (g + 3) * 32 : pn + (g + 3 - G4C) * 32;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) set[(g + 3) % 4][u] = load4(src + 8 * u);
+          __builtin_amdgcn_sched_barrier(0);  // the requests stay here: the scheduler would move them to the block's end
+#pragma unroll
+          for (int t2 = 0; t2 < 4; t2 += 2) {
+            const int st = 4 * g + t2;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) bn[t] = wl[(8 * (st + 1) + t) * 32];
+            mfma_step8<NB>(set[g % 4][t2], bw, acc);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) bw[t] = wl[(8 * ((st + 2) % (4 * G4C)) + t) * 32];
+            mfma_step8<NB>(set[g % 4][t2 + 1], bn, acc);
+          }
+        }
+        if ((rb0 + b + 1) * 32 <= n_rows) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) store_row(acc, b, r);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if ((rb0 + b) * 32 + 8 * (r / 4) + 4 * h + (r % 4) < n_rows) store_row(acc, b, r);
+        }
+        pc = pn;
+      }
+      continue;
+    }
     // A operand of group gi (block rb0 + gi / G4, steps 4 (gi % G4) ..): four 16-byte loads per lane,
     // always issued (block and k clamped to existing ones, the surplus is never used) so that the
     // loads of later groups stay in flight while earlier ones are consumed.
@@ -2095,15 +2156,27 @@ hipError_t launch_gemm(const float *X, const float *W, float *Y, const int *rows
     const int nrb = (n_rows + 31) / 32;
     const int grid = std::max(1, std::min(compute_units * per_cu, (nrb + kGemmBlock / 64 - 1) / (kGemmBlock / 64)));
     const int lds = w_bytes + (rows ? (kGemmBlock / 64) * kGemmSeg * 32 * 4 : 0);  // + the wavefronts' row numbers
-#define CALL2(NB_, LIST_)                                                                           \
-  err = allow_lds(gemm_rows_kernel<NB_, LIST_>, lds);                                               \
+#define CALL3(NB_, LIST_, G4C_)                                                                     \
+  err = allow_lds(gemm_rows_kernel<NB_, LIST_, G4C_>, lds);                                         \
   if (err == hipSuccess)                                                                            \
-    hipLaunchKernelGGL((gemm_rows_kernel<NB_, LIST_>), dim3(grid), dim3(kGemmBlock), lds, st, X, W, Y, \
+    hipLaunchKernelGGL((gemm_rows_kernel<NB_, LIST_, G4C_>), dim3(grid), dim3(kGemmBlock), lds, st, X, W, Y, \
                        rows, n_rows, K)
+  // K = 128 and 256 with up to 128 columns have kernels of their own (K built in)
+#define CALL2(NB_, LIST_)                        \
+  do {                                           \
+    if constexpr (NB_ <= 4) {                    \
+      if (K == 128) { CALL3(NB_, LIST_, 4); }    \
+      else if (K == 256) { CALL3(NB_, LIST_, 8); } \
+      else { CALL3(NB_, LIST_, 0); }             \
+    } else {                                     \
+      CALL3(NB_, LIST_, 0);                      \
+    }                                            \
+  } while (0)
 #define CALL(NB_) do { if (rows) { CALL2(NB_, true); } else { CALL2(NB_, false); } } while (0)
     TF_DISPATCH_NB(NB, CALL);
 #undef CALL
 #undef CALL2
+#undef CALL3
     return err != hipSuccess ? err : hipGetLastError();
   }
   if (rows) return hipErrorInvalidValue;  // the streamed-W kernel takes contiguous rows only
