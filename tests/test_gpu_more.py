@@ -285,6 +285,39 @@ def test_gemm_every_output_width(gpu, tf, N):
         assert np.abs(D.to_numpy() - want).max() <= TOL * np.abs(want).max(), (K, N)
 
 
+def test_row_gemm_of_a_schedule_repeats_bit_for_bit(gpu, tf):
+    """The row GEMM behind a row list with K built in (128, 256): three calls in a row on one schedule, D
+    poisoned in between and a schedule of another size used in between, give the same bits each time (a run
+    with fewer than two row blocks per wavefront and one with more)."""
+    say("gemm repeats")
+    rng = np.random.default_rng(5)
+    A = tf.workloads.make_config(3, 0.25)["A"]                 # 50,000 nodes: 1,563 row blocks, fewer than wavefronts
+    A2 = tf.workloads.make_config(3, 0.6)["A"]                 # 120,000 nodes: 3,750 row blocks
+    for K in (128, 256):
+        runs = []
+        for M_ in (A, A2):
+            n = M_.shape[0]
+            Ah = tf.CsrMatrix.from_scipy(M_)
+            B = tf.DenseMatrix.from_numpy(rng.standard_normal((n, K)).astype(np.float32))
+            W = tf.DenseMatrix.from_numpy(rng.standard_normal((K, 128)).astype(np.float32))
+            S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=K)
+            S.validate()
+            assert S.info()["n_writeback_rows"] > 0
+            want = M_.astype(np.float64) @ (B.to_numpy().astype(np.float64) @ W.to_numpy().astype(np.float64))
+            runs.append((Ah, B, W, S, tf.DenseMatrix(n, 128), want))
+        first = {}
+        for rep in range(3):
+            for i, (Ah, B, W, S, D, want) in enumerate(runs):
+                D.fill(float("nan"))
+                tf.gemm_spmm(Ah, B, W, D, S)
+                got = D.to_numpy()
+                assert np.abs(got - want).max() <= TOL * np.abs(want).max(), (K, i, rep)
+                if rep == 0:
+                    first[i] = got
+                else:
+                    assert np.array_equal(got, first[i]), (K, i, rep)
+
+
 def test_device_reports_the_workgroup_to_xcd_mapping(gpu):
     """tf_device_init probes what the XCD-pinned kernels rely on: workgroup b runs on XCD b mod 8."""
     assert gpu["xcds"] == 8 and gpu["compute_units"] == 256 and gpu["wavefront"] == 64
