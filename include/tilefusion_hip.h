@@ -152,7 +152,11 @@ typedef struct {
                             defaults for fields a caller built against an older header does not
                             have.  Must be set (TF_EINVAL when it is 0 or too small to hold N). */
   int op;                /* TF_OP_SPMM_SPMM or TF_OP_GEMM_SPMM                               */
-  int N;                 /* columns of C and D (reference: bCols / EmbedDim)                 */
+  int N;                 /* columns of C and D (reference: bCols / EmbedDim).  Any N > 0.  The
+                            MFMA kernels of GeMM-SpMM take 32, 64 .. 256 columns: for any other
+                            N the schedule is built for equal column panels of such a width
+                            (48 -> one of 64, 300 -> two of 160) and the executor runs one pass
+                            per panel through a panel of C and of D in the schedule's workspace */
   int K;                 /* GeMM-SpMM: columns of dense B = rows of C (FeatureDim); else 0.
                             Any K > 0: the kernels step k by 8, so for other K the executor
                             copies B and C, zero-padded to the next multiple of 8, into the

@@ -63,6 +63,17 @@ int main() {
     if (D2[i] != want[i]) { std::printf("gemm-spmm mismatch at %zu: %g vs %g\n", i, D2[i], want[i]); return 1; }
   if (sched.n1_ != 2 || sched.ptr1_[0] != 0 || sched.ptr2_[0] != 0) { std::printf("schedule view is off\n"); return 1; }
 
+  // A width the MFMA kernels do not take (the reference's bCols is free): 44 columns, host operands.
+  {
+    const int N2 = 44;
+    std::vector<float> W2h((size_t)K * N2, 1.f), D3((size_t)M * N2, 0.f), kk2((size_t)M * N2, (float)K), want2((size_t)M * N2);
+    def::Matrix Bq(M, K, Bh.data()), W2(K, N2, W2h.data()), D3m(M, N2, D3.data());
+    fusion::geMMSpMMExecutor(A, Bq, W2, D3m, sched, 8);
+    stencil(n, N2, kk2, want2);
+    for (size_t i = 0; i < D3.size(); ++i)
+      if (D3[i] != want2[i]) { std::printf("gemm-spmm (44 columns) mismatch at %zu: %g vs %g\n", i, D3[i], want2[i]); return 1; }
+  }
+
   // Errors throw instead of exiting.
   bool threw = false;
   try {

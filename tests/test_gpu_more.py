@@ -285,6 +285,30 @@ def test_gemm_every_output_width(gpu, tf, N):
         assert np.abs(D.to_numpy() - want).max() <= TOL * np.abs(want).max(), (K, N)
 
 
+@pytest.mark.parametrize("N", [7, 16, 48, 100, 300, 512, 700])
+def test_gemm_spmm_of_any_width(gpu, tf, N):
+    """geMMSpMMExecutor takes C of any width (the reference's bCols is free): widths the MFMA kernels do not
+    take run as column panels.  Against float64, with K that needs padding too, with and without
+    TF_ACCUMULATE, on a pattern that fuses (band) and one that does not (Erdos-Renyi)."""
+    say(f"gemm_spmm N={N}")
+    rng = np.random.default_rng(N)
+    for A in (tf.workloads.banded_random(3000, 32, 12, seed=4), tf.workloads.make_config(3, 0.02)["A"]):
+        n = A.shape[0]
+        Ah = tf.CsrMatrix.from_scipy(A)
+        for K in (20, 64):
+            B = rng.uniform(-1, 1, (n, K)).astype(np.float32)
+            W = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+            S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=N, K=K)
+            S.validate()
+            want = A.astype(np.float64) @ (B.astype(np.float64) @ W.astype(np.float64))
+            D0 = rng.uniform(-1, 1, (n, N)).astype(np.float32)
+            for acc in (False, True):
+                D = tf.DenseMatrix.from_numpy(D0.copy())
+                tf.gemm_spmm(Ah, tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W), D, S, accumulate=acc)
+                exp = want + (D0 if acc else 0)
+                assert np.abs(D.to_numpy() - exp).max() <= TOL * np.abs(exp).max(), (N, K, acc)
+
+
 def test_row_gemm_of_a_schedule_repeats_bit_for_bit(gpu, tf):
     """The row GEMM behind a row list with K built in (128, 256): three calls in a row on one schedule, D
     poisoned in between and a schedule of another size used in between, give the same bits each time (a run

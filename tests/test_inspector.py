@@ -171,9 +171,13 @@ def test_rectangular_and_bad_arguments(tf):
         with pytest.raises(tf.TileFusionError) as e:
             tf.inspector(Ah, 1, **kw)
         assert e.value.status == -1
-    with pytest.raises(tf.TileFusionError) as e:
-        tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=48, K=64)
-    assert e.value.status == -5
+    # GeMM-SpMM of any width: the schedule is built for column panels of a width the MFMA kernels take
+    # (48 -> one panel of 64, 300 -> two of 160, 700 -> three of 256) and says so in its workspace
+    sq = tf.CsrMatrix.from_scipy(A2[:, :200])
+    for N, panel in ((48, 64), (300, 160), (700, 256), (7, 32)):
+        Sp = tf.inspector(sq, 1, op=tf.OP_GEMM_SPMM, N=N, K=64)
+        Sp.validate()
+        assert Sp.info()["N"] == N and Sp.info()["workspace_bytes"] >= (200 + 64) * panel * 4
     Sq = tf.inspector(tf.CsrMatrix.from_scipy(A2[:, :200]), 1, op=tf.OP_GEMM_SPMM, N=64, K=20)  # any K: padded to 24
     assert Sq.info()["K"] == 20 and Sq.info()["workspace_bytes"] >= (200 + 64) * 24 * 4
     bad = tf.CsrMatrix(4, 4, [0, 1, 2, 3, 4], [0, 1, 9, 3], [1, 1, 1, 1])

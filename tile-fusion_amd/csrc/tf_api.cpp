@@ -59,6 +59,8 @@ struct DeviceSchedule {
   float *hidden = nullptr;   // tf_gcn_two_layers: the first layer's output, L x K of this (second-layer) schedule
   float *Bpad = nullptr;     // M x K' and K' x N copies of B and C, zero-padded, when K is not a multiple of 8
   float *Cpad = nullptr;
+  float *Cpanel = nullptr;   // K' x N and L x N: one column panel of C (zero-padded) and of D, when the caller's width is
+  float *Dpanel = nullptr;   // not one the kernels take (user_N != N)
   // marching runs: the schedule's lists, and the ELL rows with the operands' values filled in
   int *m_runs = nullptr, *m_row_ptr = nullptr, *m_load_ptr = nullptr, *m_load = nullptr, *m_row_out = nullptr;
   int *m_ell_off = nullptr, *m_ell_src = nullptr, *m_ell = nullptr;
@@ -103,6 +105,7 @@ hipError_t launch_fused_gemm_spmm_stream(const TileDesc *, int, const int *, con
 hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t);
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 hipError_t launch_pad(const float *, int, int, float *, int, int, hipStream_t);
+hipError_t launch_copy_cols(const float *, int, int, int, int, float *, int, int, int, int, int, hipStream_t);
 hipError_t launch_relu(float *, size_t, hipStream_t);
 hipError_t launch_zero_rows(const int *, int, float *, int, hipStream_t);
 hipError_t launch_xcd_probe(int *, int, hipStream_t);
@@ -148,7 +151,7 @@ void release_device_schedule(DeviceSchedule *d) {
   (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows); (void)hipFree(d->seg_groups);
   (void)hipFree(d->seg_ptr); (void)hipFree(d->ent_src); (void)hipFree(d->ent_pos); (void)hipFree(d->seg_col); (void)hipFree(d->lrow_seg); (void)hipFree(d->seg_val);
   (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
-  (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad); (void)hipFree(d->hidden);
+  (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad); (void)hipFree(d->Cpanel); (void)hipFree(d->Dpanel); (void)hipFree(d->hidden);
   (void)hipFree(d->rem_ptr); (void)hipFree(d->rem_col); (void)hipFree(d->rem_src); (void)hipFree(d->rem_val);
   (void)hipFree(d->m_runs); (void)hipFree(d->m_row_ptr); (void)hipFree(d->m_load_ptr); (void)hipFree(d->m_load);
   (void)hipFree(d->m_row_out); (void)hipFree(d->m_ell_off); (void)hipFree(d->m_ell_src); (void)hipFree(d->m_ell); (void)hipFree(d->m_trash);
@@ -239,6 +242,11 @@ static tf_status ensure_device(tf_schedule *s) {
   if (!rc && s->n_writeback_rows > 0) {
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->inter), (size_t)s->M * s->opts.N * sizeof(float));
     if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(intermediate)");
+  }
+  if (!rc && s->opts.op == TF_OP_GEMM_SPMM && s->user_N != s->opts.N) {
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->Cpanel), (size_t)s->opts.K * s->opts.N * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&d->Dpanel), (size_t)s->L * s->opts.N * sizeof(float));
+    if (e != hipSuccess) rc = hip_fail(e, "hipMalloc(column panels)");
   }
   if (!rc && s->opts.op == TF_OP_GEMM_SPMM && s->user_K != s->opts.K) {
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&d->Bpad), (size_t)s->M * s->opts.K * sizeof(float));
@@ -613,8 +621,8 @@ static tf_status check_common(const char *who, const tf_csr *A, const tf_dense *
                 who, s->L, s->M, s->nnz, A->M, A->N, A->nnz);
   if (A->hash && A->hash != s->pattern_hash)
     return fail(TF_ESCHEDULE, "%s: A has the shape and entry count the schedule was built for, but another sparsity pattern", who);
-  if (C->N != s->opts.N || D->N != s->opts.N)
-    return fail(TF_ESCHEDULE, "%s: schedule was built for N = %d, C has %d and D has %d columns", who, s->opts.N, C->N, D->N);
+  if (C->N != s->user_N || D->N != s->user_N)
+    return fail(TF_ESCHEDULE, "%s: schedule was built for N = %d, C has %d and D has %d columns", who, s->user_N, C->N, D->N);
   if (D->M != A->M) return fail(TF_EINVAL, "%s: D has %d rows, A has %d", who, D->M, A->M);
   return TF_OK;
 }
@@ -691,27 +699,11 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
   return tf::run_remainder(A, D, s, acc, false, st);
 }
 
-extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf_dense *D,
-                                  tf_schedule *s, unsigned flags, void *stream) {
-  tf_status rc = check_common("tf_gemm_spmm", A, C, D, s, TF_OP_GEMM_SPMM);
-  if (rc) return rc;
-  if (!B) return fail(TF_EINVAL, "tf_gemm_spmm: B is null");
-  if (B->M != A->N) return fail(TF_EINVAL, "tf_gemm_spmm: B has %d rows, A has %d columns", B->M, A->N);
-  if (B->N != s->user_K || C->M != s->user_K)
-    return fail(TF_ESCHEDULE, "tf_gemm_spmm: schedule was built for K = %d, B has %d columns and C has %d rows", s->user_K, B->N, C->M);
-  rc = tf::ensure_device(s);
-  if (rc) return rc;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
+// One pass of a GeMM-SpMM schedule: D (L x opts.N, dense) = A * (Bd * Cd) with Bd L' x opts.K and Cd opts.K x opts.N
+// as the kernels take them.
+static tf_status gemm_spmm_pass(const tf_csr *A, const float *Bd, const float *Cd, tf_dense *D, tf_schedule *s, int acc,
+                                unsigned flags, hipStream_t st) {
   tf::DeviceSchedule *d = s->dev;
-  d->prof_n = 0;
-  const float *Bd = B->d, *Cd = C->d;
-  if (s->user_K != s->opts.K) {  // zero-padded copies with K rounded up to 8 (the kernels' k step)
-    TF_PHASE(s, "pad_kernel (B)", st, tf::launch_pad(B->d, B->M, B->N, d->Bpad, B->M, s->opts.K, st));
-    TF_PHASE(s, "pad_kernel (C)", st, tf::launch_pad(C->d, C->M, C->N, d->Cpad, s->opts.K, C->N, st));
-    Bd = d->Bpad;
-    Cd = d->Cpad;
-  }
   const int n_launch = (int)s->launch_tiles.size();
   if (n_launch > 0) {
     if (s->gemm_stream)
@@ -749,6 +741,50 @@ extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_d
     }
   }
   return tf::run_remainder(A, D, s, acc, overlap && !s->plain_rows.empty(), st);
+}
+
+
+extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf_dense *D,
+                                  tf_schedule *s, unsigned flags, void *stream) {
+  tf_status rc = check_common("tf_gemm_spmm", A, C, D, s, TF_OP_GEMM_SPMM);
+  if (rc) return rc;
+  if (!B) return fail(TF_EINVAL, "tf_gemm_spmm: B is null");
+  if (B->M != A->N) return fail(TF_EINVAL, "tf_gemm_spmm: B has %d rows, A has %d columns", B->M, A->N);
+  if (B->N != s->user_K || C->M != s->user_K)
+    return fail(TF_ESCHEDULE, "tf_gemm_spmm: schedule was built for K = %d, B has %d columns and C has %d rows", s->user_K, B->N, C->M);
+  rc = tf::ensure_device(s);
+  if (rc) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int acc = (flags & TF_ACCUMULATE) ? 1 : 0;
+  tf::DeviceSchedule *d = s->dev;
+  d->prof_n = 0;
+  const float *Bd = B->d, *Cd = C->d;
+  const bool panels = s->user_N != s->opts.N;
+  if (s->user_K != s->opts.K) {  // zero-padded copies with K rounded up to 8 (the kernels' k step)
+    TF_PHASE(s, "pad_kernel (B)", st, tf::launch_pad(B->d, B->M, B->N, d->Bpad, B->M, s->opts.K, st));
+    Bd = d->Bpad;
+    if (!panels) {
+      TF_PHASE(s, "pad_kernel (C)", st, tf::launch_pad(C->d, C->M, C->N, d->Cpad, s->opts.K, C->N, st));
+      Cd = d->Cpad;
+    }
+  }
+  if (!panels) return gemm_spmm_pass(A, Bd, Cd, D, s, acc, flags, st);
+  // A width the MFMA kernels do not take: one pass per column panel of opts.N columns.  The panel of C is
+  // copied out (zero columns past N, zero rows past K), the pass writes a dense L x opts.N panel of D,
+  // and its columns are copied (or added, with TF_ACCUMULATE) into the caller's D.
+  tf_dense panel = *D;
+  panel.d = d->Dpanel;
+  panel.N = s->opts.N;
+  panel.owns = false;
+  for (int q = 0; q < s->n_panels; ++q) {
+    const int c0 = q * s->opts.N, w = std::min(s->opts.N, s->user_N - c0);
+    TF_PHASE(s, "copy_cols_kernel (panel of C)", st,
+             tf::launch_copy_cols(C->d, C->M, C->N, c0, w, d->Cpanel, s->opts.K, s->opts.N, 0, s->opts.N, 0, st));
+    if (tf_status rc2 = gemm_spmm_pass(A, Bd, d->Cpanel, &panel, s, 0, flags, st)) return rc2;
+    TF_PHASE(s, "copy_cols_kernel (panel of D)", st,
+             tf::launch_copy_cols(d->Dpanel, D->M, s->opts.N, 0, w, D->d, D->M, D->N, c0, w, acc, st));
+  }
+  return TF_OK;
 }
 
 extern "C" tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const tf_dense *W1, const tf_dense *W2, tf_dense *D,

@@ -67,11 +67,17 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     return tf::fail(TF_EUNSUPPORTED, "tf_inspect: rows*N exceeds int32 indexing");
   if (o.op == TF_OP_GEMM_SPMM) {
     if (o.K <= 0) return tf::fail(TF_EINVAL, "tf_inspect: GeMM-SpMM needs K > 0");
-    if (o.N % 32 != 0)
-      return tf::fail(TF_EUNSUPPORTED, "tf_inspect: the MFMA tile GEMM needs N %% 32 == 0 (N=%d)", o.N);
-    if (o.N > 256) return tf::fail(TF_EUNSUPPORTED, "tf_inspect: GeMM-SpMM supports N <= 256");
   } else {
     o.K = 0;
+  }
+  // The MFMA kernels take widths of 32, 64 .. 256 columns.  Any other N of a GeMM-SpMM is cut into equal
+  // column panels of such a width (the last one padded with zero columns of C); the executor runs the
+  // schedule once per panel.
+  const int user_N = o.N;
+  int n_panels = 1;
+  if (o.op == TF_OP_GEMM_SPMM && (o.N % 32 != 0 || o.N > 256)) {
+    n_panels = (o.N + 255) / 256;
+    o.N = ((o.N + n_panels - 1) / n_panels + 31) / 32 * 32;
   }
   // The MFMA kernels walk k in steps of 8: a K that is not a multiple of 8 is rounded up here and
   // the executor pads B's columns and C's rows with zeros into its workspace on every call.
@@ -153,6 +159,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     S->pattern_hash = tf_pattern_hash(L, Ap, Ai);
     S->gemm_kc = gemm_kc;
     S->user_K = user_K;
+    S->user_N = user_N;
+    S->n_panels = n_panels;
     S->gemm_regw = gemm_regw;
     S->gemm_stream = gemm_stream;
     S->ring_rows = ring_rows;
@@ -705,7 +713,7 @@ extern "C" void tf_schedule_free(tf_schedule *s) {
 extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info *info) {
   if (!s || !info) return tf::fail(TF_EINVAL, "tf_schedule_get_info: null argument");
   std::memset(info, 0, sizeof(*info));
-  info->op = s->opts.op; info->N = s->opts.N; info->K = s->user_K;
+  info->op = s->opts.op; info->N = s->user_N; info->K = s->user_K;
   info->rows = s->L; info->inter_rows = s->M;
   info->n_tiles = (int)s->tiles.size();
   info->n_fused_rows = (int)s->fused_ids.size();
@@ -734,6 +742,7 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   ws += (long long)s->long_chunks.size() * s->opts.N * 4;
   if (s->long_part) ws += ((long long)s->seg_ptr.size() - 1 + (long long)s->seg_groups.size()) * s->opts.N * 4 + (long long)s->seg_src.size() * 4;  // partial sums, regrouped values
   if (s->user_K != s->opts.K) ws += ((long long)s->M + s->opts.N) * s->opts.K * 4;  // padded copies of B and C
+  if (s->user_N != s->opts.N) ws += ((long long)s->L + s->opts.K) * s->opts.N * 4;  // one column panel of D and of C
   ws += (long long)s->rem_ptr.size() * 4 + (long long)s->rem_col.size() * 12;       // remainder rows in list order
   info->workspace_bytes = ws;
   return TF_OK;

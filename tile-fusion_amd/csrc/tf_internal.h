@@ -62,6 +62,8 @@ struct tf_schedule {
   std::vector<int> win;       // [2*n_tiles] first,last+1 row of C read by the tile's producer rows
   int slab_rows = 0;          // max producer rows of any tile
   int user_K = 0;             // K as given; opts.K is K rounded up to a multiple of 8 (what the kernels see)
+  int user_N = 0;             // N as given; GeMM-SpMM with a width the MFMA kernels do not take (N % 32, N > 256) runs
+  int n_panels = 1;           // as n_panels column panels of opts.N columns each, the last one zero-padded
   int gemm_kc = 0;            // rows of C staged in LDS per step (GeMM-SpMM)
   bool gemm_regw = false;     // GeMM-SpMM tiles keep C in registers (no staging; slab rows padded)
   int slab_ld = 0;            // floats between two slab rows of the general / GeMM-SpMM tile kernels

@@ -755,6 +755,19 @@ __global__ void pad_kernel(const float *__restrict__ src, int src_rows, int ld_s
   }
 }
 
+// dst[r, dst_col0 + c] (+)= src[r, src_col0 + c] for r < rows, c < cols; zero where src has no such row or column
+// (rows >= src_rows, c >= src_cols).  Column panels of C and D when N is not a width the MFMA kernels take.
+__global__ void copy_cols_kernel(const float *__restrict__ src, int src_rows, int ld_src, int src_col0, int src_cols,
+                                 float *__restrict__ dst, int rows, int ld_dst, int dst_col0, int cols, int accumulate) {
+  const size_t n = (size_t)rows * cols;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const int r = (int)(i / cols), c = (int)(i % cols);
+    const float v = (r < src_rows && c < src_cols) ? src[(size_t)r * ld_src + src_col0 + c] : 0.f;
+    float *p = dst + (size_t)r * ld_dst + dst_col0 + c;
+    *p = accumulate ? *p + v : v;
+  }
+}
+
 // p = max(p, 0), four values per thread (n is a multiple of 4: the kernels' N is).
 // Rows of zeros: Y[rows[q], :] = 0 (second-op rows without entries), V floats per thread.
 template <int V>
@@ -2192,6 +2205,16 @@ hipError_t launch_gemm(const float *X, const float *W, float *Y, const int *rows
   TF_DISPATCH_NB(NB, CALL);
 #undef CALL
   return err != hipSuccess ? err : hipGetLastError();
+}
+
+hipError_t launch_copy_cols(const float *src, int src_rows, int ld_src, int src_col0, int src_cols, float *dst, int rows,
+                            int ld_dst, int dst_col0, int cols, int accumulate, hipStream_t st) {
+  const size_t n = (size_t)rows * cols;
+  if (n == 0) return hipSuccess;
+  const int blocks = (int)std::min<size_t>((n + 255) / 256, 65536);
+  hipLaunchKernelGGL(copy_cols_kernel, dim3(blocks), dim3(256), 0, st, src, src_rows, ld_src, src_col0, src_cols, dst, rows,
+                     ld_dst, dst_col0, cols, accumulate);
+  return hipGetLastError();
 }
 
 hipError_t launch_pad(const float *src, int src_rows, int ld_src, float *dst, int rows, int ld_dst, hipStream_t st) {
