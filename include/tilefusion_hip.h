@@ -374,7 +374,8 @@ tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const tf_dense *
  * Y = A * X   (swiftware::sparse::spmmCsrParallel<float>, fusion/src/SpMM_SpMM.cpp:37-55) */
 tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, unsigned flags, void *stream);
 /* Y = X * W   (the cblas_sgemm call at fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:1144).
- * Needs K % 8 == 0, N % 32 == 0 and N <= 256 (TF_EUNSUPPORTED otherwise): it has no workspace to pad into. */
+ * K % 8 == 0, N % 32 == 0 and N <= 256 go straight to the MFMA kernel; any other shape is padded / cut into column
+ * panels in buffers allocated and freed inside the call (which then waits for the stream). */
 tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, void *stream);
 
 /* D = A * (B * C), A and B sparse, for callers that cannot allocate device memory (code under HIP

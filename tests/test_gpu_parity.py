@@ -532,6 +532,12 @@ def test_unfused_building_blocks(gpu, tf, orc):
     Z = tf.DenseMatrix(2000, 64)
     tf.gemm(tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W), Z)
     assert orc.rel_err(Z.to_numpy(), X.astype(np.float64) @ W.astype(np.float64)) <= 1e-6
+    # shapes the MFMA kernel does not take (the reference's sgemm takes any): padded / cut into panels inside the call
+    for (M, K, N) in ((700, 20, 50), (33, 7, 1), (1500, 64, 300), (257, 100, 600)):
+        Xq, Wq = tf.workloads.uniform((M, K), 73 + N), tf.workloads.uniform((K, N), 74 + N)
+        Zq = tf.DenseMatrix(M, N); Zq.fill(float("nan"))
+        tf.gemm(tf.DenseMatrix.from_numpy(Xq), tf.DenseMatrix.from_numpy(Wq), Zq)
+        assert orc.rel_err(Zq.to_numpy(), Xq.astype(np.float64) @ Wq.astype(np.float64)) <= 1e-6, (M, K, N)
 
 
 @pytest.mark.parametrize("N", [32, 64, 128, 256, 20, 320])

@@ -876,10 +876,33 @@ extern "C" tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, 
   if (!X || !W || !Y) return fail(TF_EINVAL, "tf_gemm: null argument");
   if (X->N != W->M || Y->M != X->M || Y->N != W->N)
     return fail(TF_EINVAL, "tf_gemm: shapes X %d x %d, W %d x %d, Y %d x %d", X->M, X->N, W->M, W->N, Y->M, Y->N);
-  const int K = X->N, N = W->N;
-  if (K % 8 != 0 || N % 32 != 0 || N > 256)
-    return fail(TF_EUNSUPPORTED, "tf_gemm: needs K %% 8 == 0, N %% 32 == 0, N <= 256 (K=%d N=%d)", K, N);
-  TF_HIP(tf::launch_gemm(X->d, W->d, Y->d, nullptr, X->M, K, N, tf::default_compute_units(),
-                         static_cast<hipStream_t>(stream)));
-  return TF_OK;
+  const int K = X->N, N = W->N, M = X->M;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (K <= 0 || N <= 0 || M <= 0) return fail(TF_EINVAL, "tf_gemm: empty operand");
+  if (K % 8 == 0 && N % 32 == 0 && N <= 256) {
+    TF_HIP(tf::launch_gemm(X->d, W->d, Y->d, nullptr, M, K, N, tf::default_compute_units(), st));
+    return TF_OK;
+  }
+  // Shapes the MFMA kernel does not take: K padded to 8 with zeros and N cut into equal panels of 32 .. 256 columns
+  // in buffers that live for this call (allocated and freed here; freeing waits for the stream's work).
+  const int Kp = (K + 7) / 8 * 8, n_panels = (N + 255) / 256, Wd = ((N + n_panels - 1) / n_panels + 31) / 32 * 32;
+  float *Xp = nullptr, *Wp = nullptr, *Yp = nullptr;
+  tf_status rc = TF_OK;
+  auto hip_ok = [&](hipError_t e, const char *what) {
+    if (e != hipSuccess && rc == TF_OK) rc = tf::hip_fail(e, what);
+    return e == hipSuccess;
+  };
+  if (Kp != K && hip_ok(hipMalloc(reinterpret_cast<void **>(&Xp), (size_t)M * Kp * sizeof(float)), "hipMalloc(tf_gemm: padded X)"))
+    hip_ok(tf::launch_pad(X->d, M, K, Xp, M, Kp, st), "pad_kernel");
+  if (rc == TF_OK) hip_ok(hipMalloc(reinterpret_cast<void **>(&Wp), (size_t)Kp * Wd * sizeof(float)), "hipMalloc(tf_gemm: panel of W)");
+  if (rc == TF_OK) hip_ok(hipMalloc(reinterpret_cast<void **>(&Yp), (size_t)M * Wd * sizeof(float)), "hipMalloc(tf_gemm: panel of Y)");
+  for (int q = 0; q < n_panels && rc == TF_OK; ++q) {
+    const int c0 = q * Wd, w = std::min(Wd, N - c0);
+    if (hip_ok(tf::launch_copy_cols(W->d, K, N, c0, w, Wp, Kp, Wd, 0, Wd, 0, st), "copy_cols_kernel") &&
+        hip_ok(tf::launch_gemm(Xp ? Xp : X->d, Wp, Yp, nullptr, M, Kp, Wd, tf::default_compute_units(), st), "gemm_rows_kernel"))
+      hip_ok(tf::launch_copy_cols(Yp, M, Wd, 0, w, Y->d, M, N, c0, w, 0, st), "copy_cols_kernel");
+  }
+  if (rc == TF_OK) hip_ok(hipStreamSynchronize(st), "hipStreamSynchronize");
+  (void)hipFree(Xp); (void)hipFree(Wp); (void)hipFree(Yp);
+  return rc;
 }
