@@ -63,8 +63,6 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   if (o.op != TF_OP_SPMM_SPMM && o.op != TF_OP_GEMM_SPMM)
     return tf::fail(TF_EINVAL, "tf_inspect: unknown op %d", o.op);
   if (o.N <= 0) return tf::fail(TF_EINVAL, "tf_inspect: N must be positive");
-  if ((long long)std::max(L, M) * o.N > INT_MAX)
-    return tf::fail(TF_EUNSUPPORTED, "tf_inspect: rows*N exceeds int32 indexing");
   if (o.op == TF_OP_GEMM_SPMM) {
     if (o.K <= 0) return tf::fail(TF_EINVAL, "tf_inspect: GeMM-SpMM needs K > 0");
   } else {
@@ -79,6 +77,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     n_panels = (o.N + 255) / 256;
     o.N = ((o.N + n_panels - 1) / n_panels + 31) / 32 * 32;
   }
+  if ((long long)std::max(L, M) * o.N > INT_MAX)  // (the width the kernels see: a panel's, when N is cut into panels)
+    return tf::fail(TF_EUNSUPPORTED, "tf_inspect: rows*N exceeds int32 indexing");
   // The MFMA kernels walk k in steps of 8: a K that is not a multiple of 8 is rounded up here and
   // the executor pads B's columns and C's rows with zeros into its workspace on every call.
   const int user_K = o.K;
