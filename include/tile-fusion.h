@@ -163,6 +163,7 @@ class FusedSchedule {
   void refresh() {
     if (!st_ || !st_->last_used) return;
     tf_schedule_view v;
+    v.struct_size = sizeof(v);
     detail::check(tf_schedule_get_view(st_->last_used, &v), "FusedSchedule");
     n1_ = v.n1; ptr1_ = v.ptr1; ptr2_ = v.ptr2; ker_begin_ = v.ker_begin; id_ = v.id; type_ = v.type;
   }
@@ -188,6 +189,7 @@ class FusedSchedule {
   }
   tf_schedule_info info(int op, int N, int K, bool inner_is_outer = false) {
     tf_schedule_info i;
+    i.struct_size = sizeof(i);
     detail::check(tf_schedule_get_info(lookup(op, N, K, inner_is_outer, false), &i), "FusedSchedule::info");
     refresh();
     return i;

@@ -42,7 +42,14 @@ const char *tf_version(void);
 
 /* ---- device ----------------------------------------------------------------- */
 
+/* Structs the library fills in for the caller ("out-structs": tf_device_info, tf_schedule_info,
+ * tf_schedule_view, tf_profile) start with struct_size, which the CALLER sets to sizeof(the struct)
+ * as it was compiled before the call.  Fields are only ever appended, so the library writes the
+ * first min(struct_size, its own sizeof) bytes and nothing behind them: a caller built against an
+ * older header keeps working and its stack is not overrun.  TF_EINVAL when struct_size is smaller
+ * than the struct's first version (stated at each struct) -- which includes a forgotten 0. */
 typedef struct {
+  size_t struct_size;      /* set by the caller; first version: through xcd_round_robin */
   int device;              /* HIP device ordinal in use                           */
   int compute_units;       /* 256 on MI355X                                       */
   int xcds;                /* accelerator complex dies sharing an L2 each (8)     */
@@ -255,6 +262,7 @@ tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai, const tf_inspec
 void tf_schedule_free(tf_schedule *s);
 
 typedef struct {
+  size_t struct_size;    /* set by the caller; first version: through march_slots   */
   int op, N, K;
   int rows;              /* L: rows of A / D                                        */
   int inter_rows;        /* M: rows of the intermediate                             */
@@ -293,6 +301,7 @@ tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info *info);
  * tile_range[4*t + {0,1,2,3}] = producer_begin, producer_end, own_begin, own_end.
  * Pointers are views into the schedule, valid until tf_schedule_free. */
 typedef struct {
+  size_t struct_size;   /* set by the caller; first version: through n_step_ptr */
   int n1, n_part, n_id, n_tiles;
   const int *ptr1, *ptr2, *ker_begin, *id, *type;
   const int *tile_range;
@@ -375,7 +384,10 @@ tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const tf_dense *
 tf_status tf_spmm(const tf_csr *A, const tf_dense *X, tf_dense *Y, unsigned flags, void *stream);
 /* Y = X * W   (the cblas_sgemm call at fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:1144).
  * K % 8 == 0, N % 32 == 0 and N <= 256 go straight to the MFMA kernel; any other shape is padded / cut into column
- * panels in buffers allocated and freed inside the call (which then waits for the stream). */
+ * panels in a workspace the library keeps per device.  The workspace only grows: a call whose buffers fit is
+ * asynchronous on `stream` like every other; the first call with a larger shape frees and allocates (which waits for
+ * the device, and is refused with TF_EUNSUPPORTED while `stream` is being captured).  Calls with such shapes on one
+ * device share that workspace: keep them on one stream, or order them with events. */
 tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, void *stream);
 
 /* D = A * (B * C), A and B sparse, for callers that cannot allocate device memory (code under HIP
@@ -397,6 +409,7 @@ size_t tf_noalloc_scratch_bytes(void);
  * duration in ms (kernels that ran side by side on two streams each report their own). */
 #define TF_PROFILE_MAX 16
 typedef struct {
+  size_t struct_size;   /* set by the caller; first version: through ms */
   int n;
   const char *name[TF_PROFILE_MAX];
   float ms[TF_PROFILE_MAX];

@@ -33,8 +33,8 @@ static int run(const char *name, int M, const std::vector<int> &p, const std::ve
   tf_status rc = tf_inspect(M, M, p.data(), i.data(), &o, &s);
   if (rc) { printf("%s: inspect %d %s\n", name, rc, tf::g_err); return o.op < 0 ? 0 : 1; }
   rc = tf_schedule_validate_inner(s, M, M, p.data(), i.data(), o.inner_Ap, o.inner_Ai, o.inner_cols);
-  tf_schedule_info info; tf_schedule_get_info(s, &info);
-  tf_schedule_view v; tf_schedule_get_view(s, &v);
+  tf_schedule_info info; info.struct_size = sizeof(info); tf_schedule_get_info(s, &info);
+  tf_schedule_view v; v.struct_size = sizeof(v); tf_schedule_get_view(s, &v);
   printf("%s: validate %d tiles %d fused %d long %d hot %d wide %d streamed %d ws %lld %s\n", name, rc, info.n_tiles, info.n_fused_rows, info.n_long_rows, info.long_row_hot_cols, info.wide_strips, info.streamed, info.workspace_bytes, rc ? tf::g_err : "");
   tf_schedule_free(s);
   return rc != 0;

@@ -145,6 +145,49 @@ def test_launch_times_and_second_stream(gpu, tf, orc):
         assert np.array_equal(D2.to_numpy(), a)
 
 
+def test_second_stream_on_a_first_call_and_on_wrapped_matrices(gpu, tf, orc):
+    """TF_SECOND_STREAM when the regrouped values of the long rows have to be built in the same call: on the
+    first call with a fresh schedule, and on every call with a matrix wrapped around device arrays (whose
+    values the library takes as new each time).  The cold segments run on the caller's stream and read values
+    the same call regroups, so that copy has to come before the fork: results must equal the one-stream
+    call's bit for bit, also after the wrapped matrix' values changed in place."""
+    say("second stream: first call, wrapped matrix")
+    cfg = tf.workloads.make_config(4, 2.0 ** -5)
+    A, B, W = cfg["A"], cfg["B"], cfg["C"]
+    M = A.shape[0]
+    Bd, Wd = tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S0 = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1)
+    D0 = tf.DenseMatrix(M, 128)
+    tf.gemm_spmm(Ah, Bd, Wd, D0, S0)
+    want = D0.to_numpy()
+    # a fresh schedule whose first call already forks
+    S1 = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1)
+    D1 = tf.DenseMatrix(M, 128); D1.fill(float("nan"))
+    tf.gemm_spmm(Ah, Bd, Wd, D1, S1, second_stream=True)
+    assert np.array_equal(D1.to_numpy(), want)
+    # the same matrix wrapped around device arrays: values regrouped on every call
+    as_f32 = lambda a: np.ascontiguousarray(a, dtype=np.int32).view(np.float32).reshape(1, -1)  # noqa: E731
+    dp, di = tf.DenseMatrix.from_numpy(as_f32(A.indptr)), tf.DenseMatrix.from_numpy(as_f32(A.indices))
+    dx = tf.DenseMatrix.from_numpy(A.data.reshape(1, -1))
+    Aw = tf.CsrMatrix.wrap_device(Ah, dp.device_ptr(), di.device_ptr(), dx.device_ptr(), tf.pattern_hash(A))
+    S2 = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1)
+    for second in (True, False, True):
+        D2 = tf.DenseMatrix(M, 128); D2.fill(float("nan"))
+        tf.gemm_spmm(Aw, Bd, Wd, D2, S2, second_stream=second)
+        assert np.array_equal(D2.to_numpy(), want), second
+    # new values in the same device array: the next call must use them, on both streams
+    dx.copy_from(tf.DenseMatrix.from_numpy((A.data * np.float32(0.5)).reshape(1, -1)))
+    tf.device_synchronize()
+    A2 = A.copy(); A2.data = A.data * np.float32(0.5)
+    D3 = tf.DenseMatrix(M, 128); D3.fill(float("nan"))
+    tf.gemm_spmm(Aw, Bd, Wd, D3, S2, second_stream=True)
+    want2 = tf.DenseMatrix(M, 128)
+    tf.gemm_spmm(tf.CsrMatrix.from_scipy(A2), Bd, Wd, want2, S0)
+    assert np.array_equal(D3.to_numpy(), want2.to_numpy())
+    del Aw
+
+
 def test_two_gcn_layers_in_one_call(gpu, tf, orc):
     """tf_gcn_two_layers against the oracle's executor composed twice (ReLU between, on the host), with
     and without the activation, with the hidden layer handed back, and with one schedule for both
@@ -176,6 +219,35 @@ def test_two_gcn_layers_in_one_call(gpu, tf, orc):
     with pytest.raises(tf.TileFusionError) as e:               # schedules in the wrong order
         tf.gcn_two_layers(Ah, tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W1), tf.DenseMatrix.from_numpy(W2), D, s2, s1)
     assert e.value.status == -4
+    # ... which must leave no undersized hidden-layer buffer behind: the right order still works afterwards
+    D3 = tf.DenseMatrix(M, N); D3.fill(float("nan"))
+    tf.gcn_two_layers(Ah, tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W1), tf.DenseMatrix.from_numpy(W2), D3, s1, s2, relu=False)
+    assert np.array_equal(D3.to_numpy(), D2.to_numpy())
+
+
+def test_two_gcn_layers_hidden_width_that_needs_panels(gpu, tf, orc):
+    """A hidden width the MFMA kernels do not take (30: one padded panel) on an odd row count, so that the hidden
+    layer's element count is no multiple of four: the activation kernel has a tail, the layers run in panels."""
+    say("tf_gcn_two_layers, H = 30")
+    A = tf.workloads.erdos_renyi_gcn(3001, 8.0, seed=31)
+    M = A.shape[0]
+    assert (M * 30) % 4 != 0
+    Ah = tf.CsrMatrix.from_scipy(A)
+    K, H, N = 24, 30, 10
+    X = tf.workloads.uniform((M, K), 104)
+    W1, W2 = tf.workloads.glorot(K, H, 105), tf.workloads.glorot(H, N, 106)
+    s1 = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=H, K=K)
+    s2 = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=N, K=H)
+    sch = orc.unfused_schedule(M)
+    h, _ = orc.gemm_spmm(A, X, W1, sch, nthreads=8)
+    h = np.maximum(h, 0.0)
+    want, _ = orc.gemm_spmm(A, h, W2, sch, nthreads=8)
+    D = tf.DenseMatrix(M, N); D.fill(float("nan"))
+    hid = tf.DenseMatrix(M, H); hid.fill(float("nan"))
+    tf.gcn_two_layers(Ah, tf.DenseMatrix.from_numpy(X), tf.DenseMatrix.from_numpy(W1), tf.DenseMatrix.from_numpy(W2), D, s1, s2,
+                      relu=True, hidden=hid)
+    got_h = hid.to_numpy()
+    assert (got_h >= 0).all() and orc.rel_err(got_h, h) <= TOL and orc.rel_err(D.to_numpy(), want) <= TOL
 
 
 def test_remainder_rows_in_list_order(gpu, tf, orc):

@@ -353,6 +353,56 @@ def test_opts_struct_size_is_honoured(tf):
     assert b"struct_size" in b.lib().tf_last_error_string()
 
 
+def test_out_struct_size_is_honoured(tf):
+    """The structs the library fills in carry the caller's size too: a caller compiled against a
+    struct one field shorter gets exactly its bytes, a canary right behind them stays intact, and
+    a size below the struct's first version (a forgotten 0) is refused."""
+    import ctypes as C
+    from importlib import import_module
+    b = import_module("tile-fusion_amd.binding")
+    A = tf.workloads.banded_random(2000, 32, 16, seed=3)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, op=tf.OP_GEMM_SPMM, N=128, K=128)
+    lib = b.lib()
+
+    def call_short(struct, fn, handle, cut_field):
+        """Calls fn(handle, buf) with buf = the struct cut right after `cut_field`, 0xAB behind it."""
+        full = struct(C.sizeof(struct))
+        assert fn(handle, C.byref(full)) == 0
+        fld = getattr(struct, cut_field)
+        short = fld.offset + fld.size
+        assert short < C.sizeof(struct)
+        raw = (C.c_ubyte * (C.sizeof(struct) + 64))(*([0xAB] * (C.sizeof(struct) + 64)))
+        C.cast(raw, C.POINTER(C.c_size_t))[0] = short
+        assert fn(handle, C.cast(raw, C.POINTER(struct))) == 0, lib.tf_last_error_string()
+        assert bytes(raw[C.sizeof(C.c_size_t):short]) == bytes(full)[C.sizeof(C.c_size_t):short]
+        assert all(x == 0xAB for x in raw[short:]), "the library wrote behind the caller's struct"
+        assert C.cast(raw, C.POINTER(C.c_size_t))[0] == short
+        zero = struct(0)
+        assert fn(handle, C.byref(zero)) == -1 and b"struct_size" in lib.tf_last_error_string()
+
+    # the last fields of today's structs are cut off as a later header's would be
+    last_info = b.ScheduleInfo._fields_[-1][0]
+    prev_info = b.ScheduleInfo._fields_[-2][0]
+    # (a struct cut before the end of its first version is refused, so cut only what came later)
+    first_version_end = "march_slots"
+    if last_info != first_version_end:
+        call_short(b.ScheduleInfo, lib.tf_schedule_get_info, S.h, prev_info if prev_info != first_version_end else first_version_end)
+    too_short = b.ScheduleInfo(b.ScheduleInfo.march_slots.offset)  # ends before march_slots
+    assert lib.tf_schedule_get_info(S.h, C.byref(too_short)) == -1
+    # a struct LONGER than the library's (a newer caller): only the library's bytes are written
+    class Longer(C.Structure):
+        _fields_ = b.ScheduleView._fields_ + [("future", C.c_longlong * 8)]   # (8-byte fields: behind the struct's tail padding)
+    v = Longer(C.sizeof(Longer))
+    for q in range(8):
+        v.future[q] = 0x5A5A5A5A5A5A
+    assert lib.tf_schedule_get_view(S.h, C.cast(C.byref(v), C.POINTER(b.ScheduleView))) == 0
+    assert v.n1 == 2 and all(v.future[q] == 0x5A5A5A5A5A5A for q in range(8)) and v.struct_size == C.sizeof(Longer)
+    for struct, fn in ((b.ScheduleView, lib.tf_schedule_get_view), (b.Profile, lib.tf_schedule_get_profile)):
+        zero = struct(0)
+        assert fn(S.h, C.byref(zero)) == -1 and b"struct_size" in lib.tf_last_error_string()
+
+
 def test_pattern_hash(tf):
     A = tf.workloads.banded_random(1000, 32, 16, seed=3)
     h = tf.pattern_hash(A)

@@ -56,6 +56,35 @@ def test_noalloc_matches_the_scheduled_executor(gpu, tf, orc):
     assert orc.rel_err(D.to_numpy(), D0.astype(np.float64) + (A.astype(np.float64) @ T.astype(np.float64))) <= 1e-5
 
 
+def test_noalloc_call_allocates_no_device_memory(gpu, tf):
+    """What the entry point is for: once the library is initialised on the device (tf_device_init, or one earlier
+    call, looks up the scratch array's address) a call leaves the device's free memory exactly as it was -- while
+    the probe does see the workspace a scheduled executor allocates on its first call."""
+    import torch
+    say("tf_spmm_spmm_noalloc: free device memory unchanged")
+    tf.device_init(0)
+    M, N = 30000, 64
+    A = tf.workloads.erdos_renyi_gcn(M, 8.0, seed=97)         # nothing fuses: a schedule needs the intermediate in HBM
+    Ah = tf.CsrMatrix.from_scipy(A).to_device()
+    Cm, D = tf.DenseMatrix.from_numpy(tf.workloads.uniform((M, N), 98)), tf.DenseMatrix(M, N)
+    st = tf.Stream()
+    tf.spmm_spmm_noalloc(Ah, Ah, Cm, D, stream=st)           # warm-up: kernels loaded, address looked up
+    st.synchronize()
+    torch.cuda.mem_get_info()                                # (the probe's own first call initialises torch's context)
+    tf.device_synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        tf.spmm_spmm_noalloc(Ah, Ah, Cm, D, stream=st)
+    st.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    # positive control: a scheduled executor's first call allocates its intermediate (30000 x 64 floats = 7.7 MB)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N)
+    assert S.info()["workspace_bytes"] > 4 << 20
+    tf.spmm_spmm(Ah, Ah, Cm, D, S, stream=st)
+    st.synchronize()
+    assert torch.cuda.mem_get_info()[0] < free0
+
+
 def test_noalloc_rejects_an_intermediate_beyond_the_scratch(gpu, tf):
     M, N = 70000, 128          # 70,000 x 128 floats = 35.8 MB > 32 MiB
     A = tf.workloads.banded_random(M, 8, 4, seed=96)

@@ -29,7 +29,7 @@ class TileFusionError(RuntimeError):
 
 
 class DeviceInfo(C.Structure):
-    _fields_ = [("device", C.c_int), ("compute_units", C.c_int), ("xcds", C.c_int),
+    _fields_ = [("struct_size", C.c_size_t), ("device", C.c_int), ("compute_units", C.c_int), ("xcds", C.c_int),
                 ("lds_bytes_per_block", C.c_int), ("wavefront", C.c_int), ("clock_khz", C.c_int),
                 ("hbm_bytes", C.c_size_t), ("arch", C.c_char * 64), ("xcd_round_robin", C.c_int)]
 
@@ -44,7 +44,7 @@ class InspectOpts(C.Structure):
 
 
 class ScheduleInfo(C.Structure):
-    _fields_ = [("op", C.c_int), ("N", C.c_int), ("K", C.c_int), ("rows", C.c_int),
+    _fields_ = [("struct_size", C.c_size_t), ("op", C.c_int), ("N", C.c_int), ("K", C.c_int), ("rows", C.c_int),
                 ("inter_rows", C.c_int), ("n_tiles", C.c_int), ("n_fused_rows", C.c_int),
                 ("n_remainder_rows", C.c_int), ("n_long_rows", C.c_int), ("n_long_chunks", C.c_int),
                 ("n_producer_rows", C.c_int), ("n_writeback_rows", C.c_int),
@@ -55,7 +55,7 @@ class ScheduleInfo(C.Structure):
 
 
 class ScheduleView(C.Structure):
-    _fields_ = [("n1", C.c_int), ("n_part", C.c_int), ("n_id", C.c_int), ("n_tiles", C.c_int),
+    _fields_ = [("struct_size", C.c_size_t), ("n1", C.c_int), ("n_part", C.c_int), ("n_id", C.c_int), ("n_tiles", C.c_int),
                 ("ptr1", C.POINTER(C.c_int)), ("ptr2", C.POINTER(C.c_int)),
                 ("ker_begin", C.POINTER(C.c_int)), ("id", C.POINTER(C.c_int)),
                 ("type", C.POINTER(C.c_int)), ("tile_range", C.POINTER(C.c_int)),
@@ -67,7 +67,7 @@ PROFILE_MAX = 16
 
 
 class Profile(C.Structure):
-    _fields_ = [("n", C.c_int), ("name", C.c_char_p * PROFILE_MAX), ("ms", C.c_float * PROFILE_MAX)]
+    _fields_ = [("struct_size", C.c_size_t), ("n", C.c_int), ("name", C.c_char_p * PROFILE_MAX), ("ms", C.c_float * PROFILE_MAX)]
 
 
 _PI = C.POINTER(C.c_int)
@@ -158,9 +158,9 @@ def _f32(a):
 
 
 def device_init(device=0):
-    info = DeviceInfo()
+    info = DeviceInfo(C.sizeof(DeviceInfo))
     _check(lib().tf_device_init(device, C.byref(info)))
-    return {f: (getattr(info, f).decode() if f == "arch" else getattr(info, f)) for f, _ in DeviceInfo._fields_}
+    return {f: (getattr(info, f).decode() if f == "arch" else getattr(info, f)) for f, _ in DeviceInfo._fields_ if f != "struct_size"}
 
 
 def device_synchronize():
@@ -230,6 +230,19 @@ class CsrMatrix:
             self.h = h
         return self
 
+    @classmethod
+    def wrap_device(cls, host, dAp, dAi, dAx, pattern_hash=0):
+        """A matrix whose arrays already live in device memory (tf_csr_wrap_device): `host` is the CsrMatrix
+        with the same arrays on the host (kept for its pattern), dAp/dAi/dAx are device addresses.  The
+        library neither copies nor owns them, and takes their values as new on every call."""
+        self = cls(host.M, host.N, host.Ap, host.Ai, host.Ax)
+        h = _VP()
+        _check(lib().tf_csr_wrap_device(self.M, self.N, self.nnz, _VP(dAp), _VP(dAi), _VP(dAx), C.byref(h)))
+        if pattern_hash:
+            _check(lib().tf_csr_set_pattern_hash(h, pattern_hash))
+        self.h = h
+        return self
+
     def __del__(self):
         if getattr(self, "h", None):
             lib().tf_csr_free(self.h)
@@ -293,12 +306,12 @@ class FusedSchedule:
         self._inner = inner
 
     def info(self):
-        s = ScheduleInfo()
+        s = ScheduleInfo(C.sizeof(ScheduleInfo))
         _check(lib().tf_schedule_get_info(self.h, C.byref(s)))
-        return {f: getattr(s, f) for f, _ in ScheduleInfo._fields_}
+        return {f: getattr(s, f) for f, _ in ScheduleInfo._fields_ if f != "struct_size"}
 
     def view(self):
-        v = ScheduleView()
+        v = ScheduleView(C.sizeof(ScheduleView))
         _check(lib().tf_schedule_get_view(self.h, C.byref(v)))
         P, nid, nt = v.n_part, v.n_id, v.n_tiles
 
@@ -323,7 +336,7 @@ class FusedSchedule:
 
     def profile(self):
         """[(launch name, ms)] of the last executor call with this schedule (profiling switched on)."""
-        p = Profile()
+        p = Profile(C.sizeof(Profile))
         _check(lib().tf_schedule_get_profile(self.h, C.byref(p)))
         return [(p.name[i].decode(), float(p.ms[i])) for i in range(p.n)]
 

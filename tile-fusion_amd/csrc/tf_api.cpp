@@ -57,6 +57,7 @@ struct DeviceSchedule {
   float *rem_val = nullptr;
   unsigned long long rem_val_serial = 0;
   float *hidden = nullptr;   // tf_gcn_two_layers: the first layer's output, L x K of this (second-layer) schedule
+  size_t hidden_floats = 0;
   float *Bpad = nullptr;     // M x K' and K' x N copies of B and C, zero-padded, when K is not a multiple of 8
   float *Cpad = nullptr;
   float *Cpanel = nullptr;   // K' x N and L x N: one column panel of C (zero-padded) and of D, when the caller's width is
@@ -300,12 +301,18 @@ static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 // reference's reordered adjacency (createReorderedAdj, GCN_Single_Layer_SP_Demo_Utils.h:618-653)
 // is to its executors -- are built on the first call with an uploaded matrix and kept; a wrapped
 // matrix can change between calls, so its values are regrouped every time.
-static tf_status run_hot_segments(const tf_csr *A, tf_schedule *s, hipStream_t st) {
+// ensure_segment_values fills the values of ALL segments, hot and cold, so it must run on a stream
+// that both the hot and the cold launch are ordered after: the caller's, before a second stream forks.
+static tf_status ensure_segment_values(const tf_csr *A, tf_schedule *s, hipStream_t st) {
   DeviceSchedule *d = s->dev;
   const bool have_values = A->serial != 0 && d->seg_val_serial == A->serial;
   if (!have_values)
     TF_PHASE(s, "scatter_values_kernel", st, launch_scatter_values(d->ent_src, d->ent_pos, A->x, d->seg_val, (int)s->seg_src.size(), st));
   d->seg_val_serial = A->serial;
+  return TF_OK;
+}
+static tf_status run_hot_segments(tf_schedule *s, hipStream_t st) {
+  DeviceSchedule *d = s->dev;
   TF_PHASE(s, "spmm_rows_kernel (hot long-row segments)", st,
            launch_spmm_rows(nullptr, 8 * s->seg_per_xcd, d->seg_ptr, d->seg_col, d->seg_val, d->inter, d->partial, s->opts.N, 0, -1, 1, st, /*compact=*/0, /*coalesced_pairs=*/1));
   return TF_OK;
@@ -337,8 +344,10 @@ static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int
   }
   if (s->long_part) {
     const int n_hot = 8 * s->seg_per_xcd, n_seg = (int)s->seg_ptr.size() - 1;
-    if (!hot_on_side)
-      if (tf_status rc = run_hot_segments(A, s, st)) return rc;
+    if (!hot_on_side) {
+      if (tf_status rc = ensure_segment_values(A, s, st)) return rc;
+      if (tf_status rc = run_hot_segments(s, st)) return rc;
+    }
     TF_PHASE(s, "spmm_rows_kernel (cold long-row segments)", st,
              launch_spmm_rows(nullptr, n_seg - n_hot, d->seg_ptr + n_hot, d->seg_col, d->seg_val, d->inter,
                               d->partial + (size_t)n_hot * N, N, 0, 0, 1, st));
@@ -389,6 +398,13 @@ tf_status scratch_of_current_device(float **out) {
   return TF_OK;
 }
 
+// tf_gemm's buffers for shapes off the MFMA kernel's fast path: padded X, a panel of W, a panel of Y.
+struct GemmWorkspace {
+  float *buf[3] = {nullptr, nullptr, nullptr};
+  size_t floats[3] = {0, 0, 0};
+};
+GemmWorkspace g_gemm_ws[kMaxDevices];
+
 }  // namespace
 
 
@@ -411,9 +427,15 @@ extern "C" tf_status tf_device_init(int device, tf_device_info *info) {
     if (tf_status rc = scratch_of_current_device(&unused)) return rc;
   }
   if (info) {
+    if (info->struct_size < TF_SIZE_THROUGH(tf_device_info, xcd_round_robin))  // before any work is done for it
+      return fail(TF_EINVAL, "tf_device_init: info->struct_size is %zu, the struct's first version has %zu bytes (set it to sizeof(tf_device_info))",
+                  info->struct_size, TF_SIZE_THROUGH(tf_device_info, xcd_round_robin));
     hipDeviceProp_t p;
     TF_HIP(hipGetDeviceProperties(&p, device));
-    std::memset(info, 0, sizeof(*info));
+    tf_device_info full;
+    std::memset(&full, 0, sizeof(full));
+    tf_device_info *const caller = info;
+    info = &full;
     info->device = device;
     info->compute_units = p.multiProcessorCount;
     info->xcds = 8;
@@ -441,6 +463,7 @@ extern "C" tf_status tf_device_init(int device, tf_device_info *info) {
       (void)hipFree(probe);
     }
     (void)hipGetLastError();
+    return tf::emit_out("tf_device_init", caller, full, TF_SIZE_THROUGH(tf_device_info, xcd_round_robin));
   }
   return TF_OK;
 }
@@ -668,7 +691,8 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
       return fail(TF_ESCHEDULE, "tf_spmm_spmm: B has the shape and entry count of the inner pattern the schedule was built on, but another sparsity pattern");
     // The windowed kernel walks one staged CSR chunk for both products: B must be A.
     const bool same = (B == A) || (B->p == A->p && B->i == A->i && B->x == A->x);
-    if (s->win_wide && A->nnz >= 4) {  // reads B's entries for the first product and A's for the second, in place
+    // (the kernel fetches entries four at a time and clamps the last fetch to nnz - 4: both arrays need four)
+    if (s->win_wide && A->nnz >= 4 && B->nnz >= 4) {  // reads B's entries for the first product and A's for the second, in place
       TF_PHASE(s, "fused_spmm_spmm_window64_kernel", st,
                tf::launch_fused_spmm_spmm_window64(d->tiles, d->win, n_launch, B->p, B->i, B->x,
                                                    B->nnz, C->d, A->p, A->i, A->x, A->nnz, D->d, s->opts.N,
@@ -727,9 +751,12 @@ static tf_status gemm_spmm_pass(const tf_csr *A, const float *Bd, const float *C
     if (overlap) {
       TF_PHASE(s, "gemm_rows_kernel (hot rows)", st,
                tf::launch_gemm(Bd, Cd, d->inter, d->plain_rows, s->plain_hot, s->opts.K, s->opts.N, s->opts.compute_units, st));
+      // the regrouped values (of the hot and of the cold segments) before the fork: the cold segments run on
+      // this stream and are not ordered after anything the side stream does until the join
+      if (tf_status rc2 = tf::ensure_segment_values(A, s, st)) return rc2;
       TF_HIP(hipEventRecord(d->fork, st));
       TF_HIP(hipStreamWaitEvent(d->side, d->fork, 0));
-      if (tf_status rc2 = tf::run_hot_segments(A, s, d->side)) return rc2;
+      if (tf_status rc2 = tf::run_hot_segments(s, d->side)) return rc2;
       TF_HIP(hipEventRecord(d->join, d->side));
       if (n_plain > s->plain_hot)
         TF_PHASE(s, "gemm_rows_kernel (other rows)", st,
@@ -795,16 +822,34 @@ extern "C" tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const
   if (W2->M != H) return fail(TF_EINVAL, "tf_gcn_two_layers: W1 has %d columns, W2 has %d rows", H, W2->M);
   if (hidden && (hidden->M != A->M || hidden->N != H))
     return fail(TF_EINVAL, "tf_gcn_two_layers: hidden is %d x %d, expected %d x %d", hidden->M, hidden->N, A->M, H);
+  // every check of shape and schedule before anything is allocated or run
+  if (s1->opts.op != TF_OP_GEMM_SPMM || s2->opts.op != TF_OP_GEMM_SPMM)
+    return fail(TF_ESCHEDULE, "tf_gcn_two_layers: both schedules must be built for TF_OP_GEMM_SPMM");
+  if (s1->L != A->M || s1->M != A->N || s2->L != A->M || s2->M != A->N)
+    return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the schedules were built for %d x %d and %d x %d patterns, A is %d x %d", s1->L, s1->M, s2->L, s2->M, A->M, A->N);
+  if (s1->user_N != H) return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the first schedule was built for N = %d, W1 has %d columns", s1->user_N, H);
+  if (s2->user_K != H) return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule was built for K = %d, the hidden layer has %d columns", s2->user_K, H);
+  if (X->M != A->N || X->N != s1->user_K || W1->M != s1->user_K)
+    return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the first schedule was built for K = %d, X is %d x %d and W1 has %d rows", s1->user_K, X->M, X->N, W1->M);
+  if (W2->N != s2->user_N || D->N != s2->user_N || D->M != A->M)
+    return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule was built for N = %d, W2 has %d columns and D is %d x %d", s2->user_N, W2->N, D->M, D->N);
   tf_dense h;
   h.M = A->M; h.N = H; h.owns = false;
   if (hidden) {
     h.d = hidden->d;
   } else {
     if (tf_status rc = tf::ensure_device(s2)) return rc;
-    if (!s2->dev->hidden) TF_HIP(hipMalloc(reinterpret_cast<void **>(&s2->dev->hidden), (size_t)A->M * H * sizeof(float)));
+    static std::mutex mu;  // (two threads may share a schedule object up to here; executor calls themselves are one at a time)
+    std::lock_guard<std::mutex> lock(mu);
+    const size_t need = (size_t)s2->L * s2->user_K;  // the hidden layer of THIS schedule: L x K
+    if (!s2->dev->hidden) {
+      TF_HIP(hipMalloc(reinterpret_cast<void **>(&s2->dev->hidden), need * sizeof(float)));
+      s2->dev->hidden_floats = need;
+    }
+    if (s2->dev->hidden_floats != need)
+      return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule's hidden-layer buffer holds %zu floats, %zu are needed", s2->dev->hidden_floats, need);
     h.d = s2->dev->hidden;
   }
-  if (s2->user_K != H) return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule was built for K = %d, the hidden layer has %d columns", s2->user_K, H);
   // first layer (its schedule is checked against X and W1 there), activation, second layer
   if (tf_status rc = tf_gemm_spmm(A, X, W1, &h, s1, flags & TF_SECOND_STREAM, stream)) return rc;
   if (flags & TF_RELU) TF_HIP(tf::launch_relu(h.d, (size_t)h.M * h.N, static_cast<hipStream_t>(stream)));
@@ -821,16 +866,18 @@ extern "C" tf_status tf_schedule_set_profiling(tf_schedule *s, int enable) {
 
 extern "C" tf_status tf_schedule_get_profile(tf_schedule *s, tf_profile *out) {
   if (!s || !out) return fail(TF_EINVAL, "tf_schedule_get_profile: null argument");
-  std::memset(out, 0, sizeof(*out));
-  if (!s->dev || !s->profiling) return TF_OK;
-  tf::DeviceSchedule *d = s->dev;
-  for (int q = 0; q < d->prof_n; ++q) {
-    TF_HIP(hipEventSynchronize(d->prof_ev[q][1]));
-    TF_HIP(hipEventElapsedTime(&out->ms[q], d->prof_ev[q][0], d->prof_ev[q][1]));
-    out->name[q] = d->prof_name[q];
+  tf_profile full;
+  std::memset(&full, 0, sizeof(full));
+  if (s->dev && s->profiling) {
+    tf::DeviceSchedule *d = s->dev;
+    for (int q = 0; q < d->prof_n; ++q) {
+      TF_HIP(hipEventSynchronize(d->prof_ev[q][1]));
+      TF_HIP(hipEventElapsedTime(&full.ms[q], d->prof_ev[q][0], d->prof_ev[q][1]));
+      full.name[q] = d->prof_name[q];
+    }
+    full.n = d->prof_n;
   }
-  out->n = d->prof_n;
-  return TF_OK;
+  return tf::emit_out("tf_schedule_get_profile", out, full, TF_SIZE_THROUGH(tf_profile, ms));
 }
 
 // ---- an executor that allocates nothing ----------------------------------------------------
@@ -883,26 +930,39 @@ extern "C" tf_status tf_gemm(const tf_dense *X, const tf_dense *W, tf_dense *Y, 
     TF_HIP(tf::launch_gemm(X->d, W->d, Y->d, nullptr, M, K, N, tf::default_compute_units(), st));
     return TF_OK;
   }
-  // Shapes the MFMA kernel does not take: K padded to 8 with zeros and N cut into equal panels of 32 .. 256 columns
-  // in buffers that live for this call (allocated and freed here; freeing waits for the stream's work).
+  // Shapes the MFMA kernel does not take: K padded to 8 with zeros and N cut into equal panels of 32 .. 256 columns,
+  // in a workspace this library keeps per device.  It only ever grows: a call whose buffers fit allocates
+  // nothing and does not wait for the stream; a call that needs more frees and allocates (which waits for
+  // the device) and is refused while `st` is being captured into a graph.
   const int Kp = (K + 7) / 8 * 8, n_panels = (N + 255) / 256, Wd = ((N + n_panels - 1) / n_panels + 31) / 32 * 32;
-  float *Xp = nullptr, *Wp = nullptr, *Yp = nullptr;
-  tf_status rc = TF_OK;
-  auto hip_ok = [&](hipError_t e, const char *what) {
-    if (e != hipSuccess && rc == TF_OK) rc = tf::hip_fail(e, what);
-    return e == hipSuccess;
-  };
-  if (Kp != K && hip_ok(hipMalloc(reinterpret_cast<void **>(&Xp), (size_t)M * Kp * sizeof(float)), "hipMalloc(tf_gemm: padded X)"))
-    hip_ok(tf::launch_pad(X->d, M, K, Xp, M, Kp, st), "pad_kernel");
-  if (rc == TF_OK) hip_ok(hipMalloc(reinterpret_cast<void **>(&Wp), (size_t)Kp * Wd * sizeof(float)), "hipMalloc(tf_gemm: panel of W)");
-  if (rc == TF_OK) hip_ok(hipMalloc(reinterpret_cast<void **>(&Yp), (size_t)M * Wd * sizeof(float)), "hipMalloc(tf_gemm: panel of Y)");
-  for (int q = 0; q < n_panels && rc == TF_OK; ++q) {
-    const int c0 = q * Wd, w = std::min(Wd, N - c0);
-    if (hip_ok(tf::launch_copy_cols(W->d, K, N, c0, w, Wp, Kp, Wd, 0, Wd, 0, st), "copy_cols_kernel") &&
-        hip_ok(tf::launch_gemm(Xp ? Xp : X->d, Wp, Yp, nullptr, M, Kp, Wd, tf::default_compute_units(), st), "gemm_rows_kernel"))
-      hip_ok(tf::launch_copy_cols(Yp, M, Wd, 0, w, Y->d, M, N, c0, w, 0, st), "copy_cols_kernel");
+  const size_t need[3] = {Kp != K ? (size_t)M * Kp : 0, (size_t)Kp * Wd, (size_t)M * Wd};
+  int dev = 0;
+  TF_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(TF_EUNSUPPORTED, "tf_gemm: device ordinal %d is beyond the %d this library keeps workspaces for", dev, kMaxDevices);
+  static std::mutex mu;
+  std::lock_guard<std::mutex> lock(mu);
+  GemmWorkspace &ws = g_gemm_ws[dev];
+  for (int q = 0; q < 3; ++q) {
+    if (need[q] <= ws.floats[q]) continue;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return fail(TF_EUNSUPPORTED, "tf_gemm: this shape needs a larger workspace than the library holds, which cannot be allocated while the "
+                  "stream is being captured; call it once with this shape outside the capture first");
+    (void)hipGetLastError();
+    (void)hipFree(ws.buf[q]);  // (waits for work that may still use it)
+    ws.buf[q] = nullptr;
+    ws.floats[q] = 0;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&ws.buf[q]), need[q] * sizeof(float));
+    if (e != hipSuccess) return tf::hip_fail(e, "hipMalloc(tf_gemm workspace)");
+    ws.floats[q] = need[q];
   }
-  if (rc == TF_OK) hip_ok(hipStreamSynchronize(st), "hipStreamSynchronize");
-  (void)hipFree(Xp); (void)hipFree(Wp); (void)hipFree(Yp);
-  return rc;
+  float *Xp = need[0] ? ws.buf[0] : nullptr, *Wp = ws.buf[1], *Yp = ws.buf[2];
+  if (Xp) TF_HIP(tf::launch_pad(X->d, M, K, Xp, M, Kp, st));
+  for (int q = 0; q < n_panels; ++q) {
+    const int c0 = q * Wd, w = std::min(Wd, N - c0);
+    TF_HIP(tf::launch_copy_cols(W->d, K, N, c0, w, Wp, Kp, Wd, 0, Wd, 0, st));
+    TF_HIP(tf::launch_gemm(Xp ? Xp : X->d, Wp, Yp, nullptr, M, Kp, Wd, tf::default_compute_units(), st));
+    TF_HIP(tf::launch_copy_cols(Yp, M, Wd, 0, w, Y->d, M, N, c0, w, 0, st));
+  }
+  return TF_OK;
 }

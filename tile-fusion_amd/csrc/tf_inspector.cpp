@@ -712,7 +712,10 @@ extern "C" void tf_schedule_free(tf_schedule *s) {
 
 extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info *info) {
   if (!s || !info) return tf::fail(TF_EINVAL, "tf_schedule_get_info: null argument");
-  std::memset(info, 0, sizeof(*info));
+  tf_schedule_info full;
+  std::memset(&full, 0, sizeof(full));
+  tf_schedule_info *const caller = info;
+  info = &full;
   info->op = s->opts.op; info->N = s->user_N; info->K = s->user_K;
   info->rows = s->L; info->inter_rows = s->M;
   info->n_tiles = (int)s->tiles.size();
@@ -745,11 +748,15 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   if (s->user_N != s->opts.N) ws += ((long long)s->L + s->opts.K) * s->opts.N * 4;  // one column panel of D and of C
   ws += (long long)s->rem_ptr.size() * 4 + (long long)s->rem_col.size() * 12;       // remainder rows in list order
   info->workspace_bytes = ws;
-  return TF_OK;
+  return tf::emit_out("tf_schedule_get_info", caller, full, TF_SIZE_THROUGH(tf_schedule_info, march_slots));
 }
 
 extern "C" tf_status tf_schedule_get_view(const tf_schedule *s, tf_schedule_view *v) {
   if (!s || !v) return tf::fail(TF_EINVAL, "tf_schedule_get_view: null argument");
+  tf_schedule_view full;
+  std::memset(&full, 0, sizeof(full));
+  tf_schedule_view *const caller = v;
+  v = &full;
   v->n1 = 2;
   v->n_part = s->ptr1[2];
   v->n_id = (int)s->id.size();
@@ -760,7 +767,7 @@ extern "C" tf_status tf_schedule_get_view(const tf_schedule *s, tf_schedule_view
   v->tile_step = s->gemm_stream ? s->tile_step.data() : nullptr;
   v->step_ptr = s->gemm_stream ? s->view_step_ptr.data() : nullptr;
   v->n_step_ptr = s->gemm_stream ? (int)s->view_step_ptr.size() : 0;
-  return TF_OK;
+  return tf::emit_out("tf_schedule_get_view", caller, full, TF_SIZE_THROUGH(tf_schedule_view, n_step_ptr));
 }
 
 extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, const int *Ap,

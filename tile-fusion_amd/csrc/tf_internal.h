@@ -3,7 +3,9 @@
 // include/tilefusion_hip.h.
 #pragma once
 #include <cstdarg>
+#include <cstddef>
 #include <cstdint>
+#include <cstring>
 #include <string>
 #include <vector>
 
@@ -151,6 +153,22 @@ struct tf_schedule {
 namespace tf {
 
 tf_status fail(tf_status code, const char *fmt, ...);
+
+// Out-structs (tf_device_info, tf_schedule_info, tf_schedule_view, tf_profile) begin with the size the
+// caller was compiled with.  `full` is the struct as this library knows it; the caller gets its first
+// min(struct_size, sizeof(T)) bytes and keeps its own struct_size, so nothing is written behind a
+// struct that is shorter than this library's.  min_size = the struct's size in its first version.
+template <class T> tf_status emit_out(const char *who, T *out, T &full, size_t min_size) {
+  const size_t have = out->struct_size;
+  if (have < min_size)
+    return fail(TF_EINVAL, "%s: struct_size is %zu, the struct's first version has %zu bytes (set struct_size to sizeof of the struct before the call)",
+                who, have, min_size);
+  full.struct_size = have;
+  std::memcpy(static_cast<void *>(out), &full, have < sizeof(T) ? have : sizeof(T));
+  return TF_OK;
+}
+// size of struct T up to and including its member m
+#define TF_SIZE_THROUGH(T, m) (offsetof(T, m) + sizeof(((T *)nullptr)->m))
 // tf_march.cpp: builds marching runs into S (returns false, S untouched, when the pattern does not
 // suit them), and checks such a schedule exactly against both patterns.
 bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int *Bp, const int *Bi,

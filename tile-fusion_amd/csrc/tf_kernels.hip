@@ -768,7 +768,6 @@ __global__ void copy_cols_kernel(const float *__restrict__ src, int src_rows, in
   }
 }
 
-// p = max(p, 0), four values per thread (n is a multiple of 4: the kernels' N is).
 // Rows of zeros: Y[rows[q], :] = 0 (second-op rows without entries), V floats per thread.
 template <int V>
 __global__ void zero_rows_kernel(const int *__restrict__ rows, size_t units, float *__restrict__ Y, int N) {
@@ -780,13 +779,16 @@ __global__ void zero_rows_kernel(const int *__restrict__ rows, size_t units, flo
   }
 }
 
-__global__ void relu_kernel(float *__restrict__ p, size_t n4) {
+// p = max(p, 0) over n values: four per thread, and the up to three values behind the last four one each.
+__global__ void relu_kernel(float *__restrict__ p, size_t n) {
+  const size_t n4 = n / 4;
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
     fvec<4> v = *reinterpret_cast<const fvec<4> *>(p + 4 * i);
 #pragma unroll
     for (int c = 0; c < 4; ++c) v.v[c] = fmaxf(v.v[c], 0.f);
     *reinterpret_cast<fvec<4> *>(p + 4 * i) = v;
   }
+  if (blockIdx.x == 0 && 4 * n4 + threadIdx.x < n) p[4 * n4 + threadIdx.x] = fmaxf(p[4 * n4 + threadIdx.x], 0.f);
 }
 
 // out[workgroup] = the XCD it runs on (hardware register XCC_ID, bits 3:0).
@@ -2236,9 +2238,8 @@ hipError_t launch_zero_rows(const int *rows, int n_rows, float *Y, int N, hipStr
 
 hipError_t launch_relu(float *p, size_t n, hipStream_t st) {
   if (n == 0) return hipSuccess;
-  if (n % 4 != 0) return hipErrorInvalidValue;
-  const int blocks = (int)std::min<size_t>((n / 4 + 255) / 256, 65536);
-  hipLaunchKernelGGL(relu_kernel, dim3(blocks), dim3(256), 0, st, p, n / 4);
+  const int blocks = (int)std::max<size_t>(1, std::min<size_t>((n / 4 + 255) / 256, 65536));
+  hipLaunchKernelGGL(relu_kernel, dim3(blocks), dim3(256), 0, st, p, n);
   return hipGetLastError();
 }
 
