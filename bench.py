@@ -193,7 +193,8 @@ def kernel_names(info, op_is_gemm, unfused):
                 "fused_spmm_spmm_kernel" if info["n_fused_rows"] else "spmm_rows_kernel (twice)")
     if info["n_fused_rows"] == 0:
         return "gemm_rows_kernel + spmm_rows_kernel" + (" (+ long-row segments)" if info["n_long_rows"] else "")
-    return "fused_gemm_spmm_stream_kernel" if info["streamed"] else "fused_gemm_spmm_kernel"
+    return ("fused_gemm_spmm_stream_kernel" if info["streamed"] else
+            "fused_gemm_spmm_regw_kernel" if info["register_weights"] else "fused_gemm_spmm_kernel")
 
 
 def run_config(tf, cfg, idx, steps, warmup, args):

@@ -287,7 +287,23 @@ typedef struct {
   int marched;           /* 1 when the tiles are marching runs                       */
   int march_tile_x, march_tile_y; /* grid points of a run per plane                    */
   int march_slots;       /* LDS slots (64-column rows) the fullest run uses          */
+  /* appended after the first version */
+  int march_declined;    /* TF_MARCH_*: whether marching runs were built, and if not, why */
+  int register_weights;  /* 1 when GeMM-SpMM tiles keep C in registers (fused_gemm_spmm_regw_kernel) */
+  int n_zero_rows;       /* second-op rows without entries that a fill kernel clears (counted in n_remainder_rows) */
+  int two_layer_tiles;   /* GeMM-SpMM: tiles that can carry their rows through two layers (tf_gcn_two_layers), else 0 */
 } tf_schedule_info;
+
+/* tf_schedule_info.march_declined */
+enum {
+  TF_MARCH_BUILT = 0,         /* the schedule's tiles are marching runs                                     */
+  TF_MARCH_NOT_TRIED = 1,     /* not SpMM-SpMM with an inner pattern, march = -1, or windowed tiles applied */
+  TF_MARCH_SHAPE = 2,         /* A or B not square with the same row count, or N not a multiple of 64       */
+  TF_MARCH_ROW_TOO_LONG = 3,  /* a row of A or B has more than 8 entries (27- and 9-point stencils)        */
+  TF_MARCH_NO_GRID = 4,       /* grid_nx/ny/nz do not multiply to the row count, or none given and the
+                                 pattern is not a 5- or 7-point-like stencil a grid can be read off      */
+  TF_MARCH_NO_FIT = 5         /* no column of grid points whose rows fit LDS and the run tables            */
+};
 
 tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info *info);
 

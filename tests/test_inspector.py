@@ -434,3 +434,80 @@ def test_validate_checks_windows_against_the_inner_pattern(tf):
         with pytest.raises(tf.TileFusionError) as e:
             S.validate()
         assert e.value.status == -1
+
+
+# ---- marching runs: the validator must reject what does not match --------------------------------
+
+def _moved_column(A, row, k, new_col):
+    B = A.copy()
+    B.indices = B.indices.copy()
+    B.indices[B.indptr[row] + k] = new_col
+    return B
+
+
+def test_march_validator_rejects_other_patterns(tf):
+    """A marching schedule replayed against a pattern it was not built from: one column of one row
+    moved (in A, in the inner matrix, or in both), an entry moved from one row to another (one row
+    longer, one shorter, same entry count), two columns of a row swapped -- each must be refused with
+    TF_ESCHEDULE, and the pattern it was built from must pass before and after."""
+    n = 12
+    A = tf.workloads.laplacian_3d(n)
+    M = A.shape[0]
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah, march=1)
+    info = S.info()
+    assert info["marched"] == 1 and info["march_declined"] == 0
+    S.validate()
+    mid = (n // 2 * n + n // 2) * n + n // 2           # an interior point: 7 entries, columns sorted
+    assert A.indptr[mid + 1] - A.indptr[mid] == 7
+    far = _moved_column(A, mid, 6, mid + n * n + 1)    # its +z neighbour replaced by that one's +x neighbour
+    near = _moved_column(A, mid, 4, mid + 2)           # its +x neighbour replaced by the next point
+    swapped = A.copy(); swapped.indices = swapped.indices.copy()
+    s0 = swapped.indptr[mid]
+    swapped.indices[s0 + 1], swapped.indices[s0 + 2] = swapped.indices[s0 + 2], swapped.indices[s0 + 1]
+    # an entry moved from row `mid` to the corner row 0 (3 + 1 entries -> 5, 7 -> 6), same entry count
+    lil = A.tolil(); lil[mid, mid + 1] = 0; lil[0, 5] = -1.0
+    longer = sp.csr_matrix(lil); longer.eliminate_zeros(); longer.sort_indices()
+    longer = sp.csr_matrix((longer.data.astype(np.float32), longer.indices.astype(np.int32), longer.indptr.astype(np.int32)), shape=A.shape)
+    assert longer.nnz == A.nnz
+    for name, other in (("far column", far), ("near column", near), ("swapped columns", swapped), ("longer row", longer)):
+        Oh = tf.CsrMatrix.from_scipy(other)
+        for outer, inner in ((Oh, Ah), (Ah, Oh), (Oh, Oh)):
+            S._inner = inner
+            with pytest.raises(tf.TileFusionError) as e:
+                S.validate(outer)
+            assert e.value.status == -4, (name, str(e.value))
+    S._inner = Ah
+    S.validate()
+
+
+def test_march_says_why_it_was_declined(tf):
+    """tf_schedule_info.march_declined: marching runs need N % 64 == 0, rows of at most 8 entries in both
+    patterns and a grid; a schedule without them says which of these was missing."""
+    A = tf.workloads.laplacian_3d(12)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    built = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah).info()
+    assert built["marched"] == 1 and built["march_declined"] == 0           # TF_MARCH_BUILT
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64).info()["march_declined"] == 1            # no inner pattern: not tried
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah, march=-1).info()["march_declined"] == 1
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=32, inner=Ah).info()["march_declined"] == 2  # N % 64
+    # a 27-point stencil: rows of up to 27 entries
+    e = np.ones(12)
+    t = sp.diags([e[:-1], e, e[:-1]], [-1, 0, 1])
+    W = sp.csr_matrix(sp.kron(sp.kron(t, t), t), dtype=np.float32)
+    W.sort_indices()
+    W = sp.csr_matrix((W.data, W.indices.astype(np.int32), W.indptr.astype(np.int32)), shape=W.shape)
+    Wh = tf.CsrMatrix.from_scipy(W)
+    assert tf.inspector(Wh, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Wh).info()["march_declined"] == 3
+    # short rows, but no grid to be found and none given; a grid that does not multiply to the row count
+    R = tf.workloads.erdos_renyi_gcn(1500, 2.0, seed=4)
+    R = sp.csr_matrix(R.multiply(sp.csr_matrix(np.diff(R.indptr)[:, None] <= 8)), dtype=np.float32)
+    deg = np.diff(R.indptr)
+    if deg.max() <= 8:
+        R.sort_indices()
+        R = sp.csr_matrix((R.data, R.indices.astype(np.int32), R.indptr.astype(np.int32)), shape=R.shape)
+        Rh = tf.CsrMatrix.from_scipy(R)
+        assert tf.inspector(Rh, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Rh).info()["march_declined"] == 4
+    assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah, grid=(12, 12, 11)).info()["march_declined"] == 4
+    with pytest.raises(tf.TileFusionError):
+        tf.inspector(Wh, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Wh, march=1)

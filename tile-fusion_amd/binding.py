@@ -51,7 +51,8 @@ class ScheduleInfo(C.Structure):
                 ("max_tile_producer_rows", C.c_int), ("lds_bytes", C.c_int), ("windowed", C.c_int),
                 ("strip_cols", C.c_int), ("xcd_chunk_rows", C.c_int), ("streamed", C.c_int), ("ring_rows", C.c_int), ("wide_strips", C.c_int), ("long_row_hot_cols", C.c_int),
                 ("fused_nnz", C.c_longlong), ("workspace_bytes", C.c_longlong),
-                ("marched", C.c_int), ("march_tile_x", C.c_int), ("march_tile_y", C.c_int), ("march_slots", C.c_int)]
+                ("marched", C.c_int), ("march_tile_x", C.c_int), ("march_tile_y", C.c_int), ("march_slots", C.c_int),
+                ("march_declined", C.c_int), ("register_weights", C.c_int), ("n_zero_rows", C.c_int), ("two_layer_tiles", C.c_int)]
 
 
 class ScheduleView(C.Structure):

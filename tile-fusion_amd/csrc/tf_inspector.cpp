@@ -739,6 +739,10 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   info->march_tile_x = s->march_tile[0];
   info->march_tile_y = s->march_tile[1];
   info->march_slots = s->march_slots;
+  info->march_declined = s->march_declined;
+  info->register_weights = s->gemm_regw ? 1 : 0;
+  info->n_zero_rows = (int)s->zero_rows.size();
+  info->two_layer_tiles = 0;
   long long ws = 0;
   if (s->march) ws += (long long)s->march_ell_off.size() * 16;  // ELL rows with values, their offsets and sources
   if (s->n_writeback_rows > 0) ws += (long long)s->M * s->opts.N * 4;

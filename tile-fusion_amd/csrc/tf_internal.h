@@ -124,6 +124,7 @@ struct tf_schedule {
   // go to their slots.  Every entry of an ELL row names the LDS byte offset of the row it reads; the
   // inspector assigns the slots so that a row stays until its last reader has run.
   bool march = false;
+  int march_declined = TF_MARCH_NOT_TRIED;  // why there are no marching runs (TF_MARCH_*), TF_MARCH_BUILT when there are
   int march_grid[3] = {0, 0, 0};     // the grid the runs were cut from (x fastest)
   int march_tile[2] = {0, 0};        // grid points per run and plane: x, y
   int march_slots = 0;               // LDS slots in use by the fullest run

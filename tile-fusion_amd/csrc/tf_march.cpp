@@ -61,19 +61,21 @@ bool detect_grid(int M, const int *Ap, const int *Ai, int grid[3]) {
 
 bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int *Bp, const int *Bi,
                  const tf_inspect_opts &o, const tf_inspect_opts &given) {
-  if (S->L != M || o.inner_cols != M || o.N % 64 != 0) return false;
+  // (every way out says why in S->march_declined, which tf_schedule_get_info reports)
+  auto decline = [&](int why) { S->march_declined = why; return false; };
+  if (S->L != M || o.inner_cols != M || o.N % 64 != 0) return decline(TF_MARCH_SHAPE);
   const long long nnzA = Ap[M], nnzB = Bp[M];
-  if (nnzA >= kMarchSrcA || nnzB >= kMarchSrcA) return false;
+  if (nnzA >= kMarchSrcA || nnzB >= kMarchSrcA) return decline(TF_MARCH_SHAPE);
   int width = 0;
   for (int i = 0; i < M; ++i) {
-    if (Ap[i + 1] - Ap[i] > kMarchW || Bp[i + 1] - Bp[i] > kMarchW) return false;
+    if (Ap[i + 1] - Ap[i] > kMarchW || Bp[i + 1] - Bp[i] > kMarchW) return decline(TF_MARCH_ROW_TOO_LONG);
     width = std::max(width, std::max(Ap[i + 1] - Ap[i], Bp[i + 1] - Bp[i]));
   }
   int grid[3] = {given.grid_nx, given.grid_ny, given.grid_nz};
   if (grid[0] > 0 || grid[1] > 0 || grid[2] > 0) {
-    if (grid[0] <= 0 || grid[1] <= 0 || grid[2] <= 0 || (long long)grid[0] * grid[1] * grid[2] != M) return false;
+    if (grid[0] <= 0 || grid[1] <= 0 || grid[2] <= 0 || (long long)grid[0] * grid[1] * grid[2] != M) return decline(TF_MARCH_NO_GRID);
   } else if (!detect_grid(M, Ap, Ai, grid)) {
-    return false;
+    return decline(TF_MARCH_NO_GRID);
   }
   const int nx = grid[0], ny = grid[1], nz = grid[2];
   const int slot_budget = (kMaxLds - kMarchSlot0) / kMarchRowBytes;
@@ -297,7 +299,8 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
       }
     }
   }
-  if (!ok) return false;
+  if (!ok) return decline(TF_MARCH_NO_FIT);
+  S->march_declined = TF_MARCH_BUILT;
 
   // MultiDimensionalSet-layout view: one partition per run, its grid points as first-op ids
   // (the intermediate rows it owns; halo rows it recomputes belong to their own runs), then the

@@ -41,7 +41,6 @@ from . import binding as _b
 __all__ = ["clear_cache"]
 
 _VP = C.c_void_p
-_MAX_N = 256  # widest GeMM-SpMM the library schedules in one call
 
 
 def _require_gpu(*tensors):
@@ -157,10 +156,6 @@ def clear_cache():
     _cache.clear()
 
 
-def _pad_to(x, mult):
-    return (x + mult - 1) // mult * mult
-
-
 def _gemm_spmm(ctx, X, Wkn):
     """ctx.A @ (X @ Wkn) with X [M, K], Wkn [K, N], through tf_gemm_spmm."""
     _require_gpu(X, Wkn)
@@ -171,21 +166,11 @@ def _gemm_spmm(ctx, X, Wkn):
     X = X.to(torch.float32)
     Wkn = Wkn.to(torch.float32)
     X = X.contiguous()
+    Wkn = Wkn.contiguous()
     out = torch.empty((ctx.shape[0], N), dtype=torch.float32, device=X.device)
-    for n0 in range(0, N, _MAX_N):  # the library schedules at most 256 columns per call
-        n1 = min(N, n0 + _MAX_N)
-        Np = _pad_to(n1 - n0, 32)
-        Wc = Wkn[:, n0:n1]
-        if Np != n1 - n0:
-            Wc = torch.nn.functional.pad(Wc, (0, Np - (n1 - n0)))
-        Wc = Wc.contiguous()
-        whole = (n0 == 0 and n1 == N and Np == N)
-        dst = out if whole else torch.empty((ctx.shape[0], Np), dtype=torch.float32, device=X.device)
-        S = ctx.schedule(K, Np)
-        with _Dense(X) as xb, _Dense(Wc) as wc, _Dense(dst) as db:
-            _b._check(_b.lib().tf_gemm_spmm(ctx.h, xb, wc, db, S.h, 0, _stream()))
-        if not whole:
-            out[:, n0:n1] = dst[:, :n1 - n0]
+    S = ctx.schedule(K, N)  # any K and N: the library pads K and cuts N into column panels itself
+    with _Dense(X) as xb, _Dense(Wkn) as wc, _Dense(out) as db:
+        _b._check(_b.lib().tf_gemm_spmm(ctx.h, xb, wc, db, S.h, 0, _stream()))
     return out
 
 
@@ -243,7 +228,7 @@ def inspect(Adj, MTileSize):
 
 def inspect_vt_ro(Adj, InDim, OutDim, CacheSize, NumThreads):
     del CacheSize, NumThreads
-    return _schedule_tensors(_ctx(Adj), _pad_to(int(InDim), 8), min(_MAX_N, _pad_to(int(OutDim), 32)))
+    return _schedule_tensors(_ctx(Adj), int(InDim), int(OutDim))
 
 
 def executeFusedGeMMSpMM(Adj, Weight, Feature, LevelPtr, MixPtr, Partition, NumThreads):
@@ -310,19 +295,14 @@ def _two_layers(ctx, X, W1kn, W2kn, relu):
     H, N = W1kn.shape[1], W2kn.shape[1]
     if ctx.shape[0] != ctx.shape[1] or ctx.shape[1] != M or W1kn.shape[0] != K or W2kn.shape[0] != H:
         raise RuntimeError(f"sw_gcn: shapes do not chain: Adj {ctx.shape}, Feature {tuple(X.shape)}, weights {tuple(W1kn.shape)}, {tuple(W2kn.shape)}")
-    Hp, Np = _pad_to(H, 32), _pad_to(N, 32)
-    if Hp > _MAX_N or Np > _MAX_N:  # wider layers go through the single-layer path, which splits columns
-        h = _gemm_spmm(ctx, X, W1kn)
-        return _gemm_spmm(ctx, h.relu_() if relu else h, W2kn)
     X = X.to(torch.float32).contiguous()
-    # zero columns of W1 give zero hidden columns (also after ReLU), which meet zero rows of W2
-    W1p = torch.nn.functional.pad(W1kn.to(torch.float32), (0, Hp - H)).contiguous()
-    W2p = torch.nn.functional.pad(W2kn.to(torch.float32), (0, Np - N, 0, Hp - H)).contiguous()
-    out = torch.empty((M, Np), dtype=torch.float32, device=X.device)
-    s1, s2 = ctx.schedule(K, Hp), ctx.schedule(Hp, Np)
-    with _Dense(X) as xb, _Dense(W1p) as w1, _Dense(W2p) as w2, _Dense(out) as ob:
+    W1 = W1kn.to(torch.float32).contiguous()
+    W2 = W2kn.to(torch.float32).contiguous()
+    out = torch.empty((M, N), dtype=torch.float32, device=X.device)
+    s1, s2 = ctx.schedule(K, H), ctx.schedule(H, N)  # any widths: the library cuts column panels itself
+    with _Dense(X) as xb, _Dense(W1) as w1, _Dense(W2) as w2, _Dense(out) as ob:
         _b._check(_b.lib().tf_gcn_two_layers(ctx.h, xb, w1, w2, ob, s1.h, s2.h, None, _b.RELU if relu else 0, _stream()))
-    return out if Np == N else out[:, :N].contiguous()
+    return out
 
 
 def fusedGCN(Adj, Feature, Weight1, Weight2, NumThreads):
