@@ -245,6 +245,12 @@ typedef struct {
      the 8 XCD partitions; default 12 MB, three times an XCD's L2 (the reads inside a partition are skewed
      too, and its hottest rows are what stays). */
   int hot_partition_bytes;
+  /* Short remainder rows kept in list order (reorder_adjacency) on a graph with hub rows: bytes of most-read
+     intermediate rows that those rows' gathers may keep in an L2; gathers of all other rows are marked in the
+     schedule and fetched with streaming loads, so that rows read once do not push out rows with readers.
+     0 = 8 MB when the long rows are column-partitioned (long_row_partition: a power-law graph), else off;
+     -1 = off; n > 0 = n bytes.  Only when N is a multiple of 4, and only if the set takes a quarter of the reads. */
+  int short_row_hot_bytes;
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -292,6 +298,11 @@ typedef struct {
   int register_weights;  /* 1 when GeMM-SpMM tiles keep C in registers (fused_gemm_spmm_regw_kernel) */
   int n_zero_rows;       /* second-op rows without entries that a fill kernel clears (counted in n_remainder_rows) */
   int two_layer_tiles;   /* GeMM-SpMM: tiles that can carry their rows through two layers (tf_gcn_two_layers), else 0 */
+  int short_row_hot_rows; /* intermediate rows whose gathers by the short remainder rows are left cacheable
+                            (short_row_hot_bytes), else 0                                                    */
+  int n_computed_rows;   /* intermediate rows the executor computes per call: the producer rows of the tiles it
+                            launches (halo rows included) plus, for tiles that fuse nothing, only the rows some
+                            remainder row reads -- on a graph with isolated nodes fewer than inter_rows       */
 } tf_schedule_info;
 
 /* tf_schedule_info.march_declined */

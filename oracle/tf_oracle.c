@@ -138,13 +138,26 @@ void orc_spmm_spmm_fused_separated(int M, int N, const int *Ap, const int *Ai,
 
 /* Row-major out[T x N] = X[T x K] * W[K x N], beta = 0: the call
  * cblas_sgemm(RowMajor, NoTrans, NoTrans, T, N, K, 1, X, K, W, N, 0, out, N)
- * at fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:233-237.  Textbook product,
- * k ascending, fma; MKL's internal order is not reproducible (see header). */
-static void sgemm_rows(int T, int N, int K, const float *X, const float *W, float *out) {
+ * at fusion/gcn/GCN_Layer_MKL_Forward_Utils.h:233-237.  Textbook product:
+ * every element is one chain of fused multiply-adds with k ascending; MKL's
+ * internal order is not reproducible (see header).
+ *
+ * Two bodies with the same arithmetic per element, hence the same bits:
+ *   sgemm_rows_scalar   4 x 32 blocks of plain fmaf (what -march=x86-64-v3 makes
+ *                       of it: AVX2), any shape;
+ *   sgemm_rows_avx512   register-blocked micro-kernel for hosts with AVX-512
+ *                       (checked at run time): 8 rows x 32 columns of
+ *                       accumulators in 16 zmm registers, per k two loads of W
+ *                       and eight broadcasts of X; the column block is the outer
+ *                       loop so that its 32-column panel of W stays in L1 for
+ *                       all row blocks of the tile.  This is the class of
+ *                       kernel the reference gets from MKL, so that the CPU
+ *                       baseline built on it is one worth standing next to. */
+static void sgemm_rows_scalar(int T, int N, int K, const float *X, const float *W, float *out, int j_begin) {
   enum { RB = 4, CB = 32 };
   for (int i0 = 0; i0 < T; i0 += RB) {
     const int rb = (T - i0 < RB) ? (T - i0) : RB;
-    for (int j0 = 0; j0 < N; j0 += CB) {
+    for (int j0 = j_begin; j0 < N; j0 += CB) {
       const int cb = (N - j0 < CB) ? (N - j0) : CB;
       float acc[RB][CB];
       for (int r = 0; r < RB; ++r)
@@ -170,6 +183,70 @@ static void sgemm_rows(int T, int N, int K, const float *X, const float *W, floa
         for (int c = 0; c < cb; ++c) out[(size_t)(i0 + r) * N + j0 + c] = acc[r][c];
     }
   }
+}
+
+#if defined(__x86_64__)
+#include <immintrin.h>
+#define ORC_HAVE_AVX512_BODY 1
+/* rows [0, T8) (T8 a multiple of 8) x columns [0, N32) (a multiple of 32) */
+__attribute__((target("avx512f"))) static void sgemm_rows_avx512(int T8, int N32, int N, int K, const float *X,
+                                                                  const float *W, float *out) {
+  for (int j0 = 0; j0 < N32; j0 += 32) {
+    for (int i0 = 0; i0 < T8; i0 += 8) {
+      __m512 a0[8], a1[8];
+      for (int r = 0; r < 8; ++r) { a0[r] = _mm512_setzero_ps(); a1[r] = _mm512_setzero_ps(); }
+      const float *x = X + (size_t)i0 * K;
+      const float *w = W + j0;
+      for (int k = 0; k < K; ++k) {
+        const __m512 w0 = _mm512_loadu_ps(w + (size_t)k * N);
+        const __m512 w1 = _mm512_loadu_ps(w + (size_t)k * N + 16);
+#pragma GCC unroll 8
+        for (int r = 0; r < 8; ++r) {
+          const __m512 xv = _mm512_set1_ps(x[(size_t)r * K + k]);
+          a0[r] = _mm512_fmadd_ps(xv, w0, a0[r]);
+          a1[r] = _mm512_fmadd_ps(xv, w1, a1[r]);
+        }
+      }
+      for (int r = 0; r < 8; ++r) {
+        _mm512_storeu_ps(out + (size_t)(i0 + r) * N + j0, a0[r]);
+        _mm512_storeu_ps(out + (size_t)(i0 + r) * N + j0 + 16, a1[r]);
+      }
+    }
+  }
+}
+#else
+#define ORC_HAVE_AVX512_BODY 0
+#endif
+
+static int g_simd = -1; /* -1: not decided yet; 0: scalar body only; 1: AVX-512 body where it applies */
+
+/* 1 when the AVX-512 body is in use.  orc_set_simd(0) forces the scalar body (tests compare the two). */
+int orc_simd(void) {
+  if (g_simd < 0) {
+#if ORC_HAVE_AVX512_BODY
+    g_simd = __builtin_cpu_supports("avx512f") ? 1 : 0;
+#else
+    g_simd = 0;
+#endif
+  }
+  return g_simd;
+}
+void orc_set_simd(int on) {
+  g_simd = -1;
+  if (!on || !orc_simd()) g_simd = 0;
+}
+
+static void sgemm_rows(int T, int N, int K, const float *X, const float *W, float *out) {
+#if ORC_HAVE_AVX512_BODY
+  if (orc_simd()) {
+    const int T8 = T / 8 * 8, N32 = N / 32 * 32;
+    if (T8 > 0 && N32 > 0) sgemm_rows_avx512(T8, N32, N, K, X, W, out);
+    if (T8 > 0 && N32 < N) sgemm_rows_scalar(T8, N, K, X, W, out, N32);                  /* columns behind the last 32 */
+    if (T8 < T) sgemm_rows_scalar(T - T8, N, K, X + (size_t)T8 * K, W, out + (size_t)T8 * N, 0); /* rows behind the last 8 */
+    return;
+  }
+#endif
+  sgemm_rows_scalar(T, N, K, X, W, out, 0);
 }
 
 /* out = X * W for the whole matrix (the unfused baseline's GEMM,

@@ -189,6 +189,18 @@ def spmm_spmm_separated(A, Cd, sched, nthreads=1, impl="oracle"):
     return D, T
 
 
+def simd():
+    """1 when the oracle's GEMM runs its AVX-512 body on this host."""
+    o = oracle()
+    o.orc_simd.restype = C.c_int
+    return int(o.orc_simd())
+
+
+def set_simd(on):
+    """False forces the scalar body of the oracle's GEMM (the two give the same bits)."""
+    oracle().orc_set_simd(1 if on else 0)
+
+
 def gemm(X, W, nthreads=1):
     M, K = X.shape
     N = W.shape[1]

@@ -418,3 +418,25 @@ def test_device_reports_the_workgroup_to_xcd_mapping(gpu):
     """tf_device_init probes what the XCD-pinned kernels rely on: workgroup b runs on XCD b mod 8."""
     assert gpu["xcds"] == 8 and gpu["compute_units"] == 256 and gpu["wavefront"] == 64
     assert gpu["xcd_round_robin"] == 1, gpu
+
+
+def test_streaming_gathers_of_short_rows_change_no_bit(gpu, tf, orc):
+    """short_row_hot_bytes only changes which load instruction fetches a gathered row: a power-law product with
+    the short rows' cold gathers marked (default), with a tiny hot set, and with the marks off gives the same bits."""
+    say("short rows: streaming gathers")
+    cfg = tf.workloads.make_config(4, 2.0 ** -5)
+    A, B, W = cfg["A"], cfg["B"], cfg["C"]
+    M = A.shape[0]
+    Ah = tf.CsrMatrix.from_scipy(A)
+    Bd, Wd = tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W)
+    outs = []
+    for hot in (0, 64 << 10, -1):
+        S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1, short_row_hot_bytes=hot)
+        S.validate()
+        assert (S.info()["short_row_hot_rows"] > 0) == (hot >= 0)
+        D = tf.DenseMatrix(M, 128); D.fill(float("nan"))
+        tf.gemm_spmm(Ah, Bd, Wd, D, S)
+        outs.append(D.to_numpy())
+    assert np.array_equal(outs[0], outs[2]) and np.array_equal(outs[1], outs[2])
+    want, _ = orc.gemm_spmm(A, B, W, orc.unfused_schedule(M), nthreads=8)
+    assert orc.rel_err(outs[0], want) <= TOL

@@ -511,3 +511,24 @@ def test_march_says_why_it_was_declined(tf):
     assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah, grid=(12, 12, 11)).info()["march_declined"] == 4
     with pytest.raises(tf.TileFusionError):
         tf.inspector(Wh, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Wh, march=1)
+
+
+def test_short_rows_mark_their_cold_gathers_on_power_law_graphs(tf):
+    """short_row_hot_bytes: on a graph with hub rows (long rows column-partitioned) the short remainder rows keep
+    their gathers of the most-read intermediate rows cacheable and mark all others as streaming; a graph without
+    a hot set (Erdos-Renyi) marks nothing; the schedule validates either way and -1 switches it off."""
+    cfg = tf.workloads.make_config(4, 2.0 ** -5)
+    Ah = tf.CsrMatrix.from_scipy(cfg["A"])
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1)
+    S.validate()
+    info = S.info()
+    assert info["long_row_hot_cols"] > 0 and 0 < info["short_row_hot_rows"] <= (8 << 20) // 512
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1, short_row_hot_bytes=1 << 20)
+    S.validate()
+    assert 0 < S.info()["short_row_hot_rows"] <= 2048
+    assert tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1, short_row_hot_bytes=-1).info()["short_row_hot_rows"] == 0
+    er = tf.workloads.make_config(3, 0.05)
+    Eh = tf.CsrMatrix.from_scipy(er["A"])
+    S = tf.inspector(Eh, 1, op=tf.OP_GEMM_SPMM, N=128, K=256, short_row_hot_bytes=256 << 10)   # 512 of 10,000 rows
+    S.validate()
+    assert S.info()["short_row_hot_rows"] == 0

@@ -168,3 +168,39 @@ def test_permutation_invariance(orc, tf):
     D, _ = orc.gemm_spmm(A, B, Cw, orc.unfused_schedule(M))
     Dp, _ = orc.gemm_spmm(Ap.astype(np.float32), B[perm], Cw, orc.unfused_schedule(M))
     assert np.array_equal(Dp, D[perm])
+
+
+def test_gemm_avx512_body_gives_the_scalar_bits(orc):
+    """The oracle's GEMM has a register-blocked AVX-512 body (the CPU baseline's GEMM) and a scalar one;
+    both add each element's products with k ascending through fused multiply-adds, so the bits must agree
+    -- for whole 8 x 32 blocks, for rows and columns behind them, for K of any size, and through the fused
+    executor.  Against float64 and an integer-exact product as well, so that both cannot be wrong together."""
+    rng = np.random.default_rng(7)
+    if not orc.simd():
+        pytest.skip("this host has no AVX-512: only the scalar body runs")
+    try:
+        for M, K, N in ((64, 128, 128), (61, 128, 128), (203, 40, 96), (77, 256, 72), (8, 1, 32), (5, 16, 64), (129, 33, 200)):
+            X = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+            W = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+            orc.set_simd(True)
+            fast = orc.gemm(X, W, nthreads=3)
+            orc.set_simd(False)
+            slow = orc.gemm(X, W, nthreads=3)
+            assert np.array_equal(fast, slow), (M, K, N)
+            want = X.astype(np.float64) @ W.astype(np.float64)
+            assert np.abs(fast - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
+        Xi = rng.integers(-3, 4, (96, 24)).astype(np.float32)
+        Wi = rng.integers(-3, 4, (24, 64)).astype(np.float32)   # K != N: a transposed operand cannot pass
+        orc.set_simd(True)
+        assert np.array_equal(orc.gemm(Xi, Wi), (Xi.astype(np.int64) @ Wi.astype(np.int64)).astype(np.float32))
+        A = sp.random(300, 300, density=0.03, random_state=5, format="csr", dtype=np.float32)
+        A.sort_indices()
+        B = rng.uniform(-1, 1, (300, 64)).astype(np.float32)
+        Cd = rng.uniform(-1, 1, (64, 96)).astype(np.float32)
+        S = orc.inspect_fixed_tiles(A, 64, 4)
+        d_fast, _ = orc.gemm_spmm(A, B, Cd, S, nthreads=4)
+        orc.set_simd(False)
+        d_slow, _ = orc.gemm_spmm(A, B, Cd, S, nthreads=4)
+        assert np.array_equal(d_fast, d_slow)
+    finally:
+        orc.set_simd(True)

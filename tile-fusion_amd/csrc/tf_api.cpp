@@ -88,7 +88,7 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *, const int *, int, c
                                            const float *, int, const float *, const int *, const int *,
                                            const float *, int, float *, int, int, int, int, hipStream_t);
 hipError_t launch_spmm_rows(const int *, int, const int *, const int *, const float *, const float *,
-                            float *, int, int, int, int, hipStream_t, int compact = 0, int coalesced_pairs = 0);
+                            float *, int, int, int, int, hipStream_t, int compact = 0, int coalesced_pairs = 0, int flagged = 0);
 hipError_t launch_gather_values(const int *, const float *, float *, int, hipStream_t);
 hipError_t launch_march_fill(const int *, const int *, const float *, const float *, int *, size_t, hipStream_t);
 hipError_t launch_fused_spmm_spmm_march(const int *, int, const int *, const int *, const int *, const int *, const int *,
@@ -335,7 +335,7 @@ static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int
     d->rem_val_serial = A->serial;
     TF_PHASE(s, "spmm_rows_kernel (short remainder rows)", st,
              launch_spmm_rows(d->rem_rows, (int)s->rem_rows.size(), d->rem_ptr, d->rem_col, d->rem_val, d->inter, D->d, N, accumulate,
-                              s->xcd_chunk_rows, /*streaming=*/1, st, /*compact=*/1));
+                              s->xcd_chunk_rows, /*streaming=*/1, st, /*compact=*/1, /*coalesced_pairs=*/0, s->rem_flagged ? 1 : 0));
   } else if (!s->rem_rows.empty()) {
     // identity list: no indirection needed
     TF_PHASE(s, "spmm_rows_kernel (short remainder rows)", st,

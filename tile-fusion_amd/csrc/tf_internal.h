@@ -96,6 +96,8 @@ struct tf_schedule {
   // (row q of it is row rem_rows[q] of A): rem_ptr [n + 1], rem_col, and rem_src = where each entry
   // sits in A's arrays (the executor copies the values from there).
   std::vector<int> rem_ptr, rem_col, rem_src;
+  bool rem_flagged = false;  // rem_col carries the "cold" mark in the top bit of some columns (short_row_hot_bytes)
+  int rem_hot_rows = 0;      // intermediate rows left unmarked
   int xcd_chunk_rows = 0;           // rows per XCD turn of the row kernels (0: one contiguous run per XCD)
   std::vector<tf::LongChunk> long_chunks;
   std::vector<tf::LongRow> long_rows;

@@ -94,6 +94,25 @@ template <int V> struct GlobalRows {
   __device__ __forceinline__ fvec<V> load(int row) const {
     return *reinterpret_cast<const fvec<V> *>(base + (size_t)row * ld + coff);
   }
+  // A column index whose top bit is set names a row the schedule expects no second reader to find in L2
+  // ("cold"): it is fetched with a streaming load, so that it does not push a row with readers out.
+  __device__ __forceinline__ fvec<V> load_flagged(int c) const {
+    const float *p = base + (size_t)(c & INT_MAX) * ld + coff;
+    fvec<V> r;
+    if (c < 0) {
+      if constexpr (V == 1) {
+        r.v[0] = __builtin_nontemporal_load(p);
+      } else {
+        typedef float fv __attribute__((ext_vector_type(V)));
+        const fv x = __builtin_nontemporal_load(reinterpret_cast<const fv *>(p));
+#pragma unroll
+        for (int u = 0; u < V; ++u) r.v[u] = x[u];
+      }
+    } else {
+      r = *reinterpret_cast<const fvec<V> *>(p);
+    }
+    return r;
+  }
 };
 template <int V> struct LdsRows {
   const float *base;  // slab; row r of the intermediate is at (r - first) * ld
@@ -109,7 +128,7 @@ template <int V> struct LdsRows {
 // eight (or four) at a time: all gathers of a batch are issued before its first fma, and a
 // short last batch re-reads the last entry in its unused slots and skips their fma, so a
 // short row costs one gather round trip instead of one per entry.
-template <int V, int LPR, int B, class Src>
+template <int V, int LPR, int B, class Src, bool FLAG = false>
 __device__ __forceinline__ void row_dot_batch(int c, float a, int t, int cnt, bool col_ok, const Src &src,
                                               fvec<V> &acc) {
   int cc[B];
@@ -123,7 +142,10 @@ __device__ __forceinline__ void row_dot_batch(int c, float a, int t, int cnt, bo
   if (col_ok) {
     fvec<V> x[B];
 #pragma unroll
-    for (int u = 0; u < B; ++u) x[u] = (t + u < cnt) ? src.load(cc[u]) : vzero<V>();
+    for (int u = 0; u < B; ++u) {
+      if constexpr (FLAG) x[u] = (t + u < cnt) ? src.load_flagged(cc[u]) : vzero<V>();
+      else x[u] = (t + u < cnt) ? src.load(cc[u]) : vzero<V>();
+    }
 #pragma unroll
     for (int u = 0; u < B; ++u) {
       fvec<V> next = acc;
@@ -134,17 +156,17 @@ __device__ __forceinline__ void row_dot_batch(int c, float a, int t, int cnt, bo
 }
 
 // The same for cnt <= LPR entries already in registers: lane g of the group holds entry g.
-template <int V, int LPR, class Src>
+template <int V, int LPR, class Src, bool FLAG = false>
 __device__ __forceinline__ void row_dot_loaded(int c, float a, int cnt, bool col_ok, const Src &src,
                                                fvec<V> &acc) {
   int t = 0;
   if constexpr (LPR >= 8)
-    for (; t + 8 <= cnt; t += 8) row_dot_batch<V, LPR, 8>(c, a, t, cnt, col_ok, src, acc);
-  if (t + 4 <= cnt) { row_dot_batch<V, LPR, 4>(c, a, t, cnt, col_ok, src, acc); t += 4; }
-  if (t < cnt) row_dot_batch<V, LPR, 4>(c, a, t, cnt, col_ok, src, acc);
+    for (; t + 8 <= cnt; t += 8) row_dot_batch<V, LPR, 8, Src, FLAG>(c, a, t, cnt, col_ok, src, acc);
+  if (t + 4 <= cnt) { row_dot_batch<V, LPR, 4, Src, FLAG>(c, a, t, cnt, col_ok, src, acc); t += 4; }
+  if (t < cnt) row_dot_batch<V, LPR, 4, Src, FLAG>(c, a, t, cnt, col_ok, src, acc);
 }
 
-template <int V, int LPR, class Src>
+template <int V, int LPR, class Src, bool FLAG = false>
 __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float *__restrict__ val,
                                         int kb, int ke, int glane, bool col_ok, const Src &src,
                                         fvec<V> &acc) {
@@ -153,7 +175,7 @@ __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float
     int c = 0;
     float a = 0.f;
     if (k < ke) { c = idx[k]; a = val[k]; }
-    row_dot_loaded<V, LPR>(c, a, min(LPR, ke - k0), col_ok, src, acc);
+    row_dot_loaded<V, LPR, Src, FLAG>(c, a, min(LPR, ke - k0), col_ok, src, acc);
   }
 }
 
@@ -164,7 +186,7 @@ __device__ __forceinline__ void row_dot(const int *__restrict__ idx, const float
 // 112 registers instead of 60 and halves the wavefronts in flight: the R-MAT step went from 2.24 to
 // 2.88 ms.  Wavefronts in flight are worth more to these launches than a shorter chain of dependent
 // loads per row.)
-template <int V, int LPR, class Src>
+template <int V, int LPR, class Src, bool FLAG = false>
 __device__ __forceinline__ void row_dot_direct(const int *__restrict__ idx, const float *__restrict__ val,
                                                int kb, int ke, bool col_ok, const Src &src, fvec<V> &acc) {
   for (int k0 = kb; k0 < ke; k0 += 8) {
@@ -179,7 +201,10 @@ __device__ __forceinline__ void row_dot_direct(const int *__restrict__ idx, cons
     if (col_ok) {
       fvec<V> x[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) x[u] = (k0 + u < ke) ? src.load(cc[u]) : vzero<V>();
+      for (int u = 0; u < 8; ++u) {
+        if constexpr (FLAG) x[u] = (k0 + u < ke) ? src.load_flagged(cc[u]) : vzero<V>();
+        else x[u] = (k0 + u < ke) ? src.load(cc[u]) : vzero<V>();
+      }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         fvec<V> next = acc;
@@ -622,7 +647,7 @@ __global__ __launch_bounds__(kW64Block) void fused_spmm_spmm_window64_kernel(
 // that no tile fuses, and tf_spmm.  One lane group per row and small, short-lived
 // workgroups: what hides the gather latency is the number of rows in flight.
 // ---------------------------------------------------------------------------------
-template <int V, int LPR, bool COAL>
+template <int V, int LPR, bool COAL, bool FLAG = false>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
     const int *__restrict__ rows, int n_rows, int n_blocks, int per_xcd, const int *__restrict__ Ap,
     const int *__restrict__ Ai, const float *__restrict__ Ax, const float *__restrict__ X, int ldx,
@@ -649,8 +674,9 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(
     // per eight entries (hot long-row segments of the R-MAT step, 22 entries on average: 0.86 -> 0.74
     // ms).  Rows of a few entries, and segments whose gathers all miss L2, are served as well or
     // better by every lane reading the pairs itself (cold segments 0.27 -> 0.29 ms).
-    if constexpr (COAL) row_dot<V, LPR>(Ai, Ax, kb, ke, glane, ok, src, acc);
-    else row_dot_direct<V, LPR>(Ai, Ax, kb, ke, ok, src, acc);
+    // FLAG: column indices carry the schedule's "cold" mark in their top bit (see GlobalRows::load_flagged)
+    if constexpr (COAL) row_dot<V, LPR, GlobalRows<V>, FLAG>(Ai, Ax, kb, ke, glane, ok, src, acc);
+    else row_dot_direct<V, LPR, GlobalRows<V>, FLAG>(Ai, Ax, kb, ke, ok, src, acc);
     if (ok) {
       if (streaming) store_streaming<V>(Y + (size_t)i * N + coff, acc);
       else *reinterpret_cast<fvec<V> *>(Y + (size_t)i * N + coff) = acc;
@@ -2008,20 +2034,29 @@ hipError_t launch_fused_spmm_spmm_window64(const TileDesc *tiles, const int *win
 
 hipError_t launch_spmm_rows(const int *rows, int n_rows, const int *Ap, const int *Ai, const float *Ax,
                             const float *X, float *Y, int N, int accumulate, int xcd_chunk_rows,
-                            int streaming, hipStream_t st, int compact, int coalesced_pairs) {
+                            int streaming, hipStream_t st, int compact, int coalesced_pairs, int flagged) {
   if (n_rows <= 0) return hipSuccess;
   const Shape s = pick_shape(N);
+  if (flagged && s.V != 4) return hipErrorInvalidValue;  // (schedules mark columns only when N is a multiple of 4)
   const int G = kBlock / s.LPR;
   const int n_blocks = (n_rows + G - 1) / G;
   // 0: workgroup b takes block b; > 0: chunks of rows per XCD turn; < 0: one contiguous run per XCD
   const int bpc = xcd_chunk_rows == 0 ? 0 : chunk_bpc(n_blocks, xcd_chunk_rows > 0 ? std::max(1, xcd_chunk_rows / G) : 0);
-#define CALL2(V_, L_, COAL_)                                                                                   \
-  hipLaunchKernelGGL((spmm_rows_kernel<V_, L_, COAL_>), dim3(grid_chunked(n_blocks, bpc)), dim3(kBlock), 0, st, \
+#define CALL3(V_, L_, COAL_, FLAG_)                                                                                   \
+  hipLaunchKernelGGL((spmm_rows_kernel<V_, L_, COAL_, FLAG_>), dim3(grid_chunked(n_blocks, bpc)), dim3(kBlock), 0, st, \
                      rows, n_rows, n_blocks, bpc, Ap, Ai, Ax, X, N, Y, N, accumulate, streaming, compact)
+#define CALL2(V_, L_, COAL_) CALL3(V_, L_, COAL_, false)
 #define CALL(V_, L_) do { if (coalesced_pairs) { CALL2(V_, L_, true); } else { CALL2(V_, L_, false); } } while (0)
+#define CALLF(L_) do { if (coalesced_pairs) { CALL3(4, L_, true, true); } else { CALL3(4, L_, false, true); } } while (0)
+  if (flagged) {
+    if (s.LPR == 8) { CALLF(8); } else if (s.LPR == 16) { CALLF(16); } else if (s.LPR == 32) { CALLF(32); } else { CALLF(64); }
+    return hipGetLastError();
+  }
   TF_DISPATCH_VL(s.V, s.LPR, CALL);
 #undef CALL
 #undef CALL2
+#undef CALL3
+#undef CALLF
   return hipGetLastError();
 }
 
