@@ -33,6 +33,7 @@ import numpy as np  # noqa: E402
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 MFMA_FP32_PEAK_TF = 157.3  # MI355X dense fp32 MFMA, published
 LLC_BYTES = 256 << 20      # Infinity Cache
+L2_GATHER_TBS = 17.5       # the row kernel gathering 512-byte rows that every XCD finds in its own L2 (profiles/calibration_gather.md)
 METRIC = "fused GeMM-SpMM / SpMM-SpMM GFLOP/s and % HBM roofline, 1 MI355X vs CPU"
 HEADLINE = 4               # largest single-GPU configuration, the power-law target
 
@@ -181,6 +182,47 @@ def calibrate(tf, rows=1 << 20, N=128, reps=5):
                       "copy_GBps_read_plus_write": round(2 * rows * N * 4 / dt / 1e9, 1)}))
 
 
+def calibrate_gather(tf, rows=1 << 19, per_row=32, N=128, reps=5):
+    """The rate at which the row kernel (spmm_rows_kernel through tf_spmm) gathers 4N-byte rows when they are
+    found in L2, in the Infinity Cache, or nowhere: Y = A X with `per_row` random columns per row drawn from
+    (a) a region of 4 MB per XCD -- the row kernel deals workgroup b, i.e. rows 8b .. 8b+7 at N = 128, to XCD b mod 8,
+    and row i draws from region (i / 8) mod 8, so every XCD gathers from its own 4 MB;
+    (b) one region of 16 MB shared by all XCDs; (c) 1 GB.  gathered bytes = nnz * 4N; the rows of Y written
+    (rows * 4N, streaming stores) come on top and are 1/per_row of that."""
+    import scipy.sparse as sp
+    rng = np.random.default_rng(77)
+    out = {"calibration_kernel": "spmm_rows_kernel via tf_spmm", "rows": rows, "entries_per_row": per_row, "N": N, "launches": reps,
+           "gathered_bytes_per_launch": rows * per_row * 4 * N, "cases": []}
+    row_bytes = 4 * N
+    g = 256 // max(8, N // 4)  # rows per workgroup of the row kernel
+    cases = [("own 4 MB per XCD", 8 * (4 << 20) // row_bytes, lambda i: ((i // g) % 8) * ((4 << 20) // row_bytes), (4 << 20) // row_bytes),
+             ("one 16 MB for all XCDs", (16 << 20) // row_bytes, lambda i: 0 * i, (16 << 20) // row_bytes),
+             ("1 GB", (1 << 30) // row_bytes, lambda i: 0 * i, (1 << 30) // row_bytes)]
+    for name, x_rows, base, span in cases:
+        i = np.repeat(np.arange(rows), per_row)
+        cols = base(i) + rng.integers(0, span, size=rows * per_row)
+        A = sp.csr_matrix((np.ones(rows * per_row, np.float32), cols.astype(np.int32), np.arange(0, rows * per_row + 1, per_row, dtype=np.int32)),
+                          shape=(rows, x_rows))
+        Ah = tf.CsrMatrix.from_scipy(A).to_device()
+        X = tf.DenseMatrix(x_rows, N)
+        X.fill(1.0)
+        Y = tf.DenseMatrix(rows, N)
+        st = tf.Stream()
+        tf.spmm(Ah, X, Y, stream=st)
+        st.synchronize()
+        e0, e1 = tf.Event(), tf.Event()
+        e0.record(st)
+        for _ in range(reps):
+            tf.spmm(Ah, X, Y, stream=st)
+        e1.record(st)
+        st.synchronize()
+        ms = e0.elapsed_ms(e1) / reps
+        out["cases"].append({"gathers_from": name, "ms": round(ms, 4), "gather_TBps": round(rows * per_row * row_bytes / ms / 1e9, 2)})
+        del Ah, X, Y
+        gc.collect()
+    print(json.dumps(out))
+
+
 def check_result(cfg, got, max_rows=1 << 17):
     """max |got - want| / max |want| against float64, on every row or -- for the configurations with
     millions of rows -- on a fixed sample of rows that includes the longest ones."""
@@ -283,6 +325,18 @@ def run_config(tf, cfg, idx, steps, warmup, args):
     bound = "mfma" if t_mfma > t_hbm else "hbm"
     dev_s = dev_ms * 1e-3
     operand_bytes = alg_bytes + (4.0 * A.shape[1] * N if info["n_writeback_rows"] else 0.0)
+    # What was executed, beside the nominal work model: the GEMM of the intermediate rows the executor computes
+    # (halo rows recomputed by tiles count, rows nobody reads do not), their rows of B instead of all of B; and the
+    # bytes gathered through the caches by rows that did not fuse (4N per stored entry), which at the row kernel's
+    # measured rate out of L2 (profiles/calibration_gather.md) is a third roof for steps that gather.
+    computed = info["n_computed_rows"]
+    exe_gemm_flops = 2.0 * computed * K * N if gemm else 0.0
+    exe_bytes = alg_bytes - 4.0 * (A.shape[1] - computed) * K if gemm else alg_bytes
+    gathered = 4.0 * N * (A.nnz - info["fused_nnz"])
+    if not gemm and info["n_fused_rows"] == 0:
+        gathered += 4.0 * N * cfg["B"].nnz
+    t_exe = max(exe_bytes / (HBM_PEAK_GBS * 1e9), exe_gemm_flops / (MFMA_FP32_PEAK_TF * 1e12))
+    t_gather = gathered / (L2_GATHER_TBS * 1e12)
     res = {
         "cfg": idx, "workload": cfg["name"], "op": cfg["op"], "rows": int(A.shape[0]), "nnz": int(A.nnz), "N": N, "K": K,
         "ms_per_step": round(ms_per_step, 5), "kernel_ms": round(dev_ms, 5),
@@ -290,6 +344,11 @@ def run_config(tf, cfg, idx, steps, warmup, args):
         "bound": bound, "frac": round(max(t_hbm, t_mfma) / dev_s, 4),
         "hbm_frac": round(t_hbm / dev_s, 4), "mfma_frac": round(t_mfma / dev_s, 4) if gemm else None,
         "algorithmic_bytes": int(alg_bytes), "gemm_flops": int(gemm_flops), "flops": int(flops),
+        "executed": {"computed_intermediate_rows": int(computed), "gemm_flops": int(exe_gemm_flops), "bytes": int(exe_bytes),
+                     "bound": "mfma" if exe_gemm_flops / (MFMA_FP32_PEAK_TF * 1e12) > exe_bytes / (HBM_PEAK_GBS * 1e9) else "hbm",
+                     "frac": round(t_exe / dev_s, 4),
+                     "mfma_TFLOPs": round(exe_gemm_flops / dev_s / 1e12, 2) if gemm else None},
+        "gather": {"gathered_bytes": int(gathered), "l2_gather_TBps": L2_GATHER_TBS, "frac": round(t_gather / dev_s, 4)} if gathered else None,
         "working_set_vs_llc": round(operand_bytes / LLC_BYTES, 2),
         "rel_err_vs_f64": err, "rows_checked": rows_checked,
         "kernels": kernels, "kernel": kernel_names(info, gemm, args.unfused),
@@ -352,6 +411,8 @@ def main():
     ap.add_argument("--no-check", action="store_true", help="skip the result check")
     ap.add_argument("--calibrate", action="store_true",
                     help="run a copy of known size instead (scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--calibrate-gather", action="store_true",
+                    help="measure the row kernel's gather rate out of L2 / the Infinity Cache / HBM instead (the gather roof's rate)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
@@ -363,6 +424,9 @@ def main():
     dev = tf.device_init(0)
     if args.calibrate:
         calibrate(tf)
+        return
+    if args.calibrate_gather:
+        calibrate_gather(tf)
         return
     custom = bool(args.matrix or args.scramble or args.rcm or args.unfused)
     if args.matrix:
@@ -428,10 +492,14 @@ def main():
     else:
         roof = {"bound": "hbm", **hbm}
     roof.update({"traffic": head.get("traffic"), "algorithmic_bytes": head["algorithmic_bytes"], "gemm_flops": head["gemm_flops"],
+                 "executed": head["executed"], "gather": head["gather"],
                  "kernel_ms": head["kernel_ms"], "kernel": head["kernel"], "kernels": head["kernels"],
-                 "note": "a step is several launches: achieved = algorithmic work of the whole step / HIP-event time of the step on the "
-                         "launch stream; `kernels` = each launch timed by its own events in one extra step (launches on the "
-                         "executor's second stream run beside the others, so the list can add up to more than kernel_ms)"})
+                 "note": "a step is several launches: achieved = NOMINAL algorithmic work of the whole step (2 M K N for the GEMM, every row of B) / "
+                         "HIP-event time of the step on the launch stream; `executed` = the same fraction on the work the executor does "
+                         "(the GEMM only of intermediate rows some row of A reads, their rows of B); `gather` = bytes the unfused rows "
+                         "gather through the caches / the row kernel's measured rate out of L2, as a fraction of the step: what a "
+                         "formulation that gathers could reach at best; `kernels` = each launch timed by its own events in one extra "
+                         "step (launches on the executor's second stream run beside the others, so the list can add up to more than kernel_ms)"})
     if "traffic_source" in head:
         roof["traffic_source"] = head["traffic_source"]
     out["roofline"] = roof

@@ -251,6 +251,10 @@ typedef struct {
      0 = 8 MB when the long rows are column-partitioned (long_row_partition: a power-law graph), else off;
      -1 = off; n > 0 = n bytes.  Only when N is a multiple of 4, and only if the set takes a quarter of the reads. */
   int short_row_hot_bytes;
+  /* GeMM-SpMM schedules of a square matrix with K and N of 32, 64 or 128 also get two-layer tiles when the pattern
+     allows (every tile's halo of hidden rows and the halo of those fit LDS: banded or reordered patterns): what
+     tf_gcn_two_layers runs when the schedule serves as its second layer's.  0 = build them, -1 = do not. */
+  int two_layer_tiles;
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -342,6 +346,13 @@ typedef struct {
   const int *tile_step;
   const int *step_ptr;
   int n_step_ptr;
+  /* appended after the first version */
+  /* Two-layer tiles (tf_schedule_info.two_layer_tiles of them, else null / 0): two_layer_range[8*t + {0..5}] =
+     o0, o1, h0, h1, t0, t1: tile t owns the rows [o0, o1) of D, computes the hidden rows [h0, h1) they read and
+     the rows [t0, t1) of the first layer's intermediate those read ([8*t + 6] = floats of LDS its first slab takes,
+     [8*t + 7] unused). */
+  const int *two_layer_range;
+  int n_two_layer;
 } tf_schedule_view;
 
 tf_status tf_schedule_get_view(const tf_schedule *s, tf_schedule_view *view);
@@ -371,7 +382,11 @@ enum {
                            another -- which measured as fast on the R-MAT configuration (2.32 ms
                            against 2.35 ms: the gathers and the GEMM's operand traffic meet in the
                            same memory system), so it is not the default */
-  TF_RELU = 4u           /* tf_gcn_two_layers: ReLU between the layers */
+  TF_RELU = 4u,          /* tf_gcn_two_layers: ReLU between the layers */
+  TF_FUSE_LAYERS = 8u,   /* tf_gcn_two_layers: run the second schedule's two-layer tiles (one launch, the hidden
+                           layer never leaves LDS) or fail with TF_EUNSUPPORTED if it has none; without this flag
+                           they run when they recompute little (see tf_gcn_two_layers)                      */
+  TF_COMPOSE_LAYERS = 16u /* tf_gcn_two_layers: never the two-layer tiles: one tf_gemm_spmm per layer        */
 };
 
 /* D = A * (B * C), A and B sparse.  Stands in for
@@ -397,10 +412,18 @@ tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf
  * layers with a ReLU between).  A is square (M x M), X is M x K, W1 is K x H, W2 is H x N (weights not
  * transposed, as in tf_gemm_spmm), D is M x N.  s1 must come from tf_inspect on A's pattern for
  * (TF_OP_GEMM_SPMM, K, H), s2 for (TF_OP_GEMM_SPMM, H, N); they may be one schedule when K = H = N.
- * The hidden layer stays on the device: in `hidden` (M x H) when given -- training keeps it for the
- * backward pass -- else in a buffer that s2 owns.  Each layer runs as tf_gemm_spmm does, so rows fuse
- * inside a layer; no tile carries a row through both layers (a row of the second layer needs the whole
- * neighbourhood of its neighbours from the first).  The reference's fusedGCN reads its second GEMM's input
+ * The hidden layer stays on the device.  Two ways to run, chosen per call:
+ *  - two-layer tiles (fused_gcn2_kernel; the reference's "four kernels per tile", MixPtr[4j .. 4j+3] at Functions.cpp:
+ *    228-290): when s2 carries them (tf_schedule_info.two_layer_tiles > 0: a square matrix whose rows' halos fit LDS
+ *    -- banded or reordered patterns -- and H, N of 32, 64 or 128), K is a multiple of 8 up to 256 and `hidden` is
+ *    null, ONE launch takes every tile through GEMM, SpMM, activation, GEMM, SpMM with the first intermediate, the
+ *    hidden rows and the second intermediate in LDS; only X, the weights, A and D cross HBM.  A tile recomputes the
+ *    halo rows of its neighbours: this path is taken by default when that costs at most 1.3x the GEMM rows of
+ *    the composed path, always with TF_FUSE_LAYERS, never with TF_COMPOSE_LAYERS;
+ *  - composed: each layer runs as tf_gemm_spmm does with its own schedule (rows fuse inside a layer), the hidden
+ *    layer in `hidden` (M x H) when given -- training keeps it for the backward pass -- else in a buffer that s2
+ *    owns, one small ReLU launch between the layers.
+ * The reference's fusedGCN reads its second GEMM's input
  * from the first GEMM's output instead of from the first layer's (imRes1 at :262) and has no activation;
  * this entry point computes the composition its callers mean. */
 tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const tf_dense *W1, const tf_dense *W2, tf_dense *D,

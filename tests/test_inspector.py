@@ -532,3 +532,79 @@ def test_short_rows_mark_their_cold_gathers_on_power_law_graphs(tf):
     S = tf.inspector(Eh, 1, op=tf.OP_GEMM_SPMM, N=128, K=256, short_row_hot_bytes=256 << 10)   # 512 of 10,000 rows
     S.validate()
     assert S.info()["short_row_hot_rows"] == 0
+
+
+# ---- two-layer tiles -------------------------------------------------------------------------------------------
+
+def _check_two_layer_tiles(A, rng6, H, N):
+    """Independent of the library: owned ranges partition the rows in order; every owned row reads hidden rows of
+    its tile only, every hidden row of the tile rows of the first intermediate the tile computes; slabs fit LDS."""
+    M = A.shape[0]
+    end = 0
+    for o0, o1, h0, h1, t0, t1 in rng6:
+        assert o0 == end and o1 > o0
+        end = o1
+        cols = A.indices[A.indptr[o0]:A.indptr[o1]]
+        if len(cols):
+            assert cols.min() >= h0 and cols.max() < h1
+        hc = A.indices[A.indptr[h0]:A.indptr[h1]] if h1 > h0 else np.zeros(0, int)
+        if len(hc):
+            assert hc.min() >= t0 and hc.max() < t1
+        a = max((t1 - t0) * (H + 4), (h1 - h0) * (N + 4))
+        b = max((h1 - h0) * (H + 4), 2 * 64 * 36)
+        assert (a + b) * 4 <= 163840
+    assert end == M
+
+
+def test_two_layer_tiles_on_banded_patterns(tf):
+    """GeMM-SpMM schedules of a banded matrix carry two-layer tiles (what tf_gcn_two_layers runs when the schedule
+    is its second layer's): exact ranges on a band of half-width 16, for the widths the kernel is built for; the
+    library's validator and an independent one agree; patterns without a band, other widths and the opt-out get none."""
+    M = 6000
+    A = tf.workloads.banded_random(M, 32, 16, seed=3)
+    for H, N in ((128, 128), (64, 64), (128, 64), (32, 128)):
+        S, view, info = inspect(tf, A, op=tf.OP_GEMM_SPMM, N=N, K=H, compute_units=16)
+        assert info["two_layer_tiles"] > 0 and len(view["two_layer_range"]) == info["two_layer_tiles"]
+        _check_two_layer_tiles(A, view["two_layer_range"], H, N)
+        r = view["two_layer_range"]
+        inner = r[1:-1]
+        # a band of half-width 16: hidden halo of at most 16 rows a side, the first intermediate's 16 more
+        assert np.all(inner[:, 0] - inner[:, 2] <= 16) and np.all(inner[:, 3] - inner[:, 1] <= 16)
+        assert np.all(inner[:, 2] - inner[:, 4] <= 16) and np.all(inner[:, 5] - inner[:, 3] <= 16)
+        assert np.all(inner[:, 1] - inner[:, 0] >= 32)
+    # widths the kernel is not built for, the opt-out, a pattern whose halos no LDS holds
+    assert inspect(tf, A, op=tf.OP_GEMM_SPMM, N=96, K=128)[2]["two_layer_tiles"] == 0
+    assert inspect(tf, A, op=tf.OP_GEMM_SPMM, N=128, K=40)[2]["two_layer_tiles"] == 0
+    assert inspect(tf, A, op=tf.OP_GEMM_SPMM, N=128, K=128, two_layer_tiles=-1)[2]["two_layer_tiles"] == 0
+    er = tf.workloads.make_config(3, 0.05)["A"]
+    assert inspect(tf, er, op=tf.OP_GEMM_SPMM, N=128, K=128)[2]["two_layer_tiles"] == 0
+    # rows without entries, and a 2D grid (halo of a grid line a side)
+    L2 = tf.workloads.laplacian_2d(40)
+    S, view, info = inspect(tf, L2, op=tf.OP_GEMM_SPMM, N=64, K=64, compute_units=8)
+    assert info["two_layer_tiles"] > 0
+    _check_two_layer_tiles(L2, view["two_layer_range"], 64, 64)
+    E = sp.csr_matrix(sp.diags(np.r_[np.zeros(300), np.ones(M - 300)].astype(np.float32)) @ A)
+    E.eliminate_zeros(); E.sort_indices()
+    E = sp.csr_matrix((E.data.astype(np.float32), E.indices.astype(np.int32), E.indptr.astype(np.int32)), shape=E.shape)
+    S, view, info = inspect(tf, E, op=tf.OP_GEMM_SPMM, N=64, K=64, compute_units=16)
+    assert info["two_layer_tiles"] > 0
+    _check_two_layer_tiles(E, view["two_layer_range"], 64, 64)
+
+
+def test_two_layer_tiles_are_validated_against_the_pattern(tf):
+    """The validator replays the two-layer tiles too: a pattern with one column moved out of a tile's halo is refused."""
+    M = 3000
+    A = tf.workloads.banded_random(M, 32, 16, seed=3)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=64, K=64, compute_units=16, lds_budget_bytes=163840, tile_rows=3000, max_redundancy=1.0)
+    assert S.info()["two_layer_tiles"] > 1
+    S.validate()
+    r = S.view()["two_layer_range"]
+    o0, o1, h0, h1, t0, t1 = r[1]
+    B = A.copy(); B.indices = B.indices.copy()
+    row = (o0 + o1) // 2
+    B.indices[B.indptr[row]] = max(0, h0 - 40)          # an owned row now reads a hidden row the tile does not compute
+    B.has_sorted_indices = False
+    with pytest.raises(tf.TileFusionError) as e:
+        S.validate(tf.CsrMatrix.from_scipy(B))
+    assert e.value.status == -4

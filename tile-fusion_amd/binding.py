@@ -14,6 +14,8 @@ OP_GEMM_SPMM = 1
 ACCUMULATE = 1
 SECOND_STREAM = 2
 RELU = 4
+FUSE_LAYERS = 8
+COMPOSE_LAYERS = 16
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -41,7 +43,7 @@ class InspectOpts(C.Structure):
                 ("inner_cols", C.c_int), ("strip_cols", C.c_int), ("xcd_chunk_rows", C.c_int), ("wide_strips", C.c_int), ("long_row_partition", C.c_int),
                 ("march", C.c_int), ("grid_nx", C.c_int), ("grid_ny", C.c_int), ("grid_nz", C.c_int),
                 ("march_tile_x", C.c_int), ("march_tile_y", C.c_int), ("reorder_adjacency", C.c_int), ("hot_partition_bytes", C.c_int),
-                ("short_row_hot_bytes", C.c_int)]
+                ("short_row_hot_bytes", C.c_int), ("two_layer_tiles", C.c_int)]
 
 
 class ScheduleInfo(C.Structure):
@@ -63,7 +65,8 @@ class ScheduleView(C.Structure):
                 ("ker_begin", C.POINTER(C.c_int)), ("id", C.POINTER(C.c_int)),
                 ("type", C.POINTER(C.c_int)), ("tile_range", C.POINTER(C.c_int)),
                 ("writeback", C.POINTER(C.c_int)), ("tile_step", C.POINTER(C.c_int)),
-                ("step_ptr", C.POINTER(C.c_int)), ("n_step_ptr", C.c_int)]
+                ("step_ptr", C.POINTER(C.c_int)), ("n_step_ptr", C.c_int),
+                ("two_layer_range", C.POINTER(C.c_int)), ("n_two_layer", C.c_int)]
 
 
 PROFILE_MAX = 16
@@ -325,7 +328,8 @@ class FusedSchedule:
                 "tile_range": arr(v.tile_range, 4 * nt).reshape(nt, 4),
                 "writeback": arr(v.writeback, 2 * nt).reshape(nt, 2),
                 "tile_step": arr(v.tile_step, nt) if v.n_step_ptr else None,
-                "step_ptr": arr(v.step_ptr, v.n_step_ptr) if v.n_step_ptr else None}
+                "step_ptr": arr(v.step_ptr, v.n_step_ptr) if v.n_step_ptr else None,
+                "two_layer_range": arr(v.two_layer_range, 8 * v.n_two_layer).reshape(-1, 8)[:, :6] if v.n_two_layer else None}
 
     def validate(self, A=None):
         """Exact check against the pattern (and the inner pattern, when the schedule was built with one)."""
@@ -351,7 +355,7 @@ class FusedSchedule:
 
 def inspector(A, NumThreads=1, *, op, N, K=0, lds_budget_bytes=0, tile_rows=0, max_redundancy=0.0,
               long_row_nnz=0, compute_units=0, inner=None, strip_cols=0, xcd_chunk_rows=0, wide_strips=0, long_row_partition=0,
-              march=0, grid=None, march_tile=None, reorder_adjacency=0, hot_partition_bytes=0, short_row_hot_bytes=0):
+              march=0, grid=None, march_tile=None, reorder_adjacency=0, hot_partition_bytes=0, short_row_hot_bytes=0, two_layer_tiles=0):
     """swiftware::fusion::inspector(A, NumThreads) (README.md:25).  NumThreads is accepted
     for signature parity and unused: the schedule is sized by the GPU, not by a CPU
     thread count.  The extra keywords are the parameters the reference passes to its
@@ -362,7 +366,7 @@ def inspector(A, NumThreads=1, *, op, N, K=0, lds_budget_bytes=0, tile_rows=0, m
     o = InspectOpts(C.sizeof(InspectOpts), op, N, K, lds_budget_bytes, tile_rows, max_redundancy, long_row_nnz, compute_units,
                     inner._pp if inner is not None else None, inner._pi if inner is not None else None,
                     inner.N if inner is not None else 0, strip_cols, xcd_chunk_rows, wide_strips, long_row_partition,
-                    march, *(grid or (0, 0, 0)), *(march_tile or (0, 0)), reorder_adjacency, hot_partition_bytes, short_row_hot_bytes)
+                    march, *(grid or (0, 0, 0)), *(march_tile or (0, 0)), reorder_adjacency, hot_partition_bytes, short_row_hot_bytes, two_layer_tiles)
     h = _VP()
     _check(lib().tf_inspect(A.M, A.N, A._pp, A._pi, C.byref(o), C.byref(h)))
     return FusedSchedule(h, A, inner)
@@ -384,11 +388,12 @@ def gemm_spmm(A, B, Cm, D, schedule, NumThreads=1, *, accumulate=False, stream=N
                               stream.h if stream else None))
 
 
-def gcn_two_layers(A, X, W1, W2, D, s1, s2, *, relu=True, hidden=None, accumulate=False, stream=None):
+def gcn_two_layers(A, X, W1, W2, D, s1, s2, *, relu=True, hidden=None, accumulate=False, stream=None, fuse=None):
     """D = A * (act(A * (X * W1)) * W2), the two-layer forward of the reference's end-to-end model
     (binding-project/gcn-e2e-training/FusedGCNModule.py:14-18); the hidden layer stays on the device."""
     _check(lib().tf_gcn_two_layers(A.to_device().h, X.h, W1.h, W2.h, D.h, s1.h, s2.h, hidden.h if hidden is not None else None,
-                                   (RELU if relu else 0) | (ACCUMULATE if accumulate else 0), stream.h if stream else None))
+                                   (RELU if relu else 0) | (ACCUMULATE if accumulate else 0) |
+                                   (FUSE_LAYERS if fuse is True else COMPOSE_LAYERS if fuse is False else 0), stream.h if stream else None))
 
 
 def spmm_spmm_noalloc(A, B, Cm, D, *, accumulate=False, stream=None):

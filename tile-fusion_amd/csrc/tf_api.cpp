@@ -56,6 +56,7 @@ struct DeviceSchedule {
   int *rem_ptr = nullptr, *rem_col = nullptr, *rem_src = nullptr;
   float *rem_val = nullptr;
   unsigned long long rem_val_serial = 0;
+  Tile2 *l2_tiles = nullptr; // two-layer tiles
   float *hidden = nullptr;   // tf_gcn_two_layers: the first layer's output, L x K of this (second-layer) schedule
   size_t hidden_floats = 0;
   float *Bpad = nullptr;     // M x K' and K' x N copies of B and C, zero-padded, when K is not a multiple of 8
@@ -108,8 +109,14 @@ hipError_t launch_fill(float *, size_t, float, hipStream_t);
 hipError_t launch_pad(const float *, int, int, float *, int, int, hipStream_t);
 hipError_t launch_copy_cols(const float *, int, int, int, int, float *, int, int, int, int, int, hipStream_t);
 hipError_t launch_relu(float *, size_t, hipStream_t);
+hipError_t launch_fused_gcn2(const Tile2 *, int, const float *, const float *, const float *, int, int, int, const int *, const int *,
+                             const float *, float *, int, int, int, hipStream_t);
 hipError_t launch_zero_rows(const int *, int, float *, int, hipStream_t);
 hipError_t launch_xcd_probe(int *, int, hipStream_t);
+
+// (GEMM rows computed by two-layer tiles) / (GEMM rows of the two layers computed once) up to which the tiles
+// are the default of tf_gcn_two_layers
+constexpr double kTwoLayerMaxWork = 1.3;
 
 // An intermediate larger than the 256 MB last-level cache is gone from it before its readers
 // come: such rows leave through streaming stores.
@@ -152,7 +159,7 @@ void release_device_schedule(DeviceSchedule *d) {
   (void)hipFree(d->long_chunks); (void)hipFree(d->long_rows); (void)hipFree(d->seg_groups);
   (void)hipFree(d->seg_ptr); (void)hipFree(d->ent_src); (void)hipFree(d->ent_pos); (void)hipFree(d->seg_col); (void)hipFree(d->lrow_seg); (void)hipFree(d->seg_val);
   (void)hipFree(d->step_begin); (void)hipFree(d->step_ptr); (void)hipFree(d->fused_rec);
-  (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad); (void)hipFree(d->Cpanel); (void)hipFree(d->Dpanel); (void)hipFree(d->hidden);
+  (void)hipFree(d->inter); (void)hipFree(d->partial); (void)hipFree(d->Bpad); (void)hipFree(d->Cpad); (void)hipFree(d->Cpanel); (void)hipFree(d->Dpanel); (void)hipFree(d->hidden); (void)hipFree(d->l2_tiles);
   (void)hipFree(d->rem_ptr); (void)hipFree(d->rem_col); (void)hipFree(d->rem_src); (void)hipFree(d->rem_val);
   (void)hipFree(d->m_runs); (void)hipFree(d->m_row_ptr); (void)hipFree(d->m_load_ptr); (void)hipFree(d->m_load);
   (void)hipFree(d->m_row_out); (void)hipFree(d->m_ell_off); (void)hipFree(d->m_ell_src); (void)hipFree(d->m_ell); (void)hipFree(d->m_trash);
@@ -207,6 +214,7 @@ static tf_status ensure_device(tf_schedule *s) {
     return TF_OK;
   }
   rc = upload_vec(s->launch_tiles, &d->tiles);
+  if (!rc) rc = upload_vec(s->l2_tiles, &d->l2_tiles);
   if (!rc) rc = upload_vec(s->fused_ids, &d->fused_ids);
   if (!rc) rc = upload_vec(s->win, &d->win);
   if (!rc) rc = upload_vec(s->rem_rows, &d->rem_rows);
@@ -365,6 +373,15 @@ static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int
                               (int)s->long_rows.size(), A->i, A->x, d->inter, d->partial, D->d, N,
                               accumulate, st));
   return TF_OK;
+}
+
+// Whether tf_gcn_two_layers runs a schedule's two-layer tiles without being asked to (TF_FUSE_LAYERS): when they
+// recompute little.  A tile computes (t1 - t0) rows of the first GEMM and (h1 - h0) of the second for (o1 - o0)
+// rows it owns; the composed path computes each row once per layer but moves the hidden layer through HBM twice.
+static bool two_layer_tiles_pay(const tf_schedule *s) {
+  long long own = 0, work = 0;
+  for (const auto &t : s->l2_tiles) { own += t.o1 - t.o0; work += (t.t1 - t.t0) + (t.h1 - t.h0); }
+  return own > 0 && work <= (long long)(kTwoLayerMaxWork * 2.0 * own);
 }
 
 }  // namespace tf
@@ -833,6 +850,24 @@ extern "C" tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const
     return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the first schedule was built for K = %d, X is %d x %d and W1 has %d rows", s1->user_K, X->M, X->N, W1->M);
   if (W2->N != s2->user_N || D->N != s2->user_N || D->M != A->M)
     return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule was built for N = %d, W2 has %d columns and D is %d x %d", s2->user_N, W2->N, D->M, D->N);
+  // One launch with the hidden layer in LDS, when the second schedule has two-layer tiles and the caller does not
+  // want the hidden layer back: every tile carries its rows through both layers (fused_gcn2_kernel).
+  const bool fuse_ok = !hidden && !s2->l2_tiles.empty() && s1->user_K == s1->opts.K && s1->user_K <= 256 && !(flags & TF_COMPOSE_LAYERS);
+  if ((flags & TF_FUSE_LAYERS) && !fuse_ok)
+    return fail(TF_EUNSUPPORTED, "tf_gcn_two_layers: TF_FUSE_LAYERS needs a second schedule with two-layer tiles (tf_schedule_info.two_layer_tiles: "
+                "a banded pattern, widths of 32, 64 or 128), K a multiple of 8 up to 256 and no `hidden` argument");
+  if (fuse_ok && ((flags & TF_FUSE_LAYERS) || tf::two_layer_tiles_pay(s2))) {
+    if (A->nnz != s2->nnz || (A->hash && A->hash != s2->pattern_hash))
+      return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule was built for another sparsity pattern than A's");
+    if (tf_status rc = tf::ensure_device(s2)) return rc;
+    tf::DeviceSchedule *d = s2->dev;
+    d->prof_n = 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    TF_PHASE(s2, "fused_gcn2_kernel", st,
+             tf::launch_fused_gcn2(d->l2_tiles, (int)s2->l2_tiles.size(), X->d, W1->d, W2->d, s1->user_K, H, s2->user_N, A->p, A->i, A->x,
+                                   D->d, s2->l2_lds_bytes, (flags & TF_RELU) ? 1 : 0, (flags & TF_ACCUMULATE) ? 1 : 0, st));
+    return TF_OK;
+  }
   tf_dense h;
   h.M = A->M; h.N = H; h.owns = false;
   if (hidden) {

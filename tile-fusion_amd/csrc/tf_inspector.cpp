@@ -25,6 +25,55 @@ constexpr int kMaxLds = 163840;  // LDS per workgroup on gfx950
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+
+// Two-layer tiles for tf_gcn_two_layers (see tf_internal.h: Tile2, and tf_gcn2.hip).  Greedy: a tile's owned
+// range grows row by row while the two slabs its halos need fit `budget_floats` of LDS.  H = the hidden width
+// (this schedule's K), N its output width.  Leaves S->l2_tiles empty when some single row's halos do not fit
+// (a pattern without a band: the composed path serves it).
+void build_two_layer_tiles(tf_schedule *S, int M, const int *Ap, const int *Ai, int H, int N, int compute_units) {
+  const long long budget_floats = kMaxLds / 4;
+  std::vector<int> lo(M), hi(M);  // column extent per row: [lo, hi), empty rows lo = INT_MAX, hi = -1
+  for (int i = 0; i < M; ++i) {
+    int a = INT_MAX, b = -1;
+    for (int k = Ap[i]; k < Ap[i + 1]; ++k) { a = std::min(a, Ai[k]); b = std::max(b, Ai[k] + 1); }
+    lo[i] = a; hi[i] = b;
+  }
+  const int cap = std::max(32, ceil_div(M, std::max(1, compute_units)));
+  std::vector<tf::Tile2> tiles;
+  long long max_floats = 0;
+  for (int o0 = 0; o0 < M;) {
+    int h0 = INT_MAX, h1 = -1, t0 = INT_MAX, t1 = -1, o1 = o0;
+    long long fa = 0, fb = tf::kTile2StageFloats;
+    while (o1 < M && o1 - o0 < cap) {
+      const int nh0 = std::min(h0, lo[o1]), nh1 = std::max(h1, hi[o1]);
+      int nt0 = t0, nt1 = t1;
+      if (nh1 > nh0) {  // hidden rows that the new row adds on either side
+        const int left_end = h1 > h0 ? h0 : nh1;
+        for (int j = nh0; j < left_end; ++j) { nt0 = std::min(nt0, lo[j]); nt1 = std::max(nt1, hi[j]); }
+        if (h1 > h0)
+          for (int j = h1; j < nh1; ++j) { nt0 = std::min(nt0, lo[j]); nt1 = std::max(nt1, hi[j]); }
+      }
+      const long long PH = std::max(0, nh1 - nh0), P1 = std::max(0, nt1 - nt0);
+      const long long a = std::max(P1 * (H + tf::kTile2Pad), PH * (N + tf::kTile2Pad));
+      const long long b = std::max<long long>(PH * (H + tf::kTile2Pad), tf::kTile2StageFloats);
+      if (a + b > budget_floats) break;
+      h0 = nh0; h1 = nh1; t0 = nt0; t1 = nt1; fa = a; fb = b;
+      ++o1;
+    }
+    if (o1 == o0) return;  // one row alone does not fit
+    tf::Tile2 t{};
+    t.o0 = o0; t.o1 = o1;
+    t.h0 = h1 > h0 ? h0 : 0; t.h1 = h1 > h0 ? h1 : 0;
+    t.t0 = t1 > t0 ? t0 : 0; t.t1 = t1 > t0 ? t1 : 0;
+    t.b_off = (int)fa;
+    tiles.push_back(t);
+    max_floats = std::max(max_floats, fa + fb);
+    o0 = o1;
+  }
+  S->l2_tiles.swap(tiles);
+  S->l2_lds_bytes = (int)(max_floats * 4);
+}
+
 }  // namespace
 
 // Multiply-xorshift over the row pointers and column indices; 0 is kept for "unknown".
@@ -685,6 +734,12 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
     S->lds_bytes_general = gemm_stream ? stream_fixed + ring_rows * (o.N + 4) * 4 : slab_rows * row_bytes + staging;
     if (!windowed) S->lds_bytes = S->lds_bytes_general;
 
+    // Tiles that carry their rows through two layers, for when this is the second layer's schedule of
+    // tf_gcn_two_layers (hidden width = this K, output width = this N).
+    if (o.op == TF_OP_GEMM_SPMM && L == M && n_panels == 1 && user_K == o.K && o.two_layer_tiles >= 0 &&
+        (o.K == 32 || o.K == 64 || o.K == 128) && (o.N == 32 || o.N == 64 || o.N == 128))
+      build_two_layer_tiles(S, M, Ap, Ai, o.K, o.N, o.compute_units);
+
     // MultiDimensionalSet-layout view (Fusion_Inspector.h:959-1010).
     const int nt = (int)S->tiles.size();
     std::vector<int> rem_all;
@@ -775,7 +830,7 @@ extern "C" tf_status tf_schedule_get_info(const tf_schedule *s, tf_schedule_info
   info->march_declined = s->march_declined;
   info->register_weights = s->gemm_regw ? 1 : 0;
   info->n_zero_rows = (int)s->zero_rows.size();
-  info->two_layer_tiles = 0;
+  info->two_layer_tiles = (int)s->l2_tiles.size();
   info->short_row_hot_rows = s->rem_hot_rows;
   {
     long long computed = (long long)s->plain_rows.size();
@@ -811,6 +866,8 @@ extern "C" tf_status tf_schedule_get_view(const tf_schedule *s, tf_schedule_view
   v->tile_step = s->gemm_stream ? s->tile_step.data() : nullptr;
   v->step_ptr = s->gemm_stream ? s->view_step_ptr.data() : nullptr;
   v->n_step_ptr = s->gemm_stream ? (int)s->view_step_ptr.size() : 0;
+  v->two_layer_range = s->l2_tiles.empty() ? nullptr : &s->l2_tiles[0].o0;
+  v->n_two_layer = (int)s->l2_tiles.size();
   return tf::emit_out("tf_schedule_get_view", caller, full, TF_SIZE_THROUGH(tf_schedule_view, n_step_ptr));
 }
 
@@ -980,6 +1037,32 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
   }
   for (int i = 0; i < L; ++i)
     if (done[i] != 1) return tf::fail(TF_ESCHEDULE, "second-op row %d scheduled %d times", i, done[i]);
+  // Two-layer tiles: the owned ranges partition the rows in order; every owned row reads only hidden rows of its
+  // tile, every hidden row of a tile only rows of the first intermediate that the tile computes; both slabs fit.
+  if (!s->l2_tiles.empty()) {
+    const int H = s->opts.K, N2 = s->opts.N;
+    if (L != M) return tf::fail(TF_ESCHEDULE, "two-layer tiles on a matrix that is not square");
+    if (s->l2_lds_bytes > kMaxLds) return tf::fail(TF_ESCHEDULE, "two-layer tiles: %d bytes of LDS", s->l2_lds_bytes);
+    int end = 0;
+    for (size_t ti = 0; ti < s->l2_tiles.size(); ++ti) {
+      const tf::Tile2 &t = s->l2_tiles[ti];
+      if (t.o0 != end || t.o1 <= t.o0 || t.o1 > L) return tf::fail(TF_ESCHEDULE, "two-layer tile %zu owns [%d, %d) after row %d", ti, t.o0, t.o1, end);
+      end = t.o1;
+      if (t.h0 < 0 || t.h1 < t.h0 || t.h1 > M || t.t0 < 0 || t.t1 < t.t0 || t.t1 > M)
+        return tf::fail(TF_ESCHEDULE, "two-layer tile %zu: bad ranges", ti);
+      const long long PH = t.h1 - t.h0, P1 = t.t1 - t.t0, b_floats = s->l2_lds_bytes / 4 - t.b_off;
+      if (t.b_off < 0 || (t.b_off & 3) || P1 * (H + tf::kTile2Pad) > t.b_off || PH * (N2 + tf::kTile2Pad) > t.b_off ||
+          PH * (H + tf::kTile2Pad) > b_floats || tf::kTile2StageFloats > b_floats)
+        return tf::fail(TF_ESCHEDULE, "two-layer tile %zu: %lld hidden and %lld intermediate rows do not fit its slabs", ti, PH, P1);
+      for (int i = t.o0; i < t.o1; ++i)
+        for (int k = Ap[i]; k < Ap[i + 1]; ++k)
+          if (Ai[k] < t.h0 || Ai[k] >= t.h1) return tf::fail(TF_ESCHEDULE, "two-layer tile %zu: row %d reads hidden row %d outside [%d, %d)", ti, i, Ai[k], t.h0, t.h1);
+      for (int j = t.h0; j < t.h1; ++j)
+        for (int k = Ap[j]; k < Ap[j + 1]; ++k)
+          if (Ai[k] < t.t0 || Ai[k] >= t.t1) return tf::fail(TF_ESCHEDULE, "two-layer tile %zu: hidden row %d reads row %d outside [%d, %d)", ti, j, Ai[k], t.t0, t.t1);
+    }
+    if (end != L) return tf::fail(TF_ESCHEDULE, "two-layer tiles end at row %d of %d", end, L);
+  }
   return TF_OK;
 }
 

@@ -35,6 +35,17 @@ struct LongRow {
   int row, first, count, pad;
 };
 
+// A tile that carries its rows through two GCN layers (tf_gcn_two_layers): it owns the rows [o0, o1) of D, which
+// read the rows [h0, h1) of the hidden layer, which read the rows [t0, t1) of the first layer's intermediate.
+struct Tile2 {
+  int o0, o1, h0, h1, t0, t1;
+  int b_off;  // floats of LDS in front of the tile's slab B (its slab A: the first intermediate, then the second)
+  int pad;
+};
+static_assert(sizeof(Tile2) == 32, "Tile2 is read as two int4 by the kernel");
+constexpr int kTile2Pad = 4;                 // floats behind every slab row (tf_gcn2.hip: kG2Pad)
+constexpr int kTile2StageFloats = 2 * 64 * 36;  // the two staging buffers of X (tf_gcn2.hip: kG2StageFloats)
+
 struct DeviceSchedule;  // device copies + workspace, defined in tf_api.cpp
 
 // Marching runs: LDS layout and list format shared by the inspector, the validator and the kernel.
@@ -141,6 +152,11 @@ struct tf_schedule {
   std::vector<int> march_ell_off;    // [kMarchW per ELL row] LDS byte offset of the row read (the zero row for padding)
   std::vector<int> march_ell_src;    // ... and where its value comes from: index into B's values, or into A's
                                      // with kMarchSrcA set; -1 for padding (value 0)
+  // Two-layer tiles (GeMM-SpMM schedules of a square matrix with K and N of 32, 64 or 128, when every tile's two
+  // halos fit LDS): what tf_gcn_two_layers runs when this is the second layer's schedule.  l2_lds_bytes: the LDS
+  // of the fullest tile (slab A in front, slab B -- X staging, then the hidden rows -- behind it).
+  std::vector<tf::Tile2> l2_tiles;
+  int l2_lds_bytes = 0;
   long long fused_nnz = 0;
   int n_writeback_rows = 0;
   long long n_producer_rows = 0;
