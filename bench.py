@@ -223,12 +223,15 @@ def calibrate_gather(tf, rows=1 << 19, per_row=32, N=128, reps=5):
     print(json.dumps(out))
 
 
-def check_result(cfg, got, max_rows=1 << 17):
+def check_result(cfg, got, max_rows=1 << 17, W2=None):
     """max |got - want| / max |want| against float64, on every row or -- for the configurations with
-    millions of rows -- on a fixed sample of rows that includes the longest ones."""
+    millions of rows -- on a fixed sample of rows that includes the longest ones.  W2: the second layer's
+    weights, for a two-layer step (ReLU between the layers)."""
     A = cfg["A"]
     L = A.shape[0]
     t = cfg["B"].astype(np.float64) @ cfg["C"].astype(np.float64)
+    if W2 is not None:
+        t = np.maximum(A.astype(np.float64) @ t, 0.0) @ W2.astype(np.float64)
     if L <= max_rows:
         rows = None
         want = A.astype(np.float64) @ t
@@ -284,6 +287,13 @@ def run_config(tf, cfg, idx, steps, warmup, args):
         if args.unfused:  # the two products as separate launches, the intermediate through HBM
             T = tf.DenseMatrix(A.shape[1], N)
             step = lambda st: (tf.gemm(Bd, Cd, T, stream=st), tf.spmm(Ah, T, D, stream=st))  # noqa: E731
+        if args.two_layers:  # D = A (relu(A (B C)) W2): tf_gcn_two_layers, one schedule for both layers (K = N)
+            if K != N or A.shape[0] != A.shape[1]:
+                sys.exit("bench.py --two-layers: needs a square matrix and K = N (e.g. --config 6)")
+            W2 = w.uniform((N, N), 14)
+            W2d = tf.DenseMatrix.from_numpy(W2)
+            fuse = args.two_layers == "fuse"
+            step = lambda st: tf.gcn_two_layers(Ah, Bd, Cd, W2d, D, S, S, relu=True, fuse=fuse, stream=st)  # noqa: E731
 
     st = tf.Stream()
     for _ in range(warmup):
@@ -312,7 +322,7 @@ def run_config(tf, cfg, idx, steps, warmup, args):
 
     err, rows_checked = (None, 0)
     if not args.no_check:
-        err, rows_checked = check_result(cfg, D.to_numpy())
+        err, rows_checked = check_result(cfg, D.to_numpy(), W2=W2 if (gemm and args.two_layers) else None)
         if not err <= 1e-4:
             print(f"bench.py: result check failed on {cfg['name']}, rel err {err:.3e}", file=sys.stderr)
             sys.exit(1)
@@ -320,6 +330,9 @@ def run_config(tf, cfg, idx, steps, warmup, args):
     flops = w.flops(cfg)
     alg_bytes = w.algorithmic_bytes(cfg)
     gemm_flops = 2.0 * A.shape[1] * K * N if gemm else 0.0
+    if gemm and args.two_layers:  # both layers; compulsory bytes: the hidden layer never leaves the chip, A is read once
+        flops, gemm_flops = 2.0 * flops, 2.0 * gemm_flops
+        alg_bytes += 4.0 * N * N
     t_hbm = alg_bytes / (HBM_PEAK_GBS * 1e9)
     t_mfma = gemm_flops / (MFMA_FP32_PEAK_TF * 1e12)
     bound = "mfma" if t_mfma > t_hbm else "hbm"
@@ -351,7 +364,8 @@ def run_config(tf, cfg, idx, steps, warmup, args):
         "gather": {"gathered_bytes": int(gathered), "l2_gather_TBps": L2_GATHER_TBS, "frac": round(t_gather / dev_s, 4)} if gathered else None,
         "working_set_vs_llc": round(operand_bytes / LLC_BYTES, 2),
         "rel_err_vs_f64": err, "rows_checked": rows_checked,
-        "kernels": kernels, "kernel": kernel_names(info, gemm, args.unfused),
+        "kernels": kernels, "kernel": ("fused_gcn2_kernel" if args.two_layers == "fuse" else "2 x " + kernel_names(info, gemm, False) + " + relu_kernel")
+        if (gemm and args.two_layers) else kernel_names(info, gemm, args.unfused),
         "schedule": {"lds_bytes": info["lds_bytes"], "windowed": bool(info["windowed"]), "wide_strips": bool(info["wide_strips"]),
                      "streamed": bool(info["streamed"]), "marched": bool(info["marched"]), "tiles": info["n_tiles"], "fused_rows": info["n_fused_rows"],
                      "remainder_rows": info["n_remainder_rows"], "long_rows": info["n_long_rows"],
@@ -404,6 +418,9 @@ def main():
                     help="reorder the matrix with tf_reorder_rcm / tf_permute_csr before inspecting it (after --scramble)")
     ap.add_argument("--unfused", action="store_true",
                     help="GeMM-SpMM as two launches (tf_gemm, tf_spmm) with the intermediate in HBM, for comparison")
+    ap.add_argument("--two-layers", default=None, choices=["compose", "fuse"],
+                    help="GeMM-SpMM with K = N on a square matrix (--config 6): two GCN layers per step through tf_gcn_two_layers, "
+                         "as one executor call per layer or through the schedule's two-layer tiles (TF_FUSE_LAYERS)")
     ap.add_argument("--host-buffers", action="store_true",
                     help="also time the step as the README API runs it on un-pinned operands: upload A, B/C and D, "
                          "execute, download D (reported as host_buffer_ms_per_step; never part of value)")
@@ -428,7 +445,7 @@ def main():
     if args.calibrate_gather:
         calibrate_gather(tf)
         return
-    custom = bool(args.matrix or args.scramble or args.rcm or args.unfused)
+    custom = bool(args.matrix or args.scramble or args.rcm or args.unfused or args.two_layers)
     if args.matrix:
         Af = tf.read_matrix(args.matrix)
         if Af.shape[0] != Af.shape[1]:
@@ -439,6 +456,8 @@ def main():
                    K=args.K if gemm else 0, N=args.N, name=f"file {os.path.basename(args.matrix)} {args.op} N={args.N}" + (f" K={args.K}" if gemm else ""))
     else:
         cfg = w.make_config(args.config)
+    if args.two_layers:
+        cfg["name"] += ", two layers with ReLU (tf_gcn_two_layers: " + ("two-layer tiles, hidden layer in LDS)" if args.two_layers == "fuse" else "one executor call per layer)")
     reorder_s = None
     if args.scramble or args.rcm:  # same product on a renumbered graph: A' = A[p,:][:,p], dense row operands follow
         A0 = cfg["A"]

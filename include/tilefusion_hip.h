@@ -383,10 +383,9 @@ enum {
                            against 2.35 ms: the gathers and the GEMM's operand traffic meet in the
                            same memory system), so it is not the default */
   TF_RELU = 4u,          /* tf_gcn_two_layers: ReLU between the layers */
-  TF_FUSE_LAYERS = 8u,   /* tf_gcn_two_layers: run the second schedule's two-layer tiles (one launch, the hidden
-                           layer never leaves LDS) or fail with TF_EUNSUPPORTED if it has none; without this flag
-                           they run when they recompute little (see tf_gcn_two_layers)                      */
-  TF_COMPOSE_LAYERS = 16u /* tf_gcn_two_layers: never the two-layer tiles: one tf_gemm_spmm per layer        */
+  TF_FUSE_LAYERS = 8u    /* tf_gcn_two_layers: run the second schedule's two-layer tiles (one launch, the hidden
+                           layer never leaves LDS), or fail with TF_EUNSUPPORTED if it has none; without this flag
+                           each layer is one tf_gemm_spmm (see tf_gcn_two_layers)                            */
 };
 
 /* D = A * (B * C), A and B sparse.  Stands in for
@@ -417,10 +416,12 @@ tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf
  *    228-290): when s2 carries them (tf_schedule_info.two_layer_tiles > 0: a square matrix whose rows' halos fit LDS
  *    -- banded or reordered patterns -- and H, N of 32, 64 or 128), K is a multiple of 8 up to 256 and `hidden` is
  *    null, ONE launch takes every tile through GEMM, SpMM, activation, GEMM, SpMM with the first intermediate, the
- *    hidden rows and the second intermediate in LDS; only X, the weights, A and D cross HBM.  A tile recomputes the
- *    halo rows of its neighbours: this path is taken by default when that costs at most 1.3x the GEMM rows of
- *    the composed path, always with TF_FUSE_LAYERS, never with TF_COMPOSE_LAYERS;
- *  - composed: each layer runs as tf_gemm_spmm does with its own schedule (rows fuse inside a layer), the hidden
+ *    hidden rows and the second intermediate in LDS; only X, the weights, A and D cross HBM.  Taken with
+ *    TF_FUSE_LAYERS only: a tile recomputes the halo rows of its neighbours in both GEMMs (1.4x the GEMM rows on a
+ *    band of 32 at H = N = 128) and runs its phases one after the other, which measured slower than the composed path
+ *    wherever that one streams (0.63 ms against 0.31 ms on 262,144 rows, K = H = N = 128); what it saves is the hidden
+ *    layer's trip through HBM (WRITE_SIZE = D only) and a launch;
+ *  - composed (the default): each layer runs as tf_gemm_spmm does with its own schedule (rows fuse inside a layer), the hidden
  *    layer in `hidden` (M x H) when given -- training keeps it for the backward pass -- else in a buffer that s2
  *    owns, one small ReLU launch between the layers.
  * The reference's fusedGCN reads its second GEMM's input

@@ -15,7 +15,6 @@ ACCUMULATE = 1
 SECOND_STREAM = 2
 RELU = 4
 FUSE_LAYERS = 8
-COMPOSE_LAYERS = 16
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -393,7 +392,7 @@ def gcn_two_layers(A, X, W1, W2, D, s1, s2, *, relu=True, hidden=None, accumulat
     (binding-project/gcn-e2e-training/FusedGCNModule.py:14-18); the hidden layer stays on the device."""
     _check(lib().tf_gcn_two_layers(A.to_device().h, X.h, W1.h, W2.h, D.h, s1.h, s2.h, hidden.h if hidden is not None else None,
                                    (RELU if relu else 0) | (ACCUMULATE if accumulate else 0) |
-                                   (FUSE_LAYERS if fuse is True else COMPOSE_LAYERS if fuse is False else 0), stream.h if stream else None))
+                                   (FUSE_LAYERS if fuse else 0), stream.h if stream else None))
 
 
 def spmm_spmm_noalloc(A, B, Cm, D, *, accumulate=False, stream=None):

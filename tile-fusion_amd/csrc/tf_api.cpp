@@ -114,10 +114,6 @@ hipError_t launch_fused_gcn2(const Tile2 *, int, const float *, const float *, c
 hipError_t launch_zero_rows(const int *, int, float *, int, hipStream_t);
 hipError_t launch_xcd_probe(int *, int, hipStream_t);
 
-// (GEMM rows computed by two-layer tiles) / (GEMM rows of the two layers computed once) up to which the tiles
-// are the default of tf_gcn_two_layers
-constexpr double kTwoLayerMaxWork = 1.3;
-
 // An intermediate larger than the 256 MB last-level cache is gone from it before its readers
 // come: such rows leave through streaming stores.
 inline int inter_streams(const tf_schedule *s) {
@@ -373,15 +369,6 @@ static tf_status run_remainder(const tf_csr *A, tf_dense *D, tf_schedule *s, int
                               (int)s->long_rows.size(), A->i, A->x, d->inter, d->partial, D->d, N,
                               accumulate, st));
   return TF_OK;
-}
-
-// Whether tf_gcn_two_layers runs a schedule's two-layer tiles without being asked to (TF_FUSE_LAYERS): when they
-// recompute little.  A tile computes (t1 - t0) rows of the first GEMM and (h1 - h0) of the second for (o1 - o0)
-// rows it owns; the composed path computes each row once per layer but moves the hidden layer through HBM twice.
-static bool two_layer_tiles_pay(const tf_schedule *s) {
-  long long own = 0, work = 0;
-  for (const auto &t : s->l2_tiles) { own += t.o1 - t.o0; work += (t.t1 - t.t0) + (t.h1 - t.h0); }
-  return own > 0 && work <= (long long)(kTwoLayerMaxWork * 2.0 * own);
 }
 
 }  // namespace tf
@@ -850,13 +837,15 @@ extern "C" tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const
     return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the first schedule was built for K = %d, X is %d x %d and W1 has %d rows", s1->user_K, X->M, X->N, W1->M);
   if (W2->N != s2->user_N || D->N != s2->user_N || D->M != A->M)
     return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule was built for N = %d, W2 has %d columns and D is %d x %d", s2->user_N, W2->N, D->M, D->N);
-  // One launch with the hidden layer in LDS, when the second schedule has two-layer tiles and the caller does not
-  // want the hidden layer back: every tile carries its rows through both layers (fused_gcn2_kernel).
-  const bool fuse_ok = !hidden && !s2->l2_tiles.empty() && s1->user_K == s1->opts.K && s1->user_K <= 256 && !(flags & TF_COMPOSE_LAYERS);
+  // On request (TF_FUSE_LAYERS): one launch with the hidden layer in LDS, every tile of the second schedule's two-layer
+  // tiles carrying its rows through both layers (fused_gcn2_kernel).  Not the default: a tile recomputes its
+  // neighbours' halo rows in both GEMMs and runs its four phases one after the other, which on the banded 262,144-row
+  // pattern (K = H = N = 128) takes 0.63 ms against 0.31 ms for the two streamed launches of the composed path.
+  const bool fuse_ok = !hidden && !s2->l2_tiles.empty() && s1->user_K == s1->opts.K && s1->user_K <= 256;
   if ((flags & TF_FUSE_LAYERS) && !fuse_ok)
     return fail(TF_EUNSUPPORTED, "tf_gcn_two_layers: TF_FUSE_LAYERS needs a second schedule with two-layer tiles (tf_schedule_info.two_layer_tiles: "
                 "a banded pattern, widths of 32, 64 or 128), K a multiple of 8 up to 256 and no `hidden` argument");
-  if (fuse_ok && ((flags & TF_FUSE_LAYERS) || tf::two_layer_tiles_pay(s2))) {
+  if (flags & TF_FUSE_LAYERS) {
     if (A->nnz != s2->nnz || (A->hash && A->hash != s2->pattern_hash))
       return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule was built for another sparsity pattern than A's");
     if (tf_status rc = tf::ensure_device(s2)) return rc;
