@@ -143,6 +143,16 @@ void tf_host_free(void *p);
  * component starts from a pseudo-peripheral node; components are taken in order of their
  * smallest-degree node.  Host-only. */
 tf_status tf_reorder_rcm(int M, const int *Ap, const int *Ai, int *perm);
+/* Partition-based ordering of a square matrix' pattern, symmetrised: n_parts parts of (almost) equal size, each
+ * grown breadth-first from a seed so that most edges stay inside a part, one after the other in perm; vertices
+ * with more than hub_degree neighbours (0 = sixteen times the mean degree, at least 64) are set aside first and
+ * placed in front, by falling degree -- on a power-law graph they would otherwise pull every part into one blob,
+ * and in front they make the most-read intermediate rows one stretch of memory.  Stands in for the reference's
+ * graph-partitioner ordering (METIS metis_perm_general, fusion/src/Fusion_Utils.cpp:181-203; the partitioner itself
+ * is not part of the reference tree): greedy graph growing, its classical initial partitioner.
+ * perm[new index] = old index, M entries.  part_ptr (may be null): n_parts + 2 entries, [0, part_ptr[1]) are the
+ * hubs, part p is [part_ptr[p + 1], part_ptr[p + 2]).  Host-only. */
+tf_status tf_reorder_partition(int M, const int *Ap, const int *Ai, int n_parts, int hub_degree, int *perm, int *part_ptr);
 /* B = A[perm,:][:,perm] (reorder_graphs.py:22), columns sorted; the arrays are released with
  * tf_host_free.  With C' = C[perm,:], D' = B (B C') is D[perm,:] of D = A (A C). */
 tf_status tf_permute_csr(int M, const int *Ap, const int *Ai, const float *Ax, const int *perm, int **Bp, int **Bi,

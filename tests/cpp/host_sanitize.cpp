@@ -93,6 +93,8 @@ int main() {
     o.op = TF_OP_SPMM_SPMM; o.K = 0; o.N = 20; o.long_row_partition = 1; bad += run("powerlaw spmm part", 60000, p, i, o); }
   { std::vector<int> perm(60000); tf_status rc = tf_reorder_rcm(60000, p.data(), i.data(), perm.data()); std::vector<float> x(i.size(), 1.f); int *bp, *bi; float *bx;
     rc = rc ? rc : tf_permute_csr(60000, p.data(), i.data(), x.data(), perm.data(), &bp, &bi, &bx); printf("rcm+permute %d\n", rc); bad += rc != 0; tf_host_free(bp); tf_host_free(bi); tf_host_free(bx); }
+  { std::vector<int> perm(60000), pp(18); tf_status rc = tf_reorder_partition(60000, p.data(), i.data(), 16, 0, perm.data(), pp.data());
+    printf("partition ordering %d hubs %d\n", rc, pp[1]); bad += rc != 0 || pp[17] != 60000; }
   { FILE *f = fopen("host_sanitize_t.mtx", "w"); fprintf(f, "%%%%MatrixMarket matrix coordinate real symmetric\n4 4 3\n1 1 2.0\n3 1 -1\n4 4 5e-1\n"); fclose(f);
     int M, N, nnz, *ap, *ai; float *ax; tf_status rc = tf_read_matrix("host_sanitize_t.mtx", &M, &N, &nnz, &ap, &ai, &ax); printf("read %d nnz %d\n", rc, nnz); bad += rc != 0 || nnz != 4; tf_host_free(ap); tf_host_free(ai); tf_host_free(ax); }
   printf("bad %d\n", bad);

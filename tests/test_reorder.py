@@ -81,3 +81,60 @@ def test_bad_arguments(tf):
         tf.permute_csr(B, np.zeros(50, np.int32))
     with pytest.raises(ValueError):
         tf.permute_csr(B, np.arange(49))
+
+
+def _cut_fraction(A, perm, part_ptr):
+    """Share of the off-diagonal entries whose two ends lie in different parts (hubs count as a part of their own)."""
+    M = A.shape[0]
+    part_of_new = np.searchsorted(part_ptr[1:], np.arange(M), side="right")
+    part = np.empty(M, int)
+    part[perm] = part_of_new
+    C = sp.coo_matrix(A)
+    off = C.row != C.col
+    return float((part[C.row[off]] != part[C.col[off]]).mean())
+
+
+def test_partition_ordering_cuts_few_edges_of_a_grid(tf):
+    """tf_reorder_partition on a scrambled 2D grid: a permutation, parts of equal size, and compact parts -- a small
+    share of the edges crosses between parts (16 random parts of a grid cut 15/16 of them; square blocks of a 96 x 96
+    grid cut about 1/12).  The permuted matrix equals scipy's fancy indexing, as for RCM."""
+    n = 96
+    G, _ = scrambled(tf.workloads.laplacian_2d(n), 7)
+    perm, pp = tf.reorder_partition(G, 16)
+    M = n * n
+    assert np.array_equal(np.sort(perm), np.arange(M))
+    assert pp[0] == 0 and pp[1] == 0 and pp[-1] == M           # a grid has no hubs
+    sizes = np.diff(pp[1:])
+    assert sizes.min() >= M // 16 and sizes.max() <= M // 16 + 1
+    cut = _cut_fraction(G, perm, pp)
+    assert cut < 0.2, cut
+    rnd = np.random.default_rng(1).permutation(M).astype(np.int32)
+    assert _cut_fraction(G, rnd, pp) > 0.9                      # the measure itself: random parts cut nearly all
+    R = tf.permute_csr(G, perm)
+    ref = sp.csr_matrix(G[perm, :][:, perm]); ref.sort_indices()
+    assert np.array_equal(R.indptr, ref.indptr) and np.array_equal(R.indices, ref.indices)
+
+
+def test_partition_ordering_sets_hubs_aside(tf):
+    """On a power-law graph the vertices of very high degree come first, by falling degree, and the rest is still
+    dealt into equal parts; isolated vertices, several components and one part are handled."""
+    cfg = tf.workloads.make_config(4, 2.0 ** -7)
+    A = cfg["A"]
+    M = A.shape[0]
+    S = sp.csr_matrix(A + A.T)
+    deg = np.diff(S.indptr) - (S.diagonal() != 0)
+    perm, pp = tf.reorder_partition(A, 8)
+    assert np.array_equal(np.sort(perm), np.arange(M))
+    nh = pp[1]
+    thr = max(64, 16 * (deg.sum() // M))
+    assert nh == int((deg > thr).sum()) > 0
+    assert np.all(np.diff(deg[perm[:nh]]) <= 0) and deg[perm[:nh]].min() > thr and deg[perm[nh:]].max() <= thr
+    sizes = np.diff(pp[1:])
+    assert sizes.max() - sizes.min() <= 1 and pp[-1] == M
+    perm1, pp1 = tf.reorder_partition(A, 1, hub_degree=10 ** 9)   # no hubs, one part: still a permutation
+    assert pp1[1] == 0 and np.array_equal(np.sort(perm1), np.arange(M))
+    B = sp.block_diag([tf.workloads.laplacian_2d(10), sp.csr_matrix((6, 6), dtype=np.float32), tf.workloads.laplacian_2d(7)], format="csr")
+    permb, ppb = tf.reorder_partition(B, 4)
+    assert np.array_equal(np.sort(permb), np.arange(B.shape[0])) and ppb[-1] == B.shape[0]
+    with pytest.raises(tf.TileFusionError):
+        tf.reorder_partition(A, 0)

@@ -110,6 +110,7 @@ SIGNATURES = {
     "tf_read_dense": (C.c_int, [C.c_char_p, _PI, _PI, C.POINTER(_PF)]),
     "tf_host_free": (None, [_VP]),
     "tf_reorder_rcm": (C.c_int, [C.c_int, _PI, _PI, _PI]),
+    "tf_reorder_partition": (C.c_int, [C.c_int, _PI, _PI, C.c_int, C.c_int, _PI, _PI]),
     "tf_permute_csr": (C.c_int, [C.c_int, _PI, _PI, _PF, _PI, C.POINTER(_PI), C.POINTER(_PI), C.POINTER(_PF)]),
     "tf_inspect": (C.c_int, [C.c_int, C.c_int, _PI, _PI, C.POINTER(InspectOpts), C.POINTER(_VP)]),
     "tf_schedule_free": (None, [_VP]),
@@ -470,6 +471,23 @@ def reorder_rcm(A):
     perm = np.empty(M, np.int32)
     _check(lib().tf_reorder_rcm(M, ap.ctypes.data_as(_PI), ai.ctypes.data_as(_PI), perm.ctypes.data_as(_PI)))
     return perm
+
+
+def reorder_partition(A, n_parts, hub_degree=0):
+    """Partition-based ordering (tf_reorder_partition): returns (perm, part_ptr) with perm[new] = old; the hubs are
+    perm[:part_ptr[1]], part p is perm[part_ptr[p + 1]:part_ptr[p + 2]].  The library's counterpart of the reference's
+    graph-partitioner ordering (fusion/src/Fusion_Utils.cpp:181-203)."""
+    import scipy.sparse as sp
+    A = sp.csr_matrix(A)
+    if A.shape[0] != A.shape[1]:
+        raise ValueError("reorder_partition: the matrix must be square")
+    M = A.shape[0]
+    ap, ai = _as_i32(A.indptr), _as_i32(A.indices)
+    perm = np.empty(M, np.int32)
+    part_ptr = np.zeros(n_parts + 2, np.int32)
+    _check(lib().tf_reorder_partition(M, ap.ctypes.data_as(_PI), ai.ctypes.data_as(_PI), int(n_parts), int(hub_degree),
+                                      perm.ctypes.data_as(_PI), part_ptr.ctypes.data_as(_PI)))
+    return perm, part_ptr
 
 
 def permute_csr(A, perm):

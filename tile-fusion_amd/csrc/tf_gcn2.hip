@@ -35,18 +35,17 @@ static_assert(kG2StageFloats == kTile2StageFloats && kG2Pad == kTile2Pad, "the i
 
 // One MFMA phase's share of a 64-row step: acc[bi] += A-operand rows (16 bi + j) x this wavefront's weight slice,
 // for the 16-row blocks bi this wavefront takes.  `xrow(bi)` = LDS address of row 16 bi + j, k = 0.
-// nb: how many of the step's four blocks hold rows at all (the last step of a phase may hold fewer).
 template <int RG, class RowPtr>
-__device__ __forceinline__ void g2_mfma_16k(const RowPtr &xrow, int koff, int h, int rg, int nb, const float *w, g2_v4f (&acc)[4]) {
+__device__ __forceinline__ void g2_mfma_16k(const RowPtr &xrow, int koff, int h, int rg, const float *w, g2_v4f (&acc)[4]) {
   fvec<4> a[4];
 #pragma unroll
   for (int bi = 0; bi < 4; ++bi)
-    if ((bi % RG) == rg && bi < nb) a[bi] = *reinterpret_cast<const fvec<4> *>(xrow(bi) + koff + 4 * h);
+    if ((bi % RG) == rg) a[bi] = *reinterpret_cast<const fvec<4> *>(xrow(bi) + koff + 4 * h);
 #pragma unroll
   for (int u = 0; u < 4; ++u)
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi)
-      if ((bi % RG) == rg && bi < nb) acc[bi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[bi].v[u], w[u], acc[bi], 0, 0, 0);
+      if ((bi % RG) == rg) acc[bi] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[bi].v[u], w[u], acc[bi], 0, 0, 0);
 }
 
 template <int KS1, int KS2, int NS>
@@ -112,9 +111,8 @@ __global__ __launch_bounds__(kG2Block) void fused_gcn2_kernel(
         x2 = chunk_unit(ch + 3);
         const float *xb = slabB + (ch & 1) * (kG2XRows * kG2XLd);
         auto xrow = [&](int bi) { return xb + (16 * bi + j) * kG2XLd; };
-        const int nb = (min(P1 - r0, kG2XRows) + 15) / 16;
-        g2_mfma_16k<RGH>(xrow, 0, h, rgh, nb, w1 + 4 * (2 * kc), acc);
-        g2_mfma_16k<RGH>(xrow, 16, h, rgh, nb, w1 + 4 * (2 * kc + 1), acc);
+        g2_mfma_16k<RGH>(xrow, 0, h, rgh, w1 + 4 * (2 * kc), acc);
+        g2_mfma_16k<RGH>(xrow, 16, h, rgh, w1 + 4 * (2 * kc + 1), acc);
         if (ch + 1 < nchunks) *reinterpret_cast<fvec<4> *>(slabB + ((ch + 1) & 1) * (kG2XRows * kG2XLd) + sr * kG2XLd + sk) = x0;
         x0 = x1;
         x1 = x2;
@@ -158,9 +156,8 @@ __global__ __launch_bounds__(kG2Block) void fused_gcn2_kernel(
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[b] = g2_v4f{0.f, 0.f, 0.f, 0.f};
     auto xrow = [&](int bi) { return slabB + min(r0 + 16 * bi + j, PH - 1) * ldh; };
-    const int nb = (min(PH - r0, 64) + 15) / 16;
 #pragma unroll
-    for (int m = 0; m < KS2; ++m) g2_mfma_16k<RGN>(xrow, 16 * m, h, rgn, nb, w2 + 4 * m, acc);
+    for (int m = 0; m < KS2; ++m) g2_mfma_16k<RGN>(xrow, 16 * m, h, rgn, w2 + 4 * m, acc);
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi)
       if ((bi % RGN) == rgn) {

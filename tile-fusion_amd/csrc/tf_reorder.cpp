@@ -1,5 +1,5 @@
-// Reordering for locality: reverse Cuthill-McKee on the symmetrised pattern, and the
-// symmetric permutation of a CSR matrix.  The reference reorders its inputs offline with
+// Reordering for locality: reverse Cuthill-McKee and a partition-based ordering on the symmetrised
+// pattern, and the symmetric permutation of a CSR matrix.  The reference reorders its inputs offline with
 // scipy.sparse.csgraph.reverse_cuthill_mckee and A[perm,:][:,perm]
 // (fusion/scripts/reorder_graphs.py:3,21-22) so that rows that depend on each other sit close
 // together and tiles fuse; this is the same step as a library call.  Host-only code.
@@ -117,6 +117,81 @@ extern "C" tf_status tf_reorder_rcm(int M, const int *Ap, const int *Ai, int *pe
     return tf::fail(TF_ENOMEM, "tf_reorder_rcm: out of host memory");
   } catch (const std::exception &e) {
     return tf::fail(TF_EUNSUPPORTED, "tf_reorder_rcm: %s", e.what());
+  }
+  return TF_OK;
+}
+
+// Partition-based ordering: the vertices in `n_parts` parts of (almost) equal size, each grown breadth-first
+// from a seed so that most edges stay inside a part, the parts one after the other; vertices of very high
+// degree ("hubs": more than hub_degree neighbours) are taken out first and placed in front, by falling degree.
+// The reference reorders with a graph partitioner for the same purpose (METIS, metis_perm_general at
+// fusion/src/Fusion_Utils.cpp:181-203; not shipped with it): rows that depend on each other end up in one
+// stretch of the matrix, so that tiles of consecutive rows hold their dependences.  Greedy graph growing is
+// the classical initial partitioner of such packages; it needs no refinement to cut a mesh into compact
+// pieces.  On a power-law graph the hubs would pull every part into one blob within two BFS levels, which
+// is why they are set aside: in front, they also make the most-read intermediate rows one contiguous
+// stretch of memory.
+extern "C" tf_status tf_reorder_partition(int M, const int *Ap, const int *Ai, int n_parts, int hub_degree, int *perm,
+                                          int *part_ptr) {
+  if (M < 0 || !Ap || !perm || (M > 0 && Ap[M] > 0 && !Ai)) return tf::fail(TF_EINVAL, "tf_reorder_partition: null argument");
+  if (n_parts <= 0) return tf::fail(TF_EINVAL, "tf_reorder_partition: n_parts must be positive");
+  if (M == 0) {
+    if (part_ptr) for (int p = 0; p <= n_parts + 1; ++p) part_ptr[p] = 0;
+    return TF_OK;
+  }
+  if (Ap[0] != 0) return tf::fail(TF_EINVAL, "tf_reorder_partition: Ap[0] must be 0");
+  for (int i = 0; i < M; ++i) {
+    if (Ap[i + 1] < Ap[i]) return tf::fail(TF_EINVAL, "tf_reorder_partition: row pointers decrease at row %d", i);
+    for (int k = Ap[i]; k < Ap[i + 1]; ++k)
+      if (Ai[k] < 0 || Ai[k] >= M) return tf::fail(TF_EINVAL, "tf_reorder_partition: column %d out of range in row %d (the matrix must be square)", Ai[k], i);
+  }
+  try {
+    std::vector<int> ptr, adj;
+    symmetrise(M, Ap, Ai, &ptr, &adj);
+    auto degree = [&](int v) { return ptr[v + 1] - ptr[v]; };
+    if (hub_degree <= 0) {  // default: 16 times the mean degree, at least 64
+      const long long mean = ptr[M] / std::max(M, 1);
+      hub_degree = (int)std::min<long long>(INT_MAX, std::max<long long>(64, 16 * mean));
+    }
+    std::vector<char> placed(M, 0);
+    std::vector<int> order;
+    order.reserve(M);
+    for (int v = 0; v < M; ++v)
+      if (degree(v) > hub_degree) { order.push_back(v); placed[v] = 1; }
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return degree(a) > degree(b); });
+    const int n_hubs = (int)order.size();
+    if (part_ptr) { part_ptr[0] = 0; part_ptr[1] = n_hubs; }
+    // seeds in order of rising degree: a part starts at the rim of what is left, not in its middle
+    std::vector<int> by_degree;
+    by_degree.reserve(M - n_hubs);
+    for (int v = 0; v < M; ++v)
+      if (!placed[v]) by_degree.push_back(v);
+    std::stable_sort(by_degree.begin(), by_degree.end(), [&](int a, int b) { return degree(a) < degree(b); });
+    size_t next_seed = 0;
+    const int rest = M - n_hubs;
+    for (int p = 0; p < n_parts; ++p) {
+      const int target = n_hubs + (int)((long long)rest * (p + 1) / n_parts);  // where this part ends
+      size_t head = order.size();
+      while ((int)order.size() < target) {
+        if (head == order.size()) {  // frontier empty: the next seed continues the part
+          while (next_seed < by_degree.size() && placed[by_degree[next_seed]]) ++next_seed;
+          if (next_seed == by_degree.size()) break;
+          const int s = by_degree[next_seed];
+          placed[s] = 1;
+          order.push_back(s);
+        }
+        const int v = order[head++];
+        for (int k = ptr[v]; k < ptr[v + 1] && (int)order.size() < target; ++k)
+          if (!placed[adj[k]]) { placed[adj[k]] = 1; order.push_back(adj[k]); }
+      }
+      if (part_ptr) part_ptr[p + 2] = (int)order.size();
+    }
+    if ((int)order.size() != M) return tf::fail(TF_EINVAL, "tf_reorder_partition: internal error, %zu of %d vertices placed", order.size(), M);
+    for (int i = 0; i < M; ++i) perm[i] = order[i];
+  } catch (const std::bad_alloc &) {
+    return tf::fail(TF_ENOMEM, "tf_reorder_partition: out of host memory");
+  } catch (const std::exception &e) {
+    return tf::fail(TF_EUNSUPPORTED, "tf_reorder_partition: %s", e.what());
   }
   return TF_OK;
 }
