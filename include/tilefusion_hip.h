@@ -359,8 +359,8 @@ typedef struct {
   /* appended after the first version */
   /* Two-layer tiles (tf_schedule_info.two_layer_tiles of them, else null / 0): two_layer_range[8*t + {0..5}] =
      o0, o1, h0, h1, t0, t1: tile t owns the rows [o0, o1) of D, computes the hidden rows [h0, h1) they read and
-     the rows [t0, t1) of the first layer's intermediate those read ([8*t + 6] = floats of LDS its first slab takes,
-     [8*t + 7] unused). */
+     the rows [t0, t1) of the first layer's intermediate those read ([8*t + 6], [8*t + 7]: where its second slab and its copy of A's
+     rows start in LDS, in floats). */
   const int *two_layer_range;
   int n_two_layer;
 } tf_schedule_view;

@@ -552,7 +552,10 @@ def _check_two_layer_tiles(A, rng6, H, N):
             assert hc.min() >= t0 and hc.max() < t1
         a = max((t1 - t0) * (H + 4), (h1 - h0) * (N + 4))
         b = max((h1 - h0) * (H + 4), 2 * 64 * 36)
-        assert (a + b) * 4 <= 163840
+        c0, c1 = (min(o0, h0), max(o1, h1)) if h1 > h0 else (o0, o1)   # the tile's copy of A's rows
+        al = lambda x: (x + 3) // 4 * 4  # noqa: E731
+        c = al(c1 - c0 + 1) + 2 * al(int(A.indptr[c1] - A.indptr[c0]))
+        assert (a + b + c) * 4 <= 163840
     assert end == M
 
 

@@ -103,7 +103,7 @@ hipError_t launch_fused_gemm_spmm(const TileDesc *, int, const int *, const floa
                                   float *, int, int, int, int, int, hipStream_t);
 hipError_t launch_fused_gemm_spmm_stream(const TileDesc *, int, const int *, const int *, const int *,
                                          const float *, const float *, int, int, int, const int *,
-                                         const float *, float *, float *, int, int, hipStream_t);
+                                         const float *, float *, float *, int, int, hipStream_t, int relu_in = 0);
 hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t);
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 hipError_t launch_pad(const float *, int, int, float *, int, int, hipStream_t);
@@ -729,8 +729,9 @@ extern "C" tf_status tf_spmm_spmm(const tf_csr *A, const tf_csr *B, const tf_den
 
 // One pass of a GeMM-SpMM schedule: D (L x opts.N, dense) = A * (Bd * Cd) with Bd L' x opts.K and Cd opts.K x opts.N
 // as the kernels take them.
+// relu_in: Bd holds a layer's output before its activation; only for schedules that relu_on_load_ok() accepts.
 static tf_status gemm_spmm_pass(const tf_csr *A, const float *Bd, const float *Cd, tf_dense *D, tf_schedule *s, int acc,
-                                unsigned flags, hipStream_t st) {
+                                unsigned flags, hipStream_t st, int relu_in = 0) {
   tf::DeviceSchedule *d = s->dev;
   const int n_launch = (int)s->launch_tiles.size();
   if (n_launch > 0) {
@@ -738,7 +739,7 @@ static tf_status gemm_spmm_pass(const tf_csr *A, const float *Bd, const float *C
       TF_PHASE(s, "fused_gemm_spmm_stream_kernel", st,
                tf::launch_fused_gemm_spmm_stream(d->tiles, n_launch, d->step_begin, d->step_ptr,
                                                  d->fused_rec, Bd, Cd, s->opts.K, s->opts.N, s->ring_rows,
-                                                 A->i, A->x, D->d, d->inter, s->lds_bytes, acc, st));
+                                                 A->i, A->x, D->d, d->inter, s->lds_bytes, acc, st, relu_in));
     else
       TF_PHASE(s, s->gemm_regw ? "fused_gemm_spmm_regw_kernel" : "fused_gemm_spmm_kernel", st,
                tf::launch_fused_gemm_spmm(d->tiles, n_launch, d->fused_ids, Bd, Cd,
@@ -775,8 +776,14 @@ static tf_status gemm_spmm_pass(const tf_csr *A, const float *Bd, const float *C
 }
 
 
-extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf_dense *D,
-                                  tf_schedule *s, unsigned flags, void *stream) {
+// A schedule whose every intermediate row is produced by the streamed kernel straight from B (no padded copy, no
+// column panels, no rows left to the row GEMM) can apply an activation to B as it is read.
+static bool relu_on_load_ok(const tf_schedule *s) {
+  return s->gemm_stream && s->plain_rows.empty() && s->user_K == s->opts.K && s->user_N == s->opts.N && !s->launch_tiles.empty();
+}
+
+static tf_status gemm_spmm_impl(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf_dense *D,
+                                tf_schedule *s, unsigned flags, void *stream, int relu_in) {
   tf_status rc = check_common("tf_gemm_spmm", A, C, D, s, TF_OP_GEMM_SPMM);
   if (rc) return rc;
   if (!B) return fail(TF_EINVAL, "tf_gemm_spmm: B is null");
@@ -799,7 +806,8 @@ extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_d
       Cd = d->Cpad;
     }
   }
-  if (!panels) return gemm_spmm_pass(A, Bd, Cd, D, s, acc, flags, st);
+  if (relu_in && !relu_on_load_ok(s)) return fail(TF_EINVAL, "tf_gemm_spmm: internal error, activation on load with a schedule that cannot apply it");
+  if (!panels) return gemm_spmm_pass(A, Bd, Cd, D, s, acc, flags, st, relu_in);
   // A width the MFMA kernels do not take: one pass per column panel of opts.N columns.  The panel of C is
   // copied out (zero columns past N, zero rows past K), the pass writes a dense L x opts.N panel of D,
   // and its columns are copied (or added, with TF_ACCUMULATE) into the caller's D.
@@ -816,6 +824,11 @@ extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_d
              tf::launch_copy_cols(d->Dpanel, D->M, s->opts.N, 0, w, D->d, D->M, D->N, c0, w, acc, st));
   }
   return TF_OK;
+}
+
+extern "C" tf_status tf_gemm_spmm(const tf_csr *A, const tf_dense *B, const tf_dense *C, tf_dense *D,
+                                  tf_schedule *s, unsigned flags, void *stream) {
+  return gemm_spmm_impl(A, B, C, D, s, flags, stream, 0);
 }
 
 extern "C" tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const tf_dense *W1, const tf_dense *W2, tf_dense *D,
@@ -874,10 +887,14 @@ extern "C" tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const
       return fail(TF_ESCHEDULE, "tf_gcn_two_layers: the second schedule's hidden-layer buffer holds %zu floats, %zu are needed", s2->dev->hidden_floats, need);
     h.d = s2->dev->hidden;
   }
-  // first layer (its schedule is checked against X and W1 there), activation, second layer
+  // first layer (its schedule is checked against X and W1 there), activation, second layer.  The activation is a
+  // launch of its own over the hidden layer -- unless that layer stays inside the library and the second schedule
+  // streams all its rows: then the second layer's producers apply it to the hidden rows as they read them
+  // (262,144-row band, K = H = N = 128: the pass over the hidden layer took 41 of the call's 343 us).
   if (tf_status rc = tf_gemm_spmm(A, X, W1, &h, s1, flags & TF_SECOND_STREAM, stream)) return rc;
-  if (flags & TF_RELU) TF_HIP(tf::launch_relu(h.d, (size_t)h.M * h.N, static_cast<hipStream_t>(stream)));
-  return tf_gemm_spmm(A, &h, W2, D, s2, flags & (TF_ACCUMULATE | TF_SECOND_STREAM), stream);
+  const bool relu = (flags & TF_RELU) != 0, on_load = relu && !hidden && relu_on_load_ok(s2);
+  if (relu && !on_load) TF_HIP(tf::launch_relu(h.d, (size_t)h.M * h.N, static_cast<hipStream_t>(stream)));
+  return gemm_spmm_impl(A, &h, W2, D, s2, flags & (TF_ACCUMULATE | TF_SECOND_STREAM), stream, on_load ? 1 : 0);
 }
 
 // ---- benchmark aid: per-launch times of the last executor call -------------------------

@@ -14,7 +14,9 @@
 //   3  T2[h0, h1) = Hid * W2             fp32 MFMA, W2 in registers, Hid read from slab B          -> slab A
 //   4  D[o0, o1) = A[o0, o1) * T2        lane groups gather out of slab A                          -> HBM
 //
-// Only X, the weights, A's rows and D cross HBM.  The MFMA phases are the register-W producer of
+// The rows of A that the two gather phases walk -- one stretch of the CSR arrays, [min(o0, h0), max(o1, h1)) -- are
+// copied into LDS at the start of the tile, so that no gather waits for a row pointer or a (column, value) pair
+// from memory.  Only X, the weights, A's rows and D cross HBM.  The MFMA phases are the register-W producer of
 // fused_gemm_spmm_regw_kernel: v_mfma_f32_16x16x4_f32, a wavefront owns 16 output columns and keeps its
 // K x 16 slice of the weight in registers; when the width has fewer than eight column blocks, the
 // wavefronts that share a block split the four 16-row blocks of a 64-row step among themselves.
@@ -65,6 +67,17 @@ __global__ __launch_bounds__(kG2Block) void fused_gcn2_kernel(
   const int P1 = t.t1 - t.t0, PH = t.h1 - t.h0;
   float *slabA = lds;             // T1 (P1 x ldh), later T2 (PH x ldn)
   float *slabB = lds + t.b_off;   // the staging buffers of X, later Hid (PH x ldh)
+  // the tile's rows of A: row pointers (relative), columns, values
+  const int c0 = PH > 0 ? min(t.o0, t.h0) : t.o0, c1 = PH > 0 ? max(t.o1, t.h1) : t.o1;
+  const int kbase = Ap[c0], nC = Ap[c1] - kbase;
+  int *rp = reinterpret_cast<int *>(lds + t.c_off);
+  int *ci = rp + (c1 - c0 + 1 + 3) / 4 * 4;
+  float *cv = reinterpret_cast<float *>(ci + (nC + 3) / 4 * 4);
+  for (int x = threadIdx.x; x <= c1 - c0; x += kG2Block) rp[x] = Ap[c0 + x] - kbase;
+  for (int x = threadIdx.x; x < nC; x += kG2Block) {
+    ci[x] = Ai[kbase + x];
+    cv[x] = Ax[kbase + x];
+  }
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int j = lane % 16, h = lane / 16;
   const int cbh = wave % KS2, rgh = wave / KS2;
@@ -117,7 +130,7 @@ __global__ __launch_bounds__(kG2Block) void fused_gcn2_kernel(
         x0 = x1;
         x1 = x2;
         ++ch;
-        __syncthreads();
+        lds_barrier();  // (LDS traffic only: the loads of X that are on their way stay on their way)
       }
     }
     // accumulator register r of lane (j, h) is output row 4 h + r, column j of its block
@@ -140,7 +153,7 @@ __global__ __launch_bounds__(kG2Block) void fused_gcn2_kernel(
     const LdsRows<4> src{slabA, ldh, glane * 4, t.t0};
     for (int r = t.h0 + group; r < t.h1; r += G) {
       fvec<4> acc = vzero<4>();
-      row_dot<4, LPRH>(Ai, Ax, Ap[r], Ap[r + 1], glane, true, src, acc);
+      row_dot<4, LPRH>(ci, cv, rp[r - c0], rp[r - c0 + 1], glane, true, src, acc);
       if (relu) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc.v[c] = fmaxf(acc.v[c], 0.f);
@@ -179,7 +192,7 @@ __global__ __launch_bounds__(kG2Block) void fused_gcn2_kernel(
       float *dst = D + (size_t)i * N + glane * 4;
       fvec<4> acc = vzero<4>();
       if (accumulate) acc = *reinterpret_cast<const fvec<4> *>(dst);
-      row_dot<4, LPRN>(Ai, Ax, Ap[i], Ap[i + 1], glane, true, src, acc);
+      row_dot<4, LPRN>(ci, cv, rp[i - c0], rp[i - c0 + 1], glane, true, src, acc);
       store_streaming<4>(dst, acc);
     }
   }

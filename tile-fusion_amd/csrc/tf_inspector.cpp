@@ -41,9 +41,10 @@ void build_two_layer_tiles(tf_schedule *S, int M, const int *Ap, const int *Ai, 
   const int cap = std::max(32, ceil_div(M, std::max(1, compute_units)));
   std::vector<tf::Tile2> tiles;
   long long max_floats = 0;
+  auto align4 = [](long long x) { return (x + 3) / 4 * 4; };
   for (int o0 = 0; o0 < M;) {
     int h0 = INT_MAX, h1 = -1, t0 = INT_MAX, t1 = -1, o1 = o0;
-    long long fa = 0, fb = tf::kTile2StageFloats;
+    long long fa = 0, fb = tf::kTile2StageFloats, fc = 0;
     while (o1 < M && o1 - o0 < cap) {
       const int nh0 = std::min(h0, lo[o1]), nh1 = std::max(h1, hi[o1]);
       int nt0 = t0, nt1 = t1;
@@ -56,8 +57,11 @@ void build_two_layer_tiles(tf_schedule *S, int M, const int *Ap, const int *Ai, 
       const long long PH = std::max(0, nh1 - nh0), P1 = std::max(0, nt1 - nt0);
       const long long a = std::max(P1 * (H + tf::kTile2Pad), PH * (N + tf::kTile2Pad));
       const long long b = std::max<long long>(PH * (H + tf::kTile2Pad), tf::kTile2StageFloats);
-      if (a + b > budget_floats) break;
-      h0 = nh0; h1 = nh1; t0 = nt0; t1 = nt1; fa = a; fb = b;
+      // the tile's copy of A's rows: those it owns and the hidden rows, one stretch of the CSR arrays
+      const int c0 = PH > 0 ? std::min(o0, nh0) : o0, c1 = PH > 0 ? std::max(o1 + 1, nh1) : o1 + 1;
+      const long long c = align4(c1 - c0 + 1) + 2 * align4(Ap[c1] - Ap[c0]);
+      if (a + b + c > budget_floats) break;
+      h0 = nh0; h1 = nh1; t0 = nt0; t1 = nt1; fa = a; fb = b; fc = c;
       ++o1;
     }
     if (o1 == o0) return;  // one row alone does not fit
@@ -66,8 +70,9 @@ void build_two_layer_tiles(tf_schedule *S, int M, const int *Ap, const int *Ai, 
     t.h0 = h1 > h0 ? h0 : 0; t.h1 = h1 > h0 ? h1 : 0;
     t.t0 = t1 > t0 ? t0 : 0; t.t1 = t1 > t0 ? t1 : 0;
     t.b_off = (int)fa;
+    t.c_off = (int)(fa + fb);
     tiles.push_back(t);
-    max_floats = std::max(max_floats, fa + fb);
+    max_floats = std::max(max_floats, fa + fb + fc);
     o0 = o1;
   }
   S->l2_tiles.swap(tiles);
@@ -1050,10 +1055,12 @@ extern "C" tf_status tf_schedule_validate(const tf_schedule *s, int L, int M, co
       end = t.o1;
       if (t.h0 < 0 || t.h1 < t.h0 || t.h1 > M || t.t0 < 0 || t.t1 < t.t0 || t.t1 > M)
         return tf::fail(TF_ESCHEDULE, "two-layer tile %zu: bad ranges", ti);
-      const long long PH = t.h1 - t.h0, P1 = t.t1 - t.t0, b_floats = s->l2_lds_bytes / 4 - t.b_off;
-      if (t.b_off < 0 || (t.b_off & 3) || P1 * (H + tf::kTile2Pad) > t.b_off || PH * (N2 + tf::kTile2Pad) > t.b_off ||
-          PH * (H + tf::kTile2Pad) > b_floats || tf::kTile2StageFloats > b_floats)
-        return tf::fail(TF_ESCHEDULE, "two-layer tile %zu: %lld hidden and %lld intermediate rows do not fit its slabs", ti, PH, P1);
+      const long long PH = t.h1 - t.h0, P1 = t.t1 - t.t0, b_floats = t.c_off - t.b_off;
+      const int c0 = PH > 0 ? std::min(t.o0, t.h0) : t.o0, c1 = PH > 0 ? std::max(t.o1, t.h1) : t.o1;
+      const long long c_floats = ((c1 - c0 + 1 + 3) / 4 * 4) + 2LL * ((Ap[c1] - Ap[c0] + 3) / 4 * 4);
+      if (t.b_off < 0 || (t.b_off & 3) || (t.c_off & 3) || P1 * (H + tf::kTile2Pad) > t.b_off || PH * (N2 + tf::kTile2Pad) > t.b_off ||
+          PH * (H + tf::kTile2Pad) > b_floats || tf::kTile2StageFloats > b_floats || (t.c_off + c_floats) * 4 > s->l2_lds_bytes)
+        return tf::fail(TF_ESCHEDULE, "two-layer tile %zu: %lld hidden and %lld intermediate rows and its %d entries of A do not fit LDS", ti, PH, P1, Ap[c1] - Ap[c0]);
       for (int i = t.o0; i < t.o1; ++i)
         for (int k = Ap[i]; k < Ap[i + 1]; ++k)
           if (Ai[k] < t.h0 || Ai[k] >= t.h1) return tf::fail(TF_ESCHEDULE, "two-layer tile %zu: row %d reads hidden row %d outside [%d, %d)", ti, i, Ai[k], t.h0, t.h1);

@@ -40,7 +40,7 @@ struct LongRow {
 struct Tile2 {
   int o0, o1, h0, h1, t0, t1;
   int b_off;  // floats of LDS in front of the tile's slab B (its slab A: the first intermediate, then the second)
-  int pad;
+  int c_off;  // ... and in front of its copy of A's rows [min(o0, h0), max(o1, h1)): row pointers, columns, values
 };
 static_assert(sizeof(Tile2) == 32, "Tile2 is read as two int4 by the kernel");
 constexpr int kTile2Pad = 4;                 // floats behind every slab row (tf_gcn2.hip: kG2Pad)

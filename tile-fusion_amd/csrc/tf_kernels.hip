@@ -1231,7 +1231,7 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
     const TileDesc *__restrict__ tiles, const int *__restrict__ step_begin, const int *__restrict__ step_ptr,
     const int4 *__restrict__ fused_rec, const float *__restrict__ B, const float *__restrict__ W, int K, int N,
     int ring_rows, const int *__restrict__ Ai, const float *__restrict__ Ax, float *__restrict__ D,
-    float *__restrict__ T) {
+    float *__restrict__ T, int relu_in) {
   extern __shared__ __align__(16) float lds[];
   const TileDesc t = tiles[blockIdx.x];
   constexpr int NW = kStreamProducers;
@@ -1262,8 +1262,15 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
       const int row = t.prod_begin + min(q * kXRows + sr, P - 1);
       return load_streaming4(B + (size_t)row * K + k);
     };
+    // relu_in: B is a layer's output before its activation, max(x, 0) is applied here on its way to the MFMAs
+    // (the second layer of tf_gcn_two_layers: saves a pass over the hidden layer)
     auto unit_or_zero = [&](const fvec<4> &x, int kc) -> fvec<4> {
-      return kc * kXChunk + sk < K ? x : vzero<4>();
+      fvec<4> r = kc * kXChunk + sk < K ? x : vzero<4>();
+      if (relu_in) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) r.v[c] = fmaxf(r.v[c], 0.f);
+      }
+      return r;
     };
     float *const xdst = xbuf + sr * kXLd + sk;
     {
@@ -1967,7 +1974,7 @@ hipError_t launch_fused_gemm_spmm_stream(const TileDesc *tiles, int n_tiles, con
                                          const int *step_ptr, const int *fused_rec, const float *B,
                                          const float *C, int K, int N, int ring_rows, const int *Ai,
                                          const float *Ax, float *D, float *T, int lds_bytes, int accumulate,
-                                         hipStream_t st) {
+                                         hipStream_t st, int relu_in) {
   if (n_tiles <= 0) return hipSuccess;
   const int LPR = pick_shape(N).LPR;
   const int KS = K <= 64 ? 4 : K <= 128 ? 8 : 16;
@@ -1981,7 +1988,7 @@ hipError_t launch_fused_gemm_spmm_stream(const TileDesc *tiles, int n_tiles, con
   if (err == hipSuccess)                                                                             \
     hipLaunchKernelGGL((fused_gemm_spmm_stream_kernel<KS_, 1, L_, NCW_, ACC_>), dim3(n_tiles),       \
                        dim3((kStreamProducers + NCW_) * 64), lds_bytes, st, tiles, step_begin, step_ptr, \
-                       rec, B, C, K, N, ring_rows, Ai, Ax, D, T)
+                       rec, B, C, K, N, ring_rows, Ai, Ax, D, T, relu_in)
 #define CALL3(KS_, L_, NCW_)                                                   \
   do { if (accumulate) { CALL4(KS_, L_, NCW_, true); } else { CALL4(KS_, L_, NCW_, false); } } while (0)
 #define CALL2(KS_, NCW_)                                                       \
