@@ -16,7 +16,14 @@
 //
 // The rows of A that the two gather phases walk -- one stretch of the CSR arrays, [min(o0, h0), max(o1, h1)) -- are
 // copied into LDS at the start of the tile, so that no gather waits for a row pointer or a (column, value) pair
-// from memory.  Only X, the weights, A's rows and D cross HBM.  The MFMA phases are the register-W producer of
+// from memory.  Only X, the weights, A's rows and D cross HBM.
+//
+// Where a tile's time goes (cycle counter per phase; band of 32, K = H = N = 128: 95 rows owned, 124 hidden rows,
+// 154 rows of the first intermediate, 120,000 cycles a tile): weights and A's rows 6 %, phase 1 37 % (its MFMAs
+// alone would take 20 %: one barrier per 32 values of k, with both wavefronts of a SIMD waiting for their LDS operands
+// at the same time), phase 2 21 %, phase 3 21 % (13 %), phase 4 15 %.  The phases run one after the other and all
+// wavefronts are in the same one, so MFMA, LDS and VALU never overlap -- which the streamed kernel's producer and
+// consumer wavefronts do all the time; this kernel trades that for keeping the hidden layer out of HBM.  The MFMA phases are the register-W producer of
 // fused_gemm_spmm_regw_kernel: v_mfma_f32_16x16x4_f32, a wavefront owns 16 output columns and keeps its
 // K x 16 slice of the weight in registers; when the width has fewer than eight column blocks, the
 // wavefronts that share a block split the four 16-row blocks of a 64-row step among themselves.
@@ -153,7 +160,7 @@ __global__ __launch_bounds__(kG2Block) void fused_gcn2_kernel(
     const LdsRows<4> src{slabA, ldh, glane * 4, t.t0};
     for (int r = t.h0 + group; r < t.h1; r += G) {
       fvec<4> acc = vzero<4>();
-      row_dot<4, LPRH>(ci, cv, rp[r - c0], rp[r - c0 + 1], glane, true, src, acc);
+      row_dot_direct<4, LPRH>(ci, cv, rp[r - c0], rp[r - c0 + 1], true, src, acc);
       if (relu) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc.v[c] = fmaxf(acc.v[c], 0.f);
@@ -192,7 +199,7 @@ __global__ __launch_bounds__(kG2Block) void fused_gcn2_kernel(
       float *dst = D + (size_t)i * N + glane * 4;
       fvec<4> acc = vzero<4>();
       if (accumulate) acc = *reinterpret_cast<const fvec<4> *>(dst);
-      row_dot<4, LPRN>(ci, cv, rp[i - c0], rp[i - c0 + 1], glane, true, src, acc);
+      row_dot_direct<4, LPRN>(ci, cv, rp[i - c0], rp[i - c0 + 1], true, src, acc);
       store_streaming<4>(dst, acc);
     }
   }
