@@ -33,7 +33,7 @@ import numpy as np  # noqa: E402
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 MFMA_FP32_PEAK_TF = 157.3  # MI355X dense fp32 MFMA, published
 LLC_BYTES = 256 << 20      # Infinity Cache
-L2_GATHER_TBS = 17.5       # the row kernel gathering 512-byte rows that every XCD finds in its own L2 (profiles/calibration_gather.md)
+L2_GATHER_TBS = 19.7       # the row kernel gathering 512-byte rows that every XCD finds in its own L2 (profiles/calibration_gather.md)
 METRIC = "fused GeMM-SpMM / SpMM-SpMM GFLOP/s and % HBM roofline, 1 MI355X vs CPU"
 HEADLINE = 4               # largest single-GPU configuration, the power-law target
 
