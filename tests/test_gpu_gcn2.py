@@ -131,3 +131,29 @@ def test_two_layer_tiles_refusals(gpu, tf):
     tf.gcn_two_layers(Bh, Xb, W, W, Db, sb, sb, hidden=hid)   # composed, hidden layer handed back
     tf.device_synchronize()
     assert np.isfinite(hid.to_numpy()).all()
+
+
+@pytest.mark.parametrize("lo_off,hi_off,per_row,empty", [(-40, -1, 6, 0.0), (1, 30, 5, 0.1), (-3, 3, 7, 0.3), (-64, 64, 40, 0.05)])
+def test_two_layer_tiles_on_bands_off_the_diagonal(gpu, tf, orc, lo_off, hi_off, per_row, empty):
+    """Strictly lower and strictly upper bands (a tile's owned rows then lie outside its hidden range), rows without
+    entries, rows of 40 entries: the tiles against the oracle composed twice, and exactly on integer operands."""
+    from test_inspector import _random_band
+    say(f"two-layer tiles, band [{lo_off}, {hi_off}]")
+    M, K, H, N = 7000, 64, 64, 64
+    A = _random_band(M, lo_off, hi_off, per_row, seed=11, empty_share=empty)
+    Ah = tf.CsrMatrix.from_scipy(A)
+    s = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=N, K=K, compute_units=16)
+    s.validate()
+    assert s.info()["two_layer_tiles"] > 0
+    X = tf.workloads.uniform((M, K), 131)
+    W1, W2 = tf.workloads.glorot(K, H, 132), tf.workloads.glorot(H, N, 133)
+    want = oracle_two_layers(orc, A, X, W1, W2, True)
+    assert orc.rel_err(run_two_layers(tf, Ah, X, W1, W2, s, s, True, True), want) <= TOL
+    rng = np.random.default_rng(6)
+    Ai = A.copy(); Ai.data = rng.integers(-2, 3, A.nnz).astype(np.float32)
+    Aih = tf.CsrMatrix.from_scipy(Ai)
+    Xi = rng.integers(-2, 3, (M, K)).astype(np.float32)
+    W1i, W2i = rng.integers(-1, 2, (K, H)).astype(np.float32), rng.integers(-1, 2, (H, N)).astype(np.float32)
+    wanti = oracle_two_layers(orc, Ai, Xi, W1i, W2i, True)
+    assert np.abs(wanti).max() < 2 ** 24
+    assert np.array_equal(run_two_layers(tf, Aih, Xi, W1i, W2i, s, s, True, True), wanti)

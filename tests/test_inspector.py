@@ -611,3 +611,48 @@ def test_two_layer_tiles_are_validated_against_the_pattern(tf):
     with pytest.raises(tf.TileFusionError) as e:
         S.validate(tf.CsrMatrix.from_scipy(B))
     assert e.value.status == -4
+
+
+def _random_band(M, lo_off, hi_off, per_row, seed, empty_share=0.0):
+    """Row i holds up to per_row distinct columns drawn from [i + lo_off, i + hi_off] clipped to the matrix."""
+    rng = np.random.default_rng(seed)
+    rows, cols = [], []
+    for i in range(M):
+        if rng.random() < empty_share:
+            continue
+        a, b = max(0, i + lo_off), min(M - 1, i + hi_off)
+        if a > b:
+            continue
+        c = np.unique(rng.integers(a, b + 1, per_row))
+        rows += [i] * len(c)
+        cols += c.tolist()
+    A = sp.csr_matrix((rng.uniform(-1, 1, len(rows)).astype(np.float32), (rows, cols)), shape=(M, M))
+    A.sort_indices()
+    return sp.csr_matrix((A.data, A.indices.astype(np.int32), A.indptr.astype(np.int32)), shape=A.shape)
+
+
+@pytest.mark.parametrize("lo_off,hi_off,per_row,empty", [(-16, 15, 16, 0.0), (-40, -1, 6, 0.0), (1, 30, 5, 0.1), (-3, 3, 7, 0.3),
+                                                         (-200, -150, 4, 0.0), (-64, 64, 40, 0.05)])
+def test_two_layer_tiles_on_irregular_bands(tf, lo_off, hi_off, per_row, empty):
+    """Bands that do not hold the diagonal (strictly lower, strictly upper, far off it), rows without entries, rows of
+    many entries: the owned rows of a tile then need not lie inside its hidden range, and the tile's copy of A's rows
+    spans both.  Every schedule with tiles passes the library's validator and the independent check."""
+    M = 5000
+    A = _random_band(M, lo_off, hi_off, per_row, seed=11, empty_share=empty)
+    for H, N in ((64, 64), (128, 32)):
+        S, view, info = inspect(tf, A, op=tf.OP_GEMM_SPMM, N=N, K=H, compute_units=16)
+        if info["two_layer_tiles"]:
+            _check_two_layer_tiles(A, view["two_layer_range"], H, N)
+        else:                                  # no tiles only if some single row's two halos and its rows of A exceed LDS
+            def alone(i):
+                cols = A.indices[A.indptr[i]:A.indptr[i + 1]]
+                if not len(cols):
+                    return 0
+                h0, h1 = cols.min(), cols.max() + 1
+                hc = A.indices[A.indptr[h0]:A.indptr[h1]]
+                t0, t1 = (hc.min(), hc.max() + 1) if len(hc) else (0, 0)
+                c0, c1 = min(i, h0), max(i + 1, h1)
+                al = lambda x: (x + 3) // 4 * 4  # noqa: E731
+                return (max((t1 - t0) * (H + 4), (h1 - h0) * (N + 4)) + max((h1 - h0) * (H + 4), 2 * 64 * 36)
+                        + al(c1 - c0 + 1) + 2 * al(int(A.indptr[c1] - A.indptr[c0]))) * 4
+            assert max(alone(i) for i in range(M)) > 163840
