@@ -578,6 +578,8 @@ def test_two_layer_tiles_on_banded_patterns(tf):
     # widths the kernel is not built for, the opt-out, a pattern whose halos no LDS holds
     assert inspect(tf, A, op=tf.OP_GEMM_SPMM, N=96, K=128)[2]["two_layer_tiles"] == 0
     assert inspect(tf, A, op=tf.OP_GEMM_SPMM, N=128, K=40)[2]["two_layer_tiles"] == 0
+    assert inspect(tf, A, op=tf.OP_GEMM_SPMM, N=7, K=64)[2]["two_layer_tiles"] == 0    # (runs as a padded panel of 32 columns)
+    assert inspect(tf, A, op=tf.OP_GEMM_SPMM, N=30, K=64)[2]["two_layer_tiles"] == 0
     assert inspect(tf, A, op=tf.OP_GEMM_SPMM, N=128, K=128, two_layer_tiles=-1)[2]["two_layer_tiles"] == 0
     er = tf.workloads.make_config(3, 0.05)["A"]
     assert inspect(tf, er, op=tf.OP_GEMM_SPMM, N=128, K=128)[2]["two_layer_tiles"] == 0

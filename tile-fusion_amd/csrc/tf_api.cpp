@@ -854,7 +854,7 @@ extern "C" tf_status tf_gcn_two_layers(const tf_csr *A, const tf_dense *X, const
   // tiles carrying its rows through both layers (fused_gcn2_kernel).  Not the default: a tile recomputes its
   // neighbours' halo rows in both GEMMs and runs its four phases one after the other, which on the banded 262,144-row
   // pattern (K = H = N = 128) takes 0.63 ms against 0.31 ms for the two streamed launches of the composed path.
-  const bool fuse_ok = !hidden && !s2->l2_tiles.empty() && s1->user_K == s1->opts.K && s1->user_K <= 256;
+  const bool fuse_ok = !hidden && !s2->l2_tiles.empty() && s2->user_N == s2->opts.N && s1->user_K == s1->opts.K && s1->user_K <= 256;
   if ((flags & TF_FUSE_LAYERS) && !fuse_ok)
     return fail(TF_EUNSUPPORTED, "tf_gcn_two_layers: TF_FUSE_LAYERS needs a second schedule with two-layer tiles (tf_schedule_info.two_layer_tiles: "
                 "a banded pattern, widths of 32, 64 or 128), K a multiple of 8 up to 256 and no `hidden` argument");

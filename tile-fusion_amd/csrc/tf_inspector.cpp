@@ -183,8 +183,8 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
   const int row_bytes = gemm_regw ? (o.N + 4) * 4 + 16 : o.N * 4;
   const int p_max = (o.lds_budget_bytes - staging) / row_bytes;
   if (p_max < 8)
-    return tf::fail(TF_EINVAL, "tf_inspect: LDS budget %d holds only %d intermediate rows of N=%d",
-                    o.lds_budget_bytes, p_max, o.N);
+    return tf::fail(TF_EINVAL, "tf_inspect: LDS budget %d holds only %d intermediate rows of N=%d behind %d bytes of staging",
+                    o.lds_budget_bytes, std::max(p_max, 0), o.N, staging);
   if (o.strip_cols <= 0) o.strip_cols = 32;
   if (o.strip_cols != 32 && o.strip_cols != 64)
     return tf::fail(TF_EINVAL, "tf_inspect: strip_cols must be 32 or 64");
@@ -741,7 +741,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
 
     // Tiles that carry their rows through two layers, for when this is the second layer's schedule of
     // tf_gcn_two_layers (hidden width = this K, output width = this N).
-    if (o.op == TF_OP_GEMM_SPMM && L == M && n_panels == 1 && user_K == o.K && o.two_layer_tiles >= 0 &&
+    if (o.op == TF_OP_GEMM_SPMM && L == M && n_panels == 1 && user_K == o.K && user_N == o.N && o.two_layer_tiles >= 0 &&
         (o.K == 32 || o.K == 64 || o.K == 128) && (o.N == 32 || o.N == 64 || o.N == 128))
       build_two_layer_tiles(S, M, Ap, Ai, o.K, o.N, o.compute_units);
 
