@@ -182,6 +182,27 @@ def calibrate(tf, rows=1 << 20, N=128, reps=5):
                       "copy_GBps_read_plus_write": round(2 * rows * N * 4 / dt / 1e9, 1)}))
 
 
+def calibrate_issue(tf, iters=2000):
+    """Do the fp32 MFMA path and the VALU of a SIMD work at the same time?  One workgroup of eight wavefronts per compute
+    unit (two per SIMD); the four older and the four younger wavefronts each run MFMAs, FMAs or nothing (tf_calibrate_issue)."""
+    NONE, MFMA, FMA, BF16 = 0, 1, 2, 3
+    cus = tf.device_init(0)["compute_units"]
+    cases = [("fp32 MFMA on all eight", MFMA, MFMA), ("fp32 FMA on all eight", FMA, FMA),
+             ("fp32 MFMA on the older four, the others idle", MFMA, NONE), ("fp32 FMA on the younger four, the others idle", NONE, FMA),
+             ("fp32 MFMA on the older four beside fp32 FMA on the younger four", MFMA, FMA),
+             ("fp32 FMA on the older four beside fp32 MFMA on the younger four", FMA, MFMA),
+             ("bf16 MFMA on the older four, the others idle", BF16, NONE),
+             ("bf16 MFMA on the older four beside fp32 FMA on the younger four", BF16, FMA)]
+    out = {"calibration_kernel": "issue_probe_kernel via tf_calibrate_issue", "compute_units": cus, "rounds": iters,
+           "per_round": "32 v_mfma_f32_16x16x4_f32 (65,536 flop) | 256 v_fma_f32 (32,768 flop) | 32 v_mfma_f32_16x16x32_bf16 per wavefront",
+           "cases": []}
+    for name, lo, hi in cases:
+        ms = tf.calibrate_issue(lo, hi, iters)
+        flop = sum(4 * cus * iters * {NONE: 0, MFMA: 32 * 2048, FMA: 256 * 128, BF16: 32 * 16384}[r] for r in (lo, hi))
+        out["cases"].append({"case": name, "ms": round(ms, 4), "TFLOPs": round(flop / ms * 1e-9, 1)})
+    print(json.dumps(out))
+
+
 def calibrate_gather(tf, rows=1 << 19, per_row=32, N=128, reps=5):
     """The rate at which the row kernel (spmm_rows_kernel through tf_spmm) gathers 4N-byte rows when they are
     found in L2, in the Infinity Cache, or nowhere: Y = A X with `per_row` random columns per row drawn from
@@ -428,6 +449,8 @@ def main():
     ap.add_argument("--no-check", action="store_true", help="skip the result check")
     ap.add_argument("--calibrate", action="store_true",
                     help="run a copy of known size instead (scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--calibrate-issue", action="store_true",
+                    help="time fp32 MFMA and fp32 VALU work of two wavefronts of a SIMD, alone and side by side")
     ap.add_argument("--calibrate-gather", action="store_true",
                     help="measure the row kernel's gather rate out of L2 / the Infinity Cache / HBM instead (the gather roof's rate)")
     args = ap.parse_args()
@@ -441,6 +464,9 @@ def main():
     dev = tf.device_init(0)
     if args.calibrate:
         calibrate(tf)
+        return
+    if args.calibrate_issue:
+        calibrate_issue(tf)
         return
     if args.calibrate_gather:
         calibrate_gather(tf)

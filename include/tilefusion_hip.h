@@ -69,6 +69,14 @@ typedef struct {
 tf_status tf_device_init(int device, tf_device_info *info);
 tf_status tf_device_synchronize(void);
 
+/* Measurement aid, no counterpart in the reference: one workgroup of eight wavefronts per compute unit, two per SIMD,
+ * each running `iters` rounds of 32 v_mfma_f32_16x16x4_f32 (role 1), 256 v_fma_f32 (role 2), 32
+ * v_mfma_f32_16x16x32_bf16 (role 3) or nothing (role 0); `role_older` is what the first four wavefronts (the older one
+ * of every SIMD) do, `role_younger` the other four.  *ms = average duration of five launches.  Tells whether the
+ * fp32 MFMA path and the VALU of a SIMD work at the same time (they do not: durations add), which bounds every kernel
+ * that runs the GEMM beside the gathers.  Allocates and synchronizes: not for a timed path. */
+tf_status tf_calibrate_issue(int role_older, int role_younger, int iters, float *ms);
+
 /* Streams and events are passed as void* so that callers need no HIP headers; a
  * stream argument of NULL is the default stream.  A hipStream_t obtained elsewhere
  * (e.g. torch.cuda.current_stream().cuda_stream) can be passed as is. */

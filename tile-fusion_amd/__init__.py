@@ -10,6 +10,6 @@ from .binding import (  # noqa: F401
     TileFusionError, lib, lib_path, device_init, device_synchronize, CsrMatrix, DenseMatrix,
     FusedSchedule, inspector, spmm_spmm, gemm_spmm, spmm, gemm, Stream, Event,
     OP_SPMM_SPMM, OP_GEMM_SPMM, ACCUMULATE, SECOND_STREAM, RELU, gcn_two_layers, spmm_spmm_noalloc, noalloc_scratch_bytes,
-    pattern_hash, read_matrix, read_dense, reorder_rcm, reorder_partition, permute_csr,
+    pattern_hash, read_matrix, read_dense, reorder_rcm, reorder_partition, permute_csr, calibrate_issue,
 )
 from . import workloads  # noqa: F401

@@ -127,6 +127,7 @@ SIGNATURES = {
     "tf_gcn_two_layers": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, C.c_uint, _VP]),
     "tf_spmm": (C.c_int, [_VP, _VP, _VP, C.c_uint, _VP]),
     "tf_gemm": (C.c_int, [_VP, _VP, _VP, _VP]),
+    "tf_calibrate_issue": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
 }
 
 _lib = None
@@ -167,6 +168,13 @@ def device_init(device=0):
     info = DeviceInfo(C.sizeof(DeviceInfo))
     _check(lib().tf_device_init(device, C.byref(info)))
     return {f: (getattr(info, f).decode() if f == "arch" else getattr(info, f)) for f, _ in DeviceInfo._fields_ if f != "struct_size"}
+
+
+def calibrate_issue(role_older, role_younger, iters=2000):
+    """Duration in ms of the issue probe (tf_calibrate_issue): roles 0 nothing, 1 fp32 MFMA, 2 fp32 FMA, 3 bf16 MFMA."""
+    ms = C.c_float()
+    _check(lib().tf_calibrate_issue(role_older, role_younger, iters, C.byref(ms)))
+    return ms.value
 
 
 def device_synchronize():

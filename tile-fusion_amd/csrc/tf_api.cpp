@@ -113,6 +113,7 @@ hipError_t launch_fused_gcn2(const Tile2 *, int, const float *, const float *, c
                              const float *, float *, int, int, int, hipStream_t);
 hipError_t launch_zero_rows(const int *, int, float *, int, hipStream_t);
 hipError_t launch_xcd_probe(int *, int, hipStream_t);
+hipError_t launch_issue_probe(float *, int, int, int, int, hipStream_t);
 
 // An intermediate larger than the 256 MB last-level cache is gone from it before its readers
 // come: such rows leave through streaming stores.
@@ -474,6 +475,30 @@ extern "C" tf_status tf_device_init(int device, tf_device_info *info) {
 
 extern "C" tf_status tf_device_synchronize(void) {
   TF_HIP(hipDeviceSynchronize());
+  return TF_OK;
+}
+
+extern "C" tf_status tf_calibrate_issue(int role_older, int role_younger, int iters, float *ms) {
+  if (!ms || iters <= 0 || iters > (1 << 20) || role_older < 0 || role_older > 3 || role_younger < 0 || role_younger > 3)
+    return fail(TF_EINVAL, "tf_calibrate_issue: roles are 0 .. 3, iters 1 .. 2^20");
+  float *out = nullptr;
+  TF_HIP(hipMalloc(reinterpret_cast<void **>(&out), 512 * sizeof(float)));
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipError_t err = hipEventCreate(&e0);
+  if (err == hipSuccess) err = hipEventCreate(&e1);
+  const int cus = tf::default_compute_units(), reps = 5;
+  if (err == hipSuccess) err = tf::launch_issue_probe(out, cus, iters, role_older, role_younger, nullptr);  // warm-up
+  if (err == hipSuccess) err = hipEventRecord(e0, nullptr);
+  for (int r = 0; r < reps && err == hipSuccess; ++r) err = tf::launch_issue_probe(out, cus, iters, role_older, role_younger, nullptr);
+  if (err == hipSuccess) err = hipEventRecord(e1, nullptr);
+  if (err == hipSuccess) err = hipEventSynchronize(e1);
+  float t = 0.f;
+  if (err == hipSuccess) err = hipEventElapsedTime(&t, e0, e1);
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipFree(out);
+  TF_HIP(err);
+  *ms = t / reps;
   return TF_OK;
 }
 

@@ -1292,6 +1292,13 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
           w[c][4 * m + u] = (cb < CB && k < K) ? W[(size_t)k * N + 16 * cb + j] : 0.f;
         }
     }
+    // W has landed before the loop starts.  (Otherwise the first MFMA of every step waits for "everything
+    // requested before this point" -- the compiler cannot tell the loads of W, long done, from the staging
+    // unit requested a moment ago, and a step would begin by waiting out a full trip to memory.)
+#pragma unroll
+    for (int c = 0; c < CPW; ++c)
+#pragma unroll
+      for (int i = 0; i < KS * 4; ++i) asm volatile("" : : "v"(w[c][i]));
     lds_barrier();
     for (int q = 0; q < S; ++q) {
       v4f acc[CPW][4];
