@@ -1273,6 +1273,8 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
       return r;
     };
     float *const xdst = xbuf + sr * kXLd + sk;
+    const int ld4 = ld * 4;
+    char *const ring_lane = reinterpret_cast<char *>(ring) + ((16 * rg + 4 * h) * ld + 16 * cb0 + j) * 4;
     {
       const fvec<4> first = chunk_unit(0);
       *reinterpret_cast<fvec<4> *>(xdst) = unit_or_zero(first, 0);
@@ -1337,26 +1339,44 @@ __global__ __launch_bounds__((kStreamProducers + NCW) * 64) void fused_gemm_spmm
         if (kc == NKC - 1 && cb0 < CB) {
           // last interval of the step: the 64 new rows go into the ring (and to HBM where the
           // remainder reads them) before the barrier that lets the consumers at them
+          const int row0 = t.prod_begin + q * kXRows;
+          const bool plain = (q + 1) * kXRows <= P && (row0 + kXRows <= t.wb_begin || row0 >= t.wb_end);
+          if (plain) {
+            // a whole step without a row to write back (all but a run's ends): sixteen stores off one address.
+            // A step's 64 rows never wrap in the ring (its size is a multiple of 64), so only the step's first
+            // slot is reduced; everything else is this lane's fixed place in the step plus a multiple of a row.
+            char *base = ring_lane + ((q * kXRows) & ring_mask) * ld4;
 #pragma unroll
-          for (int bi = 0; bi < 4; ++bi)
-            if (bi * RG < 4) {
+            for (int bi = 0; bi < 4; ++bi)
+              if (bi * RG < 4) {
 #pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                const int lr = q * kXRows + 16 * (rg + RG * bi) + 4 * h + r;
-                if (lr < P) {
-                  const int row = t.prod_begin + lr;
-                  const bool wb = row >= t.wb_begin && row < t.wb_end;
+                for (int r = 0; r < 4; ++r)
 #pragma unroll
-                  for (int c = 0; c < CPW; ++c) {
-                    const int col = 16 * (cb0 + NW * c) + j;
-                    if (col < N) {
-                      ring[(lr & ring_mask) * ld + col] = acc[c][bi][r];
-                      if (wb) T[(size_t)row * N + col] = acc[c][bi][r];
+                  for (int c = 0; c < CPW; ++c)
+                    *reinterpret_cast<float *>(base + (16 * RG * bi + r) * ld4 + 64 * NW * c) = acc[c][bi][r];
+              }
+          } else {
+#pragma unroll
+            for (int bi = 0; bi < 4; ++bi)
+              if (bi * RG < 4) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                  const int lr = q * kXRows + 16 * (rg + RG * bi) + 4 * h + r;
+                  if (lr < P) {
+                    const int row = t.prod_begin + lr;
+                    const bool wb = row >= t.wb_begin && row < t.wb_end;
+#pragma unroll
+                    for (int c = 0; c < CPW; ++c) {
+                      const int col = 16 * (cb0 + NW * c) + j;
+                      if (col < N) {
+                        ring[(lr & ring_mask) * ld + col] = acc[c][bi][r];
+                        if (wb) T[(size_t)row * N + col] = acc[c][bi][r];
+                      }
                     }
                   }
                 }
               }
-            }
+          }
         }
         lds_barrier();
       }
