@@ -1531,6 +1531,26 @@ __device__ __forceinline__ int4 load_streaming_i4(const int4 *p) {
   return make_int4(v[0], v[1], v[2], v[3]);
 }
 
+// Loads at a uniform base plus a 32-bit byte offset per lane: the address is formed by the load itself (scalar
+// base + vector offset) instead of by 64-bit arithmetic on the VALU, which a wavefront of this kernel pays for in
+// cycles it would otherwise issue FMAs in.  (The schedule is only built for operands these offsets reach.)
+__device__ __forceinline__ int4 march_load_i4_nt(const void *base, unsigned off) {
+  return load_streaming_i4(reinterpret_cast<const int4 *>(reinterpret_cast<const char *>(base) + off));
+}
+__device__ __forceinline__ int march_load_i(const void *base, unsigned off) {
+  return *reinterpret_cast<const int *>(reinterpret_cast<const char *>(base) + off);
+}
+__device__ __forceinline__ int2 march_load_i2(const void *base, unsigned off) {
+  return *reinterpret_cast<const int2 *>(reinterpret_cast<const char *>(base) + off);
+}
+__device__ __forceinline__ fvec<4> march_load_f4(const void *base, unsigned off) {
+  return load4(reinterpret_cast<const float *>(reinterpret_cast<const char *>(base) + off));
+}
+// row * row_bytes + lane_off for row < 2^24, row_bytes < 2^24 and a product below 2^32: one full-rate instruction
+__device__ __forceinline__ unsigned march_row_off(int row, unsigned row_bytes, unsigned lane_off) {
+  return __umul24((unsigned)row, row_bytes) + lane_off;
+}
+
 template <int G>
 __device__ __forceinline__ fvec<4> march_gather(const char *lane_base, int off) {
   return *reinterpret_cast<const fvec<4> *>(lane_base + quad_bcast<G>(off));
@@ -1604,6 +1624,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
   if (threadIdx.x < 16) *reinterpret_cast<fvec<4> *>(lds + kMarchZeroOff + threadIdx.x * 16) = vzero<4>();
   __syncthreads();
   const int group = threadIdx.x >> 4, glane = threadIdx.x & 15, q = threadIdx.x & 3;
+  const unsigned q16 = q * 16, row_bytes = (unsigned)N * 4;
   char *lane_base = lds + glane * 16;
   // List entries [b, e) dealt to the lane groups.  Nothing in the loop is under a condition: a lane
   // group without an entry loads row 0 of C into the trash row, computes a row of padding into the
@@ -1615,7 +1636,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
 #pragma unroll
     for (int u = 0; u < kMarchLpg; ++u) {
       const int x = b + group + kMarchGroups * u;
-      const int2 v = load_list[max(min(x, e - 1), 0)];
+      const int2 v = march_load_i2(load_list, (unsigned)max(min(x, e - 1), 0) << 3);
       const int m = opaque_mask(x < e);
       l[u] = make_int2(v.x, (v.y & m) | (kMarchTrashOff & ~m));  // a group without an entry re-reads another's row into the trash row
     }
@@ -1627,23 +1648,23 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
     for (int u = 0; u < kMarchTpg; ++u) {
       const int x = b0 + group + kMarchGroups * u, xc = max(min(x, b1 - 1), 0);
       const bool ok = x < b1;
-      const int o = row_out[xc], m = opaque_mask(ok);
-      L.et[u] = load_streaming_i4(ell + (size_t)xc * 4 + q);  // a group without a row recomputes another's, into the trash row
+      const int o = march_load_i(row_out, (unsigned)xc << 2), m = opaque_mask(ok);
+      L.et[u] = march_load_i4_nt(ell, ((unsigned)xc << 6) + q16);  // a group without a row recomputes another's, into the trash row
       L.ot[u] = (o & m) | (~kMarchTrashOff & ~m);
     }
 #pragma unroll
     for (int u = 0; u < kMarchDpg; ++u) {
       const int x = b1 + group + kMarchGroups * u, xc = max(min(x, b2 - 1), 0);
       const bool ok = x < b2;
-      const int o = row_out[xc], m = opaque_mask(ok);
-      L.ed[u] = load_streaming_i4(ell + (size_t)xc * 4 + q);
+      const int o = march_load_i(row_out, (unsigned)xc << 2), m = opaque_mask(ok);
+      L.ed[u] = march_load_i4_nt(ell, ((unsigned)xc << 6) + q16);
       L.od[u] = o | ~m;  // -1: no row
     }
     fetch_loads(it + 2, L.ll);
   };
 
   for (int c0 = 0; c0 < N; c0 += 64) {
-    const float *Cl = C + c0 + glane * 4;
+    const unsigned lane_off = (c0 + glane * 4) * 4;  // this lane's four columns of the strip, in bytes
     float *Dl = D + c0 + glane * 4;
     float *Tl = trash + glane * 4;
     // (plain loads: a run's rows of C are its neighbours' halo rows an iteration or two later, and
@@ -1651,7 +1672,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
     // grid against 1.05 GB)
     auto issue = [&](MarchStage &S) {
 #pragma unroll
-      for (int u = 0; u < kMarchLpg; ++u) S.c[u] = load4(Cl + (size_t)S.ll[u].x * N);
+      for (int u = 0; u < kMarchLpg; ++u) S.c[u] = march_load_f4(C, march_row_off(S.ll[u].x, row_bytes, lane_off));
     };
     // One iteration.  `cur` holds its lists; `fut` is free and takes those of iteration it + 2.  Stage
     // X is free (its rows went to LDS an iteration ago) and takes list it + 2, whose entries came with
@@ -1667,21 +1688,21 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
       auto share = [&](auto vc) __attribute__((always_inline)) {
         constexpr int v = decltype(vc)::value;
         X.ll[v] = cur.ll[v];
-        X.c[v] = load4(Cl + (size_t)X.ll[v].x * N);
+        X.c[v] = march_load_f4(C, march_row_off(X.ll[v].x, row_bytes, lane_off));
         if constexpr (v < kMarchTpg) {
           const int x = b0 + group + kMarchGroups * v, xc = max(min(x, b1 - 1), 0);
-          const int o = row_out[xc], m = opaque_mask(x < b1);
-          fut.et[v] = load_streaming_i4(ell + (size_t)xc * 4 + q);  // a group without a row recomputes another's, into the trash row
+          const int o = march_load_i(row_out, (unsigned)xc << 2), m = opaque_mask(x < b1);
+          fut.et[v] = march_load_i4_nt(ell, ((unsigned)xc << 6) + q16);  // a group without a row recomputes another's, into the trash row
           fut.ot[v] = (o & m) | (~kMarchTrashOff & ~m);
         } else {
           constexpr int u = v - kMarchTpg;
           const int x = b1 + group + kMarchGroups * u, xc = max(min(x, b2 - 1), 0);
-          const int o = row_out[xc], m = opaque_mask(x < b2);
-          fut.ed[u] = load_streaming_i4(ell + (size_t)xc * 4 + q);
+          const int o = march_load_i(row_out, (unsigned)xc << 2), m = opaque_mask(x < b2);
+          fut.ed[u] = march_load_i4_nt(ell, ((unsigned)xc << 6) + q16);
           fut.od[u] = o | ~m;  // -1: no row
         }
         const int x = lb + group + kMarchGroups * v;
-        const int2 l = load_list[max(min(x, le - 1), 0)];
+        const int2 l = march_load_i2(load_list, (unsigned)max(min(x, le - 1), 0) << 3);
         const int m = opaque_mask(x < le);
         fut.ll[v] = make_int2(l.x, (l.y & m) | (kMarchTrashOff & ~m));  // a group without an entry re-reads another's row into the trash row
       };
@@ -1715,7 +1736,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
     fetch_lists(1, E1);
     for (int x = tab[2] + group; x < tab[6]; x += kMarchGroups) {
       const int2 l = load_list[x];
-      *reinterpret_cast<fvec<4> *>(lane_base + l.y) = load4(Cl + (size_t)l.x * N);
+      *reinterpret_cast<fvec<4> *>(lane_base + l.y) = march_load_f4(C, march_row_off(l.x, row_bytes, lane_off));
     }
     issue(S1);
     __syncthreads();

@@ -66,6 +66,8 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
   if (S->L != M || o.inner_cols != M || o.N % 64 != 0) return decline(TF_MARCH_SHAPE);
   const long long nnzA = Ap[M], nnzB = Bp[M];
   if (nnzA >= kMarchSrcA || nnzB >= kMarchSrcA) return decline(TF_MARCH_SHAPE);
+  // the kernel reaches the rows of C and its lists through 32-bit byte offsets (row * 4N by a 24-bit multiply)
+  if (M >= (1 << 24) || (long long)M * o.N * 4 >= (1LL << 32)) return decline(TF_MARCH_SHAPE);
   int width = 0;
   for (int i = 0; i < M; ++i) {
     if (Ap[i + 1] - Ap[i] > kMarchW || Bp[i + 1] - Bp[i] > kMarchW) return decline(TF_MARCH_ROW_TOO_LONG);
@@ -252,7 +254,9 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
           tiles.push_back(td);
         }
     }
-    if ((long long)row_out.size() * kMarchW > INT_MAX || max_t > kMarchTpg * kMarchGroups || max_d > kMarchDpg * kMarchGroups ||
+    // (the kernel reaches its lists through 32-bit byte offsets: 64 bytes per ELL row, 8 per load-list entry)
+    if ((long long)row_out.size() * kMarchW * 8 >= (1LL << 32) || (long long)load.size() * 4 >= (1LL << 32) ||
+        max_t > kMarchTpg * kMarchGroups || max_d > kMarchDpg * kMarchGroups ||
         max_loads > kMarchLpg * kMarchGroups || (int)ids.size() != M)
       return false;
     S->march = true;
