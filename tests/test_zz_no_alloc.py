@@ -56,11 +56,22 @@ def test_noalloc_matches_the_scheduled_executor(gpu, tf, orc):
     assert orc.rel_err(D.to_numpy(), D0.astype(np.float64) + (A.astype(np.float64) @ T.astype(np.float64))) <= 1e-5
 
 
+def _free_device_bytes():
+    """hipMemGetInfo of the HIP runtime the library itself is linked against (already loaded into this process)."""
+    import ctypes
+    with open("/proc/self/maps") as f:
+        paths = sorted({line.split()[-1] for line in f if "libamdhip64.so" in line})
+    assert paths, "no HIP runtime is loaded"
+    hip = ctypes.CDLL(paths[0])   # (free memory is the device's: every runtime in the process reports the same)
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
 def test_noalloc_call_allocates_no_device_memory(gpu, tf):
     """What the entry point is for: once the library is initialised on the device (tf_device_init, or one earlier
     call, looks up the scratch array's address) a call leaves the device's free memory exactly as it was -- while
     the probe does see the workspace a scheduled executor allocates on its first call."""
-    import torch
     say("tf_spmm_spmm_noalloc: free device memory unchanged")
     tf.device_init(0)
     M, N = 30000, 64
@@ -70,19 +81,18 @@ def test_noalloc_call_allocates_no_device_memory(gpu, tf):
     st = tf.Stream()
     tf.spmm_spmm_noalloc(Ah, Ah, Cm, D, stream=st)           # warm-up: kernels loaded, address looked up
     st.synchronize()
-    torch.cuda.mem_get_info()                                # (the probe's own first call initialises torch's context)
     tf.device_synchronize()
-    free0 = torch.cuda.mem_get_info()[0]
+    free0 = _free_device_bytes()
     for _ in range(3):
         tf.spmm_spmm_noalloc(Ah, Ah, Cm, D, stream=st)
     st.synchronize()
-    assert torch.cuda.mem_get_info()[0] == free0
+    assert _free_device_bytes() == free0
     # positive control: a scheduled executor's first call allocates its intermediate (30000 x 64 floats = 7.7 MB)
     S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N)
     assert S.info()["workspace_bytes"] > 4 << 20
     tf.spmm_spmm(Ah, Ah, Cm, D, S, stream=st)
     st.synchronize()
-    assert torch.cuda.mem_get_info()[0] < free0
+    assert _free_device_bytes() < free0
 
 
 def test_noalloc_rejects_an_intermediate_beyond_the_scratch(gpu, tf):
