@@ -111,13 +111,17 @@ def cpu_baseline(cfg, budget_s=40.0):
 
     # pass 1: every variant once (the first call of all is a warm-up and not counted)
     run("unfused", None)
-    first = []
+    first, skipped = [], []
     for kind, par in variants:
         if time.perf_counter() - t_start > 0.6 * budget_s and first:
-            break
+            skipped.append(f"{kind} {par}: time budget")
+            continue
         try:
             S = make(kind, par)
         except ValueError:
+            # (variable tiles: the reference's first tile is (cache / 4 - K N) / (K + N) rows, Fusion_Inspector.h:1029-1031,
+            # which is negative when the cache budget is smaller than the weights)
+            skipped.append(f"{kind} {par}: the inspector has no schedule for it (cache budget below K x N weights)")
             continue
         first.append((run(kind, S), kind, par, S))
     if not first:
@@ -154,6 +158,7 @@ def cpu_baseline(cfg, budget_s=40.0):
             "best_fused_ms": round(fused[0][0] * 1e3, 3) if fused else None,
             "unfused_ms": round(unf[0][0] * 1e3, 3) if unf else None,
             "sweep_first_trial_ms": {f"{k} {p}" if k != "unfused" else k: round(t * 1e3, 2) for t, k, p, _ in first},
+            "sweep_skipped": skipped,
             "gemm_gflops": gemm_gflops, "gemm_simd": ("avx512" if O.simd() else "avx2") if gemm else None,
             "os_cpu_count": os.cpu_count(), "usable_cores": have, "omp_num_threads_env": limit or None,
             "omp_proc_bind": os.environ.get("OMP_PROC_BIND"), "omp_dynamic": os.environ.get("OMP_DYNAMIC"),
