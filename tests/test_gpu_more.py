@@ -440,3 +440,50 @@ def test_streaming_gathers_of_short_rows_change_no_bit(gpu, tf, orc):
     assert np.array_equal(outs[0], outs[2]) and np.array_equal(outs[1], outs[2])
     want, _ = orc.gemm_spmm(A, B, W, orc.unfused_schedule(M), nthreads=8)
     assert orc.rel_err(outs[0], want) <= TOL
+
+
+def test_two_host_threads_with_their_own_schedules(gpu, tf, orc):
+    """Two host threads, each with its own operands, schedules and stream, call the executors at the same time (ctypes
+    releases the interpreter lock during a call): every result equals the oracle's, as if each had run alone.  What the
+    threads share is the library's per-process state: the loaded kernels and their attributes, the device properties."""
+    import threading
+    say("two host threads, own schedules and streams")
+    jobs = []
+    for seed, (M, N, K) in enumerate([(6000, 64, 40), (9000, 128, 128)]):
+        A = tf.workloads.banded_random(M, 32, 12, seed=300 + seed)
+        G = tf.workloads.erdos_renyi_gcn(M, 6.0, seed=310 + seed)
+        B, W = tf.workloads.uniform((M, K), 320 + seed), tf.workloads.uniform((K, N), 330 + seed)
+        Cd = tf.workloads.uniform((M, N), 340 + seed)
+        jobs.append(dict(A=A, G=G, B=B, W=W, Cd=Cd, N=N, K=K, M=M,
+                         want_ss=oracle_spmm_spmm(orc, A, A, Cd),
+                         want_gs=orc.gemm_spmm(G, B, W, orc.unfused_schedule(M), nthreads=4)[0]))
+    errors = []
+
+    def work(job):
+        try:
+            M, N, K = job["M"], job["N"], job["K"]
+            st = tf.Stream()
+            Ah, Gh = tf.CsrMatrix.from_scipy(job["A"]), tf.CsrMatrix.from_scipy(job["G"])
+            S1 = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=N, inner=Ah)
+            S2 = tf.inspector(Gh, 1, op=tf.OP_GEMM_SPMM, N=N, K=K)
+            S1.validate(); S2.validate()
+            Cm, Bm, Wm = (tf.DenseMatrix.from_numpy(job[k]) for k in ("Cd", "B", "W"))
+            D1, D2 = tf.DenseMatrix(M, N), tf.DenseMatrix(M, N)
+            for _ in range(15):
+                D1.fill(float("nan"), stream=st); D2.fill(float("nan"), stream=st)
+                tf.spmm_spmm(Ah, Ah, Cm, D1, S1, stream=st)
+                tf.gemm_spmm(Gh, Bm, Wm, D2, S2, stream=st)
+                st.synchronize()
+                if not np.array_equal(D1.to_numpy(), job["want_ss"]):
+                    errors.append((M, "spmm_spmm differs"))
+                if orc.rel_err(D2.to_numpy(), job["want_gs"]) > TOL:
+                    errors.append((M, "gemm_spmm differs"))
+        except Exception as e:  # noqa: BLE001  (reported by the asserting thread)
+            errors.append((job["M"], repr(e)))
+
+    threads = [threading.Thread(target=work, args=(j,)) for j in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[:5]
