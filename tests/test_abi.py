@@ -35,6 +35,11 @@ def test_version_and_error_channel(tf):
     # a null output pointer is rejected before any device work
     assert lib.tf_inspect(4, 4, None, None, None, None) == -1
     assert b"tf_inspect" in lib.tf_last_error_string()
+    # the issue probe checks its roles and rounds before it touches the device
+    ms = C.c_float(-1.0)
+    assert lib.tf_calibrate_issue(4, 0, 10, C.byref(ms)) == -1 and lib.tf_calibrate_issue(1, 2, 0, C.byref(ms)) == -1
+    assert lib.tf_calibrate_issue(1, 2, 10, None) == -1 and ms.value == -1.0
+    assert b"tf_calibrate_issue" in lib.tf_last_error_string()
 
 
 def test_cpp_header_compiles(tmp_path):
