@@ -1,6 +1,8 @@
 """tf_spmm_spmm_noalloc: D = A*(B*C) for callers that cannot allocate device memory.  Its output
 must equal tf_spmm_spmm's bit for bit (and the oracle's), on two calls in a row, the second
 with a smaller input -- the fixed scratch array keeps the first call's contents."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -56,16 +58,20 @@ def test_noalloc_matches_the_scheduled_executor(gpu, tf, orc):
     assert orc.rel_err(D.to_numpy(), D0.astype(np.float64) + (A.astype(np.float64) @ T.astype(np.float64))) <= 1e-5
 
 
-def _free_device_bytes():
-    """hipMemGetInfo of the HIP runtime the library itself is linked against (already loaded into this process)."""
+def _hip_runtime():
+    """The HIP runtime the library itself is linked against (already loaded into this process)."""
     import ctypes
     with open("/proc/self/maps") as f:
         paths = sorted({line.split()[-1] for line in f if "libamdhip64.so" in line})
     assert paths, "no HIP runtime is loaded"
-    hip = ctypes.CDLL(paths[0])   # (free memory is the device's: every runtime in the process reports the same)
+    return ctypes.CDLL(paths[0])
+
+
+def _free_device_bytes():
+    import ctypes
     free, total = ctypes.c_size_t(), ctypes.c_size_t()
-    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
-    return free.value
+    assert _hip_runtime().hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value   # (of the device: every runtime in the process reports the same)
 
 
 def test_noalloc_call_allocates_no_device_memory(gpu, tf):
@@ -103,3 +109,40 @@ def test_noalloc_rejects_an_intermediate_beyond_the_scratch(gpu, tf):
     with pytest.raises(tf.TileFusionError) as e:
         tf.spmm_spmm_noalloc(Ah, Ah, Cm, D)
     assert e.value.status == -5 and "scratch" in str(e.value)
+
+
+def test_noalloc_call_replays_from_a_graph(gpu, tf, orc):
+    """The callers the entry point is for: its two launches are captured into a HIP graph (a capture refuses any
+    allocation) and the graph is replayed three times with other values in C, eager work and synchronizations in
+    between; every replay equals the eager call and the oracle bit for bit."""
+    say("tf_spmm_spmm_noalloc under stream capture")
+    hip = _hip_runtime()
+    tf.device_init(0)
+    M, N = 20000, 64
+    A = tf.workloads.banded_random(M, 32, 12, seed=401)
+    Ah = tf.CsrMatrix.from_scipy(A).to_device()
+    Cs = [tf.workloads.uniform((M, N), 402 + i) for i in range(3)]
+    Cm, D = tf.DenseMatrix.from_numpy(Cs[0]), tf.DenseMatrix(M, N)
+    st = tf.Stream()
+    tf.spmm_spmm_noalloc(Ah, Ah, Cm, D, stream=st)   # eager once: kernels loaded, scratch address looked up
+    st.synchronize()
+    graph, gexec = C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamBeginCapture(st.h, 0) == 0
+    try:
+        tf.spmm_spmm_noalloc(Ah, Ah, Cm, D, stream=st)
+    finally:
+        rc = hip.hipStreamEndCapture(st.h, C.byref(graph))
+    assert rc == 0 and graph.value
+    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+    try:
+        for i in range(3):
+            Cm.copy_from(tf.DenseMatrix.from_numpy(Cs[i]), stream=st)
+            D.fill(float("nan"), stream=st)
+            st.synchronize()
+            assert hip.hipGraphLaunch(gexec, st.h) == 0
+            st.synchronize()
+            got = D.to_numpy()
+            assert np.array_equal(got, oracle_spmm_spmm(orc, A, A, Cs[i])), i
+    finally:
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
