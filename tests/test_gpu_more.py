@@ -487,3 +487,73 @@ def test_two_host_threads_with_their_own_schedules(gpu, tf, orc):
     for t in threads:
         t.join()
     assert not errors, errors[:5]
+
+
+def test_executors_replay_from_a_graph(gpu, tf, orc):
+    """After one eager call (which allocates the schedule's workspace) an executor call is kernel launches only: it is
+    captured into a HIP graph and replayed three times with other values in the dense operands, eager work and
+    synchronizations in between; every replay equals the oracle (SpMM-SpMM bit for bit).  Launch-bound loops over small
+    products (the 64 x 64 grid of cfg1) are what a caller would capture."""
+    import ctypes as C
+    say("executors under stream capture")
+    with open("/proc/self/maps") as f:
+        hip = C.CDLL(sorted({line.split()[-1] for line in f if "libamdhip64.so" in line})[0])
+    L = tf.workloads.laplacian_2d(64)
+    A = tf.workloads.banded_random(5000, 32, 12, seed=411)
+    st = tf.Stream()
+
+    def replay(call, refresh, check):
+        call()                                   # eager: workspace allocated, kernels loaded
+        st.synchronize()
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert hip.hipStreamBeginCapture(st.h, 0) == 0
+        try:
+            call()
+        finally:
+            rc = hip.hipStreamEndCapture(st.h, C.byref(graph))
+        assert rc == 0 and graph.value
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+        try:
+            for i in range(3):
+                refresh(i)
+                st.synchronize()
+                assert hip.hipGraphLaunch(gexec, st.h) == 0
+                st.synchronize()
+                check(i)
+        finally:
+            hip.hipGraphExecDestroy(gexec)
+            hip.hipGraphDestroy(graph)
+
+    # GeMM-SpMM on the 64 x 64 grid, K = N = 64 (the tile kernel with the weights in registers)
+    M = L.shape[0]
+    Lh = tf.CsrMatrix.from_scipy(L).to_device()
+    Bs = [tf.workloads.uniform((M, 64), 420 + i) for i in range(3)]
+    W = tf.workloads.uniform((64, 64), 430)
+    Bm, Wm, D = tf.DenseMatrix.from_numpy(Bs[0]), tf.DenseMatrix.from_numpy(W), tf.DenseMatrix(M, 64)
+    S = tf.inspector(Lh, 1, op=tf.OP_GEMM_SPMM, N=64, K=64)
+    S.validate()
+
+    def fresh_b(i):
+        Bm.copy_from(tf.DenseMatrix.from_numpy(Bs[i]), stream=st)
+        D.fill(float("nan"), stream=st)
+
+    def check_gs(i):
+        want, _ = orc.gemm_spmm(L, Bs[i], W, orc.unfused_schedule(M))
+        assert orc.rel_err(D.to_numpy(), want) <= TOL, i
+    replay(lambda: tf.gemm_spmm(Lh, Bm, Wm, D, S, stream=st), fresh_b, check_gs)
+
+    # SpMM-SpMM on a band (windowed tiles)
+    M2 = A.shape[0]
+    Ah = tf.CsrMatrix.from_scipy(A).to_device()
+    Cs = [tf.workloads.uniform((M2, 128), 440 + i) for i in range(3)]
+    Cm, D2 = tf.DenseMatrix.from_numpy(Cs[0]), tf.DenseMatrix(M2, 128)
+    S2 = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128, inner=Ah)
+    S2.validate()
+
+    def fresh_c(i):
+        Cm.copy_from(tf.DenseMatrix.from_numpy(Cs[i]), stream=st)
+        D2.fill(float("nan"), stream=st)
+
+    def check_ss(i):
+        assert np.array_equal(D2.to_numpy(), oracle_spmm_spmm(orc, A, A, Cs[i])), i
+    replay(lambda: tf.spmm_spmm(Ah, Ah, Cm, D2, S2, stream=st), fresh_c, check_ss)
