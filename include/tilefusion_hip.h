@@ -235,7 +235,7 @@ typedef struct {
                             executors): built on the first call with a matrix from tf_csr_upload, whose
                             device arrays never change, and on every call with one from
                             tf_csr_wrap_device, whose owner may change them between calls            */
-  /* SpMM-SpMM with an inner pattern, N a multiple of 64, rows of at most 8 entries: marching runs for
+  /* SpMM-SpMM with an inner pattern, N a multiple of 64, rows of at most 32 entries: marching runs for
      patterns whose dependences no range of consecutive rows holds (stencils on a 3D grid).  A run is a
      column of march_tile_x x march_tile_y grid points that one workgroup walks plane by plane, keeping
      the rows of C and of the intermediate that the coming planes need in LDS and recomputing the
@@ -332,7 +332,7 @@ enum {
   TF_MARCH_BUILT = 0,         /* the schedule's tiles are marching runs                                     */
   TF_MARCH_NOT_TRIED = 1,     /* not SpMM-SpMM with an inner pattern, march = -1, or windowed tiles applied */
   TF_MARCH_SHAPE = 2,         /* A or B not square with the same row count, or N not a multiple of 64       */
-  TF_MARCH_ROW_TOO_LONG = 3,  /* a row of A or B has more than 8 entries (27- and 9-point stencils)        */
+  TF_MARCH_ROW_TOO_LONG = 3,  /* a row of A or B has more than 32 entries                                  */
   TF_MARCH_NO_GRID = 4,       /* grid_nx/ny/nz do not multiply to the row count, or none given and the
                                  pattern is not a 5- or 7-point-like stencil a grid can be read off      */
   TF_MARCH_NO_FIT = 5         /* no column of grid points whose rows fit LDS and the run tables            */

@@ -135,3 +135,63 @@ def test_march_full_size_all_ones_exact(gpu, tf):
     T = A.astype(np.float64) @ Cd.astype(np.float64)
     ref = A[rows].astype(np.float64) @ T
     assert np.abs(got[rows] - ref).max() / np.abs(ref).max() <= 1e-5
+
+
+def box_stencil(nx, ny, nz, corners, seed):
+    """The stencil of all neighbours within one step in every direction on an nx x ny x nz grid, x fastest:
+    27 points -- or 19 without the eight corners of the cube.  Random values."""
+    def t(n):
+        e = np.ones(n)
+        return sp.diags([e[:-1], e, e[:-1]], [-1, 0, 1])
+
+    def off(n):
+        e = np.ones(n)
+        return sp.diags([e[:-1], e[:-1]], [-1, 1])
+    A = sp.csr_matrix(sp.kron(sp.kron(t(nz), t(ny)), t(nx)))
+    if not corners:
+        A = A - sp.csr_matrix(sp.kron(sp.kron(off(nz), off(ny)), off(nx)))
+        A.eliminate_zeros()
+    A.sort_indices()
+    A = sp.csr_matrix((A.data.astype(np.float32), A.indices.astype(np.int32), A.indptr.astype(np.int32)), shape=A.shape)
+    A.data = np.random.default_rng(seed).uniform(-1, 1, A.nnz).astype(np.float32)
+    return A
+
+
+@pytest.mark.parametrize("dims,corners,N", [((12, 12, 12), True, 64), ((20, 17, 9), True, 64), ((9, 14, 31), False, 64),
+                                            ((24, 24, 24), True, 128), ((40, 40, 40), True, 64), ((17, 6, 23), False, 192)])
+def test_march_wide_stencils_bit_exact(gpu, tf, orc, dims, corners, N):
+    """27- and 19-point stencils: rows of more than eight entries march with ELL rows of 32 pairs, a lane of the
+    16-lane group holding two, passed on by DPP row broadcasts.  The same bits as the oracle, the grid found from
+    the pattern's distances."""
+    say(f"march wide {dims} corners={corners} N={N}")
+    A = box_stencil(*dims, corners, seed=21)
+    assert np.diff(A.indptr).max() == (27 if corners else 19)
+    Cd = tf.workloads.uniform((A.shape[0], N), 22)
+    want = oracle_spmm_spmm(orc, A, A, Cd)
+    got, info = march(tf, A, A, Cd)
+    assert np.array_equal(got, want), (dims, N, info)
+    got, info = march(tf, A, A, Cd, compute_units=16)
+    assert np.array_equal(got, want), (dims, N, info)
+
+
+def test_march_wide_accumulate_other_values_and_flat_grid(gpu, tf, orc):
+    """Wide rows with D accumulated into, with an inner matrix of the same pattern and other values, and a 9-point
+    stencil on a flat grid (rows of nine entries: the narrowest of the wide kernels)."""
+    say("march wide: accumulate, B != A, 9 points on a flat grid")
+    A = box_stencil(14, 11, 10, True, seed=23)
+    B = A.copy()
+    B.data = np.random.default_rng(24).uniform(-1, 1, B.nnz).astype(np.float32)
+    M = A.shape[0]
+    Cd = tf.workloads.uniform((M, 64), 25)
+    D0 = tf.workloads.uniform((M, 64), 26)
+    want = oracle_spmm_spmm(orc, A, B, Cd)
+    got, _ = march(tf, A, B, Cd)
+    assert np.array_equal(got, want)
+    got, _ = march(tf, A, B, Cd, accumulate=True, D0=D0)
+    assert orc.rel_err(got, want.astype(np.float64) + D0) <= 1e-6
+    F = box_stencil(200, 1, 60, True, seed=27)     # nz x nx grid of 9-point rows
+    assert np.diff(F.indptr).max() == 9
+    Cf = tf.workloads.uniform((F.shape[0], 64), 28)
+    got, info = march(tf, F, F, Cf)
+    assert np.array_equal(got, oracle_spmm_spmm(orc, F, F, Cf)), info
+

@@ -482,7 +482,7 @@ def test_march_validator_rejects_other_patterns(tf):
 
 
 def test_march_says_why_it_was_declined(tf):
-    """tf_schedule_info.march_declined: marching runs need N % 64 == 0, rows of at most 8 entries in both
+    """tf_schedule_info.march_declined: marching runs need N % 64 == 0, rows of at most 32 entries in both
     patterns and a grid; a schedule without them says which of these was missing."""
     A = tf.workloads.laplacian_3d(12)
     Ah = tf.CsrMatrix.from_scipy(A)
@@ -491,13 +491,21 @@ def test_march_says_why_it_was_declined(tf):
     assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64).info()["march_declined"] == 1            # no inner pattern: not tried
     assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Ah, march=-1).info()["march_declined"] == 1
     assert tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=32, inner=Ah).info()["march_declined"] == 2  # N % 64
-    # a 27-point stencil: rows of up to 27 entries
+    # a 27-point stencil (rows of up to 27 entries) marches, with ELL rows of 32 pairs; a stencil that reaches two
+    # points each way (125 points) has rows of more than 32 entries
     e = np.ones(12)
     t = sp.diags([e[:-1], e, e[:-1]], [-1, 0, 1])
-    W = sp.csr_matrix(sp.kron(sp.kron(t, t), t), dtype=np.float32)
-    W.sort_indices()
-    W = sp.csr_matrix((W.data, W.indices.astype(np.int32), W.indptr.astype(np.int32)), shape=W.shape)
-    Wh = tf.CsrMatrix.from_scipy(W)
+    t2 = sp.diags([e[:-2], e[:-1], e, e[:-1], e[:-2]], [-2, -1, 0, 1, 2])
+
+    def box(t):
+        W = sp.csr_matrix(sp.kron(sp.kron(t, t), t), dtype=np.float32)
+        W.sort_indices()
+        return sp.csr_matrix((W.data, W.indices.astype(np.int32), W.indptr.astype(np.int32)), shape=W.shape)
+    W27h = tf.CsrMatrix.from_scipy(box(t))
+    S27 = tf.inspector(W27h, 1, op=tf.OP_SPMM_SPMM, N=64, inner=W27h)
+    S27.validate()
+    assert S27.info()["marched"] == 1 and S27.info()["march_declined"] == 0
+    Wh = tf.CsrMatrix.from_scipy(box(t2))
     assert tf.inspector(Wh, 1, op=tf.OP_SPMM_SPMM, N=64, inner=Wh).info()["march_declined"] == 3
     # short rows, but no grid to be found and none given; a grid that does not multiply to the row count
     R = tf.workloads.erdos_renyi_gcn(1500, 2.0, seed=4)

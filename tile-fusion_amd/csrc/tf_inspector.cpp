@@ -354,7 +354,7 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       }
       if (o.march > 0) {
         delete S;
-        return tf::fail(TF_EUNSUPPORTED, "tf_inspect: no marching schedule for this pattern (needs a square matrix with at most 8 entries "
+        return tf::fail(TF_EUNSUPPORTED, "tf_inspect: no marching schedule for this pattern (needs a square matrix with at most 32 entries "
                         "per row in both patterns, N a multiple of 64, a grid given or found, and a column of grid points whose rows fit LDS)");
       }
     }

@@ -49,7 +49,10 @@ constexpr int kTile2StageFloats = 2 * 64 * 36;  // the two staging buffers of X 
 struct DeviceSchedule;  // device copies + workspace, defined in tf_api.cpp
 
 // Marching runs: LDS layout and list format shared by the inspector, the validator and the kernel.
-constexpr int kMarchW = 8;               // entries per ELL row (longer rows do not march)
+constexpr int kMarchW = 8;               // entries per ELL row when no row of either pattern has more: a lane of a quad holds two
+constexpr int kMarchWideW = 32;          // ... and when one has (up to 32: longer rows do not march): a lane of a group holds two
+// entries per ELL row in a schedule whose longest row has `width` entries
+constexpr int march_ell_stride(int width) { return width <= kMarchW ? kMarchW : kMarchWideW; }
 constexpr int kMarchRowBytes = 256;      // an LDS slot: 64 columns of one row
 constexpr int kMarchTabBytes = 4096;     // per-iteration table of a run, staged at the start of LDS
 constexpr int kMarchMaxIter = kMarchTabBytes / 16 - 2;  // (16 bytes of table per iteration)
@@ -149,7 +152,7 @@ struct tf_schedule {
   std::vector<int> march_load;       // (row of C, LDS byte offset) pairs
   std::vector<int> march_row_out;    // per ELL row: >= 0 row of D, < 0 ~(LDS byte offset) of an intermediate row
   std::vector<int> march_row_id;     // per ELL row: the matrix row it computes (of B when out < 0, of A otherwise)
-  std::vector<int> march_ell_off;    // [kMarchW per ELL row] LDS byte offset of the row read (the zero row for padding)
+  std::vector<int> march_ell_off;    // [march_ell_stride(march_width) per ELL row] LDS byte offset of the row read (the zero row for padding)
   std::vector<int> march_ell_src;    // ... and where its value comes from: index into B's values, or into A's
                                      // with kMarchSrcA set; -1 for padding (value 0)
   // Two-layer tiles (GeMM-SpMM schedules of a square matrix with K and N of 32, 64 or 128, when every tile's two

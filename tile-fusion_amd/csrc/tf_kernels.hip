@@ -1580,6 +1580,72 @@ __device__ __forceinline__ fvec<4> march_row(const int4 e, const char *lane_base
   return acc;
 }
 
+// The same for rows of up to 32 entries: a lane of the 16-lane group holds two (LDS offset, value) pairs, lane l the
+// pairs 2l and 2l + 1, and a pair reaches the group's other lanes through a DPP row broadcast (row_newbcast: the value
+// of one lane of every row of sixteen).  Entry j's gather address is one v_add_u32 with the broadcast as its operand,
+// its four FMAs take the broadcast value as theirs.  Four gathers in flight; entries in CSR order.
+template <int L> __device__ __forceinline__ unsigned march_bcast_add(int off, unsigned lane_addr) {
+  unsigned r;
+  asm("s_nop 1\n\t"
+      "v_add_u32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+      : "=v"(r)
+      : "v"(off), "v"(lane_addr), "n"(L));
+  return r;
+}
+template <int L> __device__ __forceinline__ void march_bcast_fma(int val, const fvec<4> &x, fvec<4> &acc) {
+  asm("s_nop 1\n\t"
+      "v_fmac_f32_dpp %0, %4, %5 row_newbcast:%9 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %1, %4, %6 row_newbcast:%9 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %2, %4, %7 row_newbcast:%9 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %3, %4, %8 row_newbcast:%9 row_mask:0xf bank_mask:0xf"
+      : "+v"(acc.v[0]), "+v"(acc.v[1]), "+v"(acc.v[2]), "+v"(acc.v[3])
+      : "v"(val), "v"(x.v[0]), "v"(x.v[1]), "v"(x.v[2]), "v"(x.v[3]), "n"(L));
+}
+__device__ __forceinline__ fvec<4> march_lds_read(unsigned addr) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const f4 v = *reinterpret_cast<const __attribute__((address_space(3))) f4 *>(addr);
+  fvec<4> r;
+  r.v[0] = v[0]; r.v[1] = v[1]; r.v[2] = v[2]; r.v[3] = v[3];
+  return r;
+}
+template <int J, int W>
+__device__ __forceinline__ void march_wide_gather4(const int4 e, unsigned lane_addr, fvec<4> (&x)[4]) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    if (J + u < W) {
+      // (J is a multiple of 4: entries J, J+1 sit in lane J/2, entries J+2, J+3 in lane J/2 + 1)
+      if (u == 0) x[0] = march_lds_read(march_bcast_add<J / 2>(e.x, lane_addr));
+      if (u == 1) x[1] = march_lds_read(march_bcast_add<J / 2>(e.z, lane_addr));
+      if (u == 2) x[2] = march_lds_read(march_bcast_add<J / 2 + 1>(e.x, lane_addr));
+      if (u == 3) x[3] = march_lds_read(march_bcast_add<J / 2 + 1>(e.z, lane_addr));
+    }
+  }
+}
+template <int J, int W>
+__device__ __forceinline__ void march_wide_fma4(const int4 e, const fvec<4> (&x)[4], fvec<4> &acc) {
+  if (J + 0 < W) march_bcast_fma<J / 2>(e.y, x[0], acc);
+  if (J + 1 < W) march_bcast_fma<J / 2>(e.w, x[1], acc);
+  if (J + 2 < W) march_bcast_fma<J / 2 + 1>(e.y, x[2], acc);
+  if (J + 3 < W) march_bcast_fma<J / 2 + 1>(e.w, x[3], acc);
+}
+template <int B, int NB, int W>
+__device__ __forceinline__ void march_wide_blocks(const int4 e, unsigned lane_addr, fvec<4> (&cur)[4], fvec<4> (&nxt)[4], fvec<4> &acc) {
+  if constexpr (B < NB) {
+    if constexpr (B + 1 < NB) march_wide_gather4<4 * (B + 1), W>(e, lane_addr, nxt);
+    march_wide_fma4<4 * B, W>(e, cur, acc);
+    march_wide_blocks<B + 1, NB, W>(e, lane_addr, nxt, cur, acc);
+  }
+}
+template <int W>
+__device__ __forceinline__ fvec<4> march_row_wide(const int4 e, unsigned lane_addr) {
+  static_assert(W >= 9 && W <= 32, "rows of up to 8 entries take the quad layout");
+  fvec<4> xa[4], xb[4];
+  fvec<4> acc = vzero<4>();
+  march_wide_gather4<0, W>(e, lane_addr, xa);
+  march_wide_blocks<0, (W + 3) / 4, W>(e, lane_addr, xa, xb, acc);
+  return acc;
+}
+
 template <int I, int N, class F>
 __device__ __forceinline__ void static_for(F &&f) {
   if constexpr (I < N) {
@@ -1602,7 +1668,7 @@ struct MarchStage {
   fvec<4> c[kMarchLpg];
 };
 
-template <bool ACC, int W>
+template <bool ACC, int W, bool WIDE = false>
 __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
     const int2 *__restrict__ runs, int n_runs, int per_xcd, const int *__restrict__ row_ptr,
     const int *__restrict__ load_ptr, const int2 *__restrict__ load_list, const int *__restrict__ row_out,
@@ -1624,8 +1690,15 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
   if (threadIdx.x < 16) *reinterpret_cast<fvec<4> *>(lds + kMarchZeroOff + threadIdx.x * 16) = vzero<4>();
   __syncthreads();
   const int group = threadIdx.x >> 4, glane = threadIdx.x & 15, q = threadIdx.x & 3;
-  const unsigned q16 = q * 16, row_bytes = (unsigned)N * 4;
+  // an ELL row is 64 bytes, four lanes of a quad take 16 each -- or 256 bytes, sixteen lanes of the group take 16 each
+  const unsigned q16 = (WIDE ? glane : q) * 16, row_bytes = (unsigned)N * 4;
+  constexpr int ELLS = WIDE ? 8 : 6;  // log2 of an ELL row's bytes
   char *lane_base = lds + glane * 16;
+  const unsigned lane_addr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)lane_base;
+  auto ell_row = [&](const int4 e) __attribute__((always_inline)) {
+    if constexpr (WIDE) return march_row_wide<W>(e, lane_addr);
+    else return march_row<W>(e, lane_base);
+  };
   // List entries [b, e) dealt to the lane groups.  Nothing in the loop is under a condition: a lane
   // group without an entry loads row 0 of C into the trash row, computes a row of padding into the
   // trash row, stores it to the trash row in global memory.  A wait for an older load can then leave
@@ -1649,7 +1722,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
       const int x = b0 + group + kMarchGroups * u, xc = max(min(x, b1 - 1), 0);
       const bool ok = x < b1;
       const int o = march_load_i(row_out, (unsigned)xc << 2), m = opaque_mask(ok);
-      L.et[u] = march_load_i4_nt(ell, ((unsigned)xc << 6) + q16);  // a group without a row recomputes another's, into the trash row
+      L.et[u] = march_load_i4_nt(ell, ((unsigned)xc << ELLS) + q16);  // a group without a row recomputes another's, into the trash row
       L.ot[u] = (o & m) | (~kMarchTrashOff & ~m);
     }
 #pragma unroll
@@ -1657,7 +1730,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
       const int x = b1 + group + kMarchGroups * u, xc = max(min(x, b2 - 1), 0);
       const bool ok = x < b2;
       const int o = march_load_i(row_out, (unsigned)xc << 2), m = opaque_mask(ok);
-      L.ed[u] = march_load_i4_nt(ell, ((unsigned)xc << 6) + q16);
+      L.ed[u] = march_load_i4_nt(ell, ((unsigned)xc << ELLS) + q16);
       L.od[u] = o | ~m;  // -1: no row
     }
     fetch_loads(it + 2, L.ll);
@@ -1692,13 +1765,13 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
         if constexpr (v < kMarchTpg) {
           const int x = b0 + group + kMarchGroups * v, xc = max(min(x, b1 - 1), 0);
           const int o = march_load_i(row_out, (unsigned)xc << 2), m = opaque_mask(x < b1);
-          fut.et[v] = march_load_i4_nt(ell, ((unsigned)xc << 6) + q16);  // a group without a row recomputes another's, into the trash row
+          fut.et[v] = march_load_i4_nt(ell, ((unsigned)xc << ELLS) + q16);  // a group without a row recomputes another's, into the trash row
           fut.ot[v] = (o & m) | (~kMarchTrashOff & ~m);
         } else {
           constexpr int u = v - kMarchTpg;
           const int x = b1 + group + kMarchGroups * u, xc = max(min(x, b2 - 1), 0);
           const int o = march_load_i(row_out, (unsigned)xc << 2), m = opaque_mask(x < b2);
-          fut.ed[u] = march_load_i4_nt(ell, ((unsigned)xc << 6) + q16);
+          fut.ed[u] = march_load_i4_nt(ell, ((unsigned)xc << ELLS) + q16);
           fut.od[u] = o | ~m;  // -1: no row
         }
         const int x = lb + group + kMarchGroups * v;
@@ -1710,7 +1783,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
       static_for<0, kMarchTpg>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
         share(uc);
-        const fvec<4> acc = march_row<W>(cur.et[u], lane_base);
+        const fvec<4> acc = ell_row(cur.et[u]);
         *reinterpret_cast<fvec<4> *>(lane_base + ~cur.ot[u]) = acc;
       });
       lds_barrier();
@@ -1718,7 +1791,7 @@ __global__ __launch_bounds__(kMarchBlock) void fused_spmm_spmm_march_kernel(
       static_for<0, kMarchDpg>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
         share(std::integral_constant<int, kMarchTpg + u>{});
-        fvec<4> acc = march_row<W>(cur.ed[u], lane_base);
+        fvec<4> acc = ell_row(cur.ed[u]);
         float *dst = cur.od[u] >= 0 ? Dl + (size_t)cur.od[u] * N : Tl;
         if (ACC) vadd<4>(*reinterpret_cast<const fvec<4> *>(dst), acc);
         store_streaming<4>(dst, acc);
@@ -2163,23 +2236,33 @@ hipError_t launch_fused_spmm_spmm_march(const int *runs, int n_runs, const int *
   if (n_runs <= 0) return hipSuccess;
   // (rows per lane group and iteration beyond what the kernel's register sets hold would be skipped silently)
   if (N % 64 != 0 || tpg < 1 || tpg > kMarchTpg || dpg < 1 || dpg > kMarchDpg || lpg < 1 || lpg > kMarchLpg || lds_bytes > 163840 ||
-      width < 0 || width > kMarchW)
+      width < 0 || width > kMarchWideW)
     return hipErrorInvalidValue;
   const int per = per_xcd_of(n_runs);
   hipError_t err = hipSuccess;
-#define CALLM(ACC_, W_)                                                                                           \
-  err = allow_lds(fused_spmm_spmm_march_kernel<ACC_, W_>, lds_bytes);                                             \
+#define CALLM3(ACC_, W_, WIDE_)                                                                                   \
+  err = allow_lds(fused_spmm_spmm_march_kernel<ACC_, W_, WIDE_>, lds_bytes);                                      \
   if (err == hipSuccess)                                                                                          \
-    hipLaunchKernelGGL((fused_spmm_spmm_march_kernel<ACC_, W_>), dim3(grid_of(n_runs)), dim3(kMarchBlock),        \
+    hipLaunchKernelGGL((fused_spmm_spmm_march_kernel<ACC_, W_, WIDE_>), dim3(grid_of(n_runs)), dim3(kMarchBlock), \
                        lds_bytes, st, reinterpret_cast<const int2 *>(runs), n_runs, per, row_ptr, load_ptr,       \
                        reinterpret_cast<const int2 *>(load_list), row_out, reinterpret_cast<const int4 *>(ell), C, D, trash, N)
-  switch (width <= 5 ? 5 : width) {
-    case 5: if (accumulate) { CALLM(true, 5); } else { CALLM(false, 5); } break;
-    case 6: if (accumulate) { CALLM(true, 6); } else { CALLM(false, 6); } break;
-    case 7: if (accumulate) { CALLM(true, 7); } else { CALLM(false, 7); } break;
-    default: if (accumulate) { CALLM(true, 8); } else { CALLM(false, 8); } break;
+#define CALLM(W_, WIDE_) do { if (accumulate) { CALLM3(true, W_, WIDE_); } else { CALLM3(false, W_, WIDE_); } } while (0)
+  if (width <= kMarchW) {  // 64-byte ELL rows, the pairs spread over a quad
+    switch (width <= 5 ? 5 : width) {
+      case 5: CALLM(5, false); break;
+      case 6: CALLM(6, false); break;
+      case 7: CALLM(7, false); break;
+      default: CALLM(8, false); break;
+    }
+  } else {  // 256-byte ELL rows, the pairs spread over the lane group: the kernel built for the next width up
+    if (width <= 12) CALLM(12, true);
+    else if (width <= 16) CALLM(16, true);
+    else if (width <= 20) CALLM(20, true);
+    else if (width <= 28) CALLM(28, true);
+    else CALLM(32, true);
   }
 #undef CALLM
+#undef CALLM3
   return err != hipSuccess ? err : hipGetLastError();
 }
 

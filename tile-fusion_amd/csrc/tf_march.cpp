@@ -19,6 +19,7 @@
 #include <cstring>
 #include <iterator>
 #include <map>
+#include <vector>
 
 #include "tf_internal.h"
 
@@ -31,30 +32,65 @@ constexpr int kMaxLds = 163840;
 // The grid a pattern was generated on, from the distances between a row and its columns: a
 // 7-point-like stencil on nx x ny x nz points, x fastest, has the distances 1, nx and nx*ny; a
 // 5-point-like stencil on nx x n points the distances 1 and nx (a grid of nx x 1 x n: the runs then
-// walk the grid's lines, a stretch of a line at a time).
+// walk the grid's lines, a stretch of a line at a time).  Stencils with diagonal neighbours (9, 19, 27
+// points) have the distances |a + b nx + c nx ny| with a, b, c in -1 .. 1: up to thirteen of them.
 bool detect_grid(int M, const int *Ap, const int *Ai, int grid[3]) {
   std::map<int, long long> dist;
   for (int i = 0; i < M; ++i)
     for (int k = Ap[i]; k < Ap[i + 1]; ++k) {
       const int d = std::abs(Ai[k] - i);
       if (d == 0) continue;
-      if (dist.size() > 3 && !dist.count(d)) return false;
+      if (dist.size() >= 13 && !dist.count(d)) return false;
       ++dist[d];
     }
   if (dist.size() == 2) {
     const int d1 = dist.begin()->first, d2 = std::next(dist.begin())->first;
-    if (d1 != 1 || d2 < 16 || M % d2 != 0 || M / d2 < 2) return false;
-    grid[0] = d2; grid[1] = 1; grid[2] = M / d2;
-    return true;
+    if (d1 == 1 && d2 >= 16 && M % d2 == 0 && M / d2 >= 2) {
+      grid[0] = d2; grid[1] = 1; grid[2] = M / d2;
+      return true;
+    }
   }
-  if (dist.size() != 3) return false;
-  auto it = dist.begin();
-  const int d1 = it->first; ++it;
-  const int d2 = it->first; ++it;
-  const int d3 = it->first;
-  if (d1 != 1 || d2 < 2 || d3 % d2 != 0 || d3 / d2 < 2 || M % d3 != 0 || M / d3 < 2) return false;
-  grid[0] = d2; grid[1] = d3 / d2; grid[2] = M / d3;
-  return true;
+  if (dist.size() == 3) {
+    auto it = dist.begin();
+    const int d1 = it->first; ++it;
+    const int d2 = it->first; ++it;
+    const int d3 = it->first;
+    if (d1 == 1 && d2 >= 2 && d3 % d2 == 0 && d3 / d2 >= 2 && M % d3 == 0 && M / d3 >= 2) {
+      grid[0] = d2; grid[1] = d3 / d2; grid[2] = M / d3;
+      return true;
+    }
+  }
+  // diagonal neighbours: the second distance is nx - 1 or nx, the first one beyond nx + 1 one of the plane's
+  if (dist.size() < 2 || dist.begin()->first != 1) return false;
+  std::vector<int> D;
+  for (const auto &kv : dist) D.push_back(kv.first);
+  auto all_fit = [&](long long nx, long long P) {
+    for (int d : D) {
+      bool ok = false;
+      for (int c = -1; c <= 1 && !ok; ++c)
+        for (int b = -1; b <= 1 && !ok; ++b)
+          for (int a = -1; a <= 1 && !ok; ++a) ok = std::llabs(a + b * nx + c * P) == d;
+      if (!ok) return false;
+    }
+    return true;
+  };
+  for (const int nx : {D[1], D[1] + 1}) {
+    if (nx < 3 || M % nx != 0) continue;
+    auto far = std::upper_bound(D.begin(), D.end(), nx + 1);
+    if (far == D.end()) {  // a flat grid
+      if (nx >= 16 && M / nx >= 2 && all_fit(nx, (long long)M * 4)) {
+        grid[0] = nx; grid[1] = 1; grid[2] = M / nx;
+        return true;
+      }
+      continue;
+    }
+    for (const int P : {*far + nx + 1, *far + nx, *far + nx - 1, *far + 1, *far, *far - 1})
+      if (P > 0 && P % nx == 0 && P / nx >= 2 && M % P == 0 && M / P >= 2 && all_fit(nx, P)) {
+        grid[0] = nx; grid[1] = P / nx; grid[2] = M / P;
+        return true;
+      }
+  }
+  return false;
 }
 
 }  // namespace
@@ -70,7 +106,7 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
   if (M >= (1 << 24) || (long long)M * o.N * 4 >= (1LL << 32)) return decline(TF_MARCH_SHAPE);
   int width = 0;
   for (int i = 0; i < M; ++i) {
-    if (Ap[i + 1] - Ap[i] > kMarchW || Bp[i + 1] - Bp[i] > kMarchW) return decline(TF_MARCH_ROW_TOO_LONG);
+    if (Ap[i + 1] - Ap[i] > kMarchWideW || Bp[i + 1] - Bp[i] > kMarchWideW) return decline(TF_MARCH_ROW_TOO_LONG);
     width = std::max(width, std::max(Ap[i + 1] - Ap[i], Bp[i + 1] - Bp[i]));
   }
   int grid[3] = {given.grid_nx, given.grid_ny, given.grid_nz};
@@ -80,6 +116,7 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
     return decline(TF_MARCH_NO_GRID);
   }
   const int nx = grid[0], ny = grid[1], nz = grid[2];
+  const int ell_w = march_ell_stride(width);  // pairs per ELL row: 8, or 32 when a row has more than 8 entries
   const int slot_budget = (kMaxLds - kMarchSlot0) / kMarchRowBytes;
 
   // Runs: columns of bx x by points, cut along z so that every compute unit gets a run.
@@ -95,6 +132,20 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
       nzc = nzc_min;
       for (int c = nzc_min; c <= 2 * nzc_min; ++c)
         if ((long long)per_plane * c % o.compute_units == 0) { nzc = c; break; }
+    }
+    // When the runs are more than the compute units but not a whole number of turns of them (352 columns on 256
+    // units: the second turn is a third full), more cuts along z fill the last turn -- against the three or so
+    // iterations of start-up that every run pays: the number of cuts with the best product of the two.
+    if (per_plane * nzc > o.compute_units) {
+      auto score = [&](int c) {
+        const long long n = (long long)per_plane * c, turns = (n + o.compute_units - 1) / o.compute_units;
+        const double len = (double)nz / c;
+        return (double)n / (double)(turns * o.compute_units) * len / (len + 3.0);
+      };
+      int best = nzc;
+      for (int c = nzc + 1; c <= std::min(std::max(1, nz / 8), 8 * nzc); ++c)
+        if (score(c) > score(best) + 0.02) best = c;
+      nzc = best;
     }
     const int zlen = (nz + nzc - 1) / nzc;
 
@@ -219,7 +270,7 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
                   row_id.push_back(i);
                   ids.push_back(i);
                   lo = std::min(lo, i); hi = std::max(hi, i);
-                  for (int k = Ap[i]; k < Ap[i] + kMarchW; ++k) {
+                  for (int k = Ap[i]; k < Ap[i] + ell_w; ++k) {
                     const bool real = k < Ap[i + 1];
                     ell_off.push_back(real ? kMarchSlot0 + slotT[Ai[k]] * kMarchRowBytes : kMarchZeroOff);
                     ell_src.push_back(real ? (k | kMarchSrcA) : -1);
@@ -235,7 +286,7 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
                 rel[2 * lastT[t] + 1 + 1 + 1].push_back(slotT[t]);
                 row_out.push_back(~(kMarchSlot0 + slotT[t] * kMarchRowBytes));
                 row_id.push_back(t);
-                for (int k = Bp[t]; k < Bp[t] + kMarchW; ++k) {
+                for (int k = Bp[t]; k < Bp[t] + ell_w; ++k) {
                   const bool real = k < Bp[t + 1];
                   ell_off.push_back(real ? kMarchSlot0 + slotC[Bi[k]] * kMarchRowBytes : kMarchZeroOff);
                   ell_src.push_back(real ? k : -1);
@@ -254,8 +305,8 @@ bool build_march(tf_schedule *S, int M, const int *Ap, const int *Ai, const int 
           tiles.push_back(td);
         }
     }
-    // (the kernel reaches its lists through 32-bit byte offsets: 64 bytes per ELL row, 8 per load-list entry)
-    if ((long long)row_out.size() * kMarchW * 8 >= (1LL << 32) || (long long)load.size() * 4 >= (1LL << 32) ||
+    // (the kernel reaches its lists through 32-bit byte offsets: 8 bytes per pair of an ELL row and per load-list entry)
+    if ((long long)row_out.size() * ell_w * 8 >= (1LL << 32) || (long long)load.size() * 4 >= (1LL << 32) ||
         max_t > kMarchTpg * kMarchGroups || max_d > kMarchDpg * kMarchGroups ||
         max_loads > kMarchLpg * kMarchGroups || (int)ids.size() != M)
       return false;
@@ -341,7 +392,9 @@ tf_status validate_march(const tf_schedule *s, int M, const int *Ap, const int *
   if (s->lds_bytes > kMaxLds || s->march_slots > n_slots || s->lds_bytes != kMarchSlot0 + s->march_slots * kMarchRowBytes)
     return fail(TF_ESCHEDULE, "marching schedule: %d bytes of LDS for %d slots", s->lds_bytes, s->march_slots);
   const size_t n_rows = s->march_row_out.size();
-  if (s->march_row_id.size() != n_rows || s->march_ell_off.size() != n_rows * kMarchW || s->march_ell_src.size() != n_rows * kMarchW ||
+  if (s->march_width < 0 || s->march_width > kMarchWideW) return fail(TF_ESCHEDULE, "marching schedule: rows of %d entries", s->march_width);
+  const int ell_w = march_ell_stride(s->march_width);
+  if (s->march_row_id.size() != n_rows || s->march_ell_off.size() != n_rows * ell_w || s->march_ell_src.size() != n_rows * ell_w ||
       s->march_row_ptr.empty() || s->march_row_ptr.back() != (int)n_rows || s->march_row_ptr.size() != 2 * s->march_load_ptr.size() - 1 ||
       s->march_load_ptr.back() * 2 != (int)s->march_load.size())
     return fail(TF_ESCHEDULE, "marching schedule: tables do not match");
@@ -365,9 +418,9 @@ tf_status validate_march(const tf_schedule *s, int M, const int *Ap, const int *
       if (row < 0 || row >= M) return fail(TF_ESCHEDULE, "run %d: row %d out of range", r, row);
       const int *P = want_t ? Bp : Ap, *I = want_t ? Bi : Ai;
       if (!want_t && out != row) return fail(TF_ESCHEDULE, "run %d: second-op row %d is stored to row %d", r, row, out);
-      if (P[row + 1] - P[row] > kMarchW) return fail(TF_ESCHEDULE, "run %d: row %d has more than %d entries", r, row, kMarchW);
-      for (int u = 0; u < kMarchW; ++u) {
-        const int off = s->march_ell_off[(size_t)q * kMarchW + u], src = s->march_ell_src[(size_t)q * kMarchW + u];
+      if (P[row + 1] - P[row] > ell_w) return fail(TF_ESCHEDULE, "run %d: row %d has more than %d entries", r, row, ell_w);
+      for (int u = 0; u < ell_w; ++u) {
+        const int off = s->march_ell_off[(size_t)q * ell_w + u], src = s->march_ell_src[(size_t)q * ell_w + u];
         const int k = P[row] + u;
         if (k >= P[row + 1]) {
           if (off != kMarchZeroOff || src != -1) return fail(TF_ESCHEDULE, "run %d: row %d has an entry past its end", r, row);
