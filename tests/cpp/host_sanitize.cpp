@@ -64,6 +64,19 @@ int main() {
     bad += run("stencil march", M, p, i, o);
     o.march_tile_x = 5; o.march_tile_y = 3; o.compute_units = 7; bad += run("stencil march 5x3", M, p, i, o);
     o.march_tile_x = o.march_tile_y = 0; o.grid_nx = ny; o.grid_ny = nx; o.grid_nz = nz; bad += run("stencil march, wrong grid", M, p, i, o); }
+  {  // 27-point stencil on a 13 x 11 x 9 grid: marching runs with ELL rows of 32 pairs, the grid found from thirteen distances
+    const int nx = 13, ny = 11, nz = 9, M = nx * ny * nz;
+    p.assign(1, 0); i.clear();
+    for (int z = 0; z < nz; ++z) for (int y = 0; y < ny; ++y) for (int x = 0; x < nx; ++x) {
+      for (int dz = -1; dz <= 1; ++dz) for (int dy = -1; dy <= 1; ++dy) for (int dx = -1; dx <= 1; ++dx) {
+        const int X = x + dx, Y = y + dy, Z = z + dz;
+        if (X >= 0 && X < nx && Y >= 0 && Y < ny && Z >= 0 && Z < nz) i.push_back((Z * ny + Y) * nx + X);
+      }
+      p.push_back((int)i.size());
+    }
+    tf_inspect_opts o{}; o.struct_size = sizeof(o); o.op = TF_OP_SPMM_SPMM; o.N = 128; o.inner_Ap = p.data(); o.inner_Ai = i.data(); o.inner_cols = M; o.march = 1;
+    bad += run("27-point stencil march", M, p, i, o);
+    o.compute_units = 5; bad += run("27-point stencil march, 5 units", M, p, i, o); }
   {  // 5-point stencil on a 300 x 90 grid (runs along the grid's lines) and a tall 7-point grid (more planes
      // than a run's table holds: cut into several runs along z)
     auto stencil = [&](int nx, int ny, int nz) {

@@ -22,10 +22,10 @@ def csr32(m):
 
 
 def random_pattern(wl, rng):
-    """One of: random band, Erdos-Renyi, R-MAT, 2D / 3D stencil, a few hub rows over a sparse background, a band with
+    """One of: random band, Erdos-Renyi, R-MAT, 2D / 3D stencil (5, 7, 19, 27 points), a few hub rows over a sparse background, a band with
     a third of its rows emptied, a band off the diagonal, diagonal blocks.  Values uniform in [-1, 1]."""
     seed = int(rng.integers(1 << 30))
-    kind = str(rng.choice(["band", "band", "er", "rmat", "lap2", "lap3", "hub", "empty", "bandoff", "block"]))
+    kind = str(rng.choice(["band", "band", "er", "rmat", "lap2", "lap3", "box3", "hub", "empty", "bandoff", "block"]))
     if kind == "band":
         bw = int(rng.choice([2, 4, 16, 32, 64, 100]))
         A = wl.banded_random(int(rng.integers(40, 6000)), bw, int(rng.integers(1, min(bw // 2, 24) + 1)), seed=seed)
@@ -38,6 +38,15 @@ def random_pattern(wl, rng):
         A = wl.laplacian_2d(int(rng.integers(4, 70)), int(rng.integers(4, 70)))
     elif kind == "lap3":
         A = wl.laplacian_3d(int(rng.integers(3, 18)))
+    elif kind == "box3":   # 27 points, or 19 without the corners of the cube
+        def line(n, centre=True):
+            e = np.ones(n)
+            return sp.diags([e[:-1], e, e[:-1]], [-1, 0, 1]) if centre else sp.diags([e[:-1], e[:-1]], [-1, 1])
+        nx, ny, nz = (int(v) for v in rng.integers(3, 15, size=3))
+        A = sp.csr_matrix(sp.kron(sp.kron(line(nz), line(ny)), line(nx)))
+        if rng.random() < 0.5:
+            A = A - sp.csr_matrix(sp.kron(sp.kron(line(nz, False), line(ny, False)), line(nx, False)))
+            A.eliminate_zeros()
     elif kind == "hub":
         M = int(rng.integers(200, 4000))
         A = sp.random(M, M, density=4.0 / M, random_state=seed, format="lil")
