@@ -415,7 +415,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=HEADLINE, choices=[1, 2, 3, 4, 5, 6],
+    ap.add_argument("--config", type=int, default=HEADLINE, choices=[1, 2, 3, 4, 5, 6, 7],
                     help="the configuration of the timed line (default: 4, the largest)")
     ap.add_argument("--only", action="store_true", help="skip the per_config table of the other configurations")
     ap.add_argument("--lds", type=int, default=0, help="LDS budget per tile in bytes (0 = library default)")

@@ -42,6 +42,20 @@ def laplacian_3d(n):
     return _csr32(m)
 
 
+def box_stencil_3d(n, corners=True):
+    """The stencil of all neighbours within one step in every direction on an n^3 grid, x fastest: 27 points (19
+    without the cube's corners), every row scaled to sum 1."""
+    e = np.ones(n)
+    t = sp.diags([e[:-1], e, e[:-1]], [-1, 0, 1])
+    m = sp.csr_matrix(sp.kron(sp.kron(t, t), t))
+    if not corners:
+        o = sp.diags([e[:-1], e[:-1]], [-1, 1])
+        m = sp.csr_matrix(m - sp.kron(sp.kron(o, o), o))
+        m.eliminate_zeros()
+    deg = np.asarray(m.sum(axis=1)).ravel()
+    return _csr32(sp.diags(1.0 / deg) @ m)
+
+
 def banded_random(M, bandwidth=32, per_row=16, seed=3):
     """Each row holds `per_row` distinct columns drawn uniformly from
     [i - bandwidth/2, i + bandwidth/2) clipped to [0, M), values uniform[-1, 1]."""
@@ -117,6 +131,8 @@ CONFIG_NAMES = {
     # not one of the reference's configurations: the banded pattern of cfg2 under GeMM-SpMM, the
     # workload on which the fused GeMM-SpMM kernel has rows to fuse at full size
     6: "extra GeMM-SpMM banded bw32 262144 rows, K=N=128",
+    # ... and a stencil with diagonal neighbours: rows of 27 entries, the wide form of the marching runs
+    7: "extra SpMM-SpMM 27-point stencil 128^3, N=64",
 }
 
 
@@ -150,6 +166,11 @@ def make_config(idx, scale=1.0):
         M = max(256, int(262144 * scale))
         A = banded_random(M, 32, 16, seed=3)
         return dict(op="gemm_spmm", A=A, B=uniform((M, 128), 12), C=uniform((128, 128), 13), K=128, N=128, name=CONFIG_NAMES[6])
+    if idx == 7:
+        g = 128 if scale >= 1.0 else max(8, int(round(128 * scale ** (1.0 / 3.0))))
+        A = box_stencil_3d(g)
+        M = A.shape[0]
+        return dict(op="spmm_spmm", A=A, B=A, C=uniform((M, 64), 14), K=0, N=64, name=CONFIG_NAMES[7])
     raise ValueError(f"unknown config {idx}")
 
 
