@@ -442,6 +442,8 @@ def main():
                     help="permute the rows and columns of the (square) matrix at random first")
     ap.add_argument("--rcm", action="store_true",
                     help="reorder the matrix with tf_reorder_rcm / tf_permute_csr before inspecting it (after --scramble)")
+    ap.add_argument("--partition", type=int, default=0,
+                    help="renumber the graph with tf_reorder_partition into this many parts first (hubs in front)")
     ap.add_argument("--unfused", action="store_true",
                     help="GeMM-SpMM as two launches (tf_gemm, tf_spmm) with the intermediate in HBM, for comparison")
     ap.add_argument("--two-layers", default=None, choices=["compose", "fuse"],
@@ -476,7 +478,7 @@ def main():
     if args.calibrate_gather:
         calibrate_gather(tf)
         return
-    custom = bool(args.matrix or args.scramble or args.rcm or args.unfused or args.two_layers)
+    custom = bool(args.matrix or args.scramble or args.rcm or args.partition or args.unfused or args.two_layers)
     if args.matrix:
         Af = tf.read_matrix(args.matrix)
         if Af.shape[0] != Af.shape[1]:
@@ -490,10 +492,10 @@ def main():
     if args.two_layers:
         cfg["name"] += ", two layers with ReLU (tf_gcn_two_layers: " + ("two-layer tiles, hidden layer in LDS)" if args.two_layers == "fuse" else "one executor call per layer)")
     reorder_s = None
-    if args.scramble or args.rcm:  # same product on a renumbered graph: A' = A[p,:][:,p], dense row operands follow
+    if args.scramble or args.rcm or args.partition:  # same product on a renumbered graph: A' = A[p,:][:,p], dense row operands follow
         A0 = cfg["A"]
         if A0.shape[0] != A0.shape[1]:
-            sys.exit("bench.py --scramble/--rcm: the matrix must be square")
+            sys.exit("bench.py --scramble/--rcm/--partition: the matrix must be square")
         same_b = cfg["B"] is A0
         rows_follow = ["B"] if cfg["op"] == "gemm_spmm" else ["C"]
         if args.scramble:
@@ -510,6 +512,14 @@ def main():
             for k in rows_follow:
                 cfg[k] = cfg[k][p]
             cfg["name"] += ", RCM"
+        if args.partition:
+            t0 = time.perf_counter()
+            p, _ = tf.reorder_partition(A0, args.partition)
+            A0 = tf.permute_csr(A0, p)
+            reorder_s = time.perf_counter() - t0
+            for k in rows_follow:
+                cfg[k] = cfg[k][p]
+            cfg["name"] += f", partition ordering ({args.partition} parts, hubs in front)"
         cfg["A"] = A0
         if same_b:
             cfg["B"] = A0

@@ -273,6 +273,11 @@ typedef struct {
      allows (every tile's halo of hidden rows and the halo of those fit LDS: banded or reordered patterns): what
      tf_gcn_two_layers runs when the schedule serves as its second layer's.  0 = build them, -1 = do not. */
   int two_layer_tiles;
+  /* GeMM-SpMM schedules in which nothing fuses (the step is a GEMM of the intermediate rows that are read, then
+     gathers through the schedule's own lists): the intermediate's rows are stored in the order in which they are
+     read most -- the rows of the hot partitions first, then by falling number of reads -- instead of at their own
+     index.  Invisible to the caller (results identical); 0 = do so, -1 = rows at their own index. */
+  int place_intermediate;
 } tf_inspect_opts;
 
 typedef struct tf_schedule tf_schedule;
@@ -325,6 +330,7 @@ typedef struct {
   int n_computed_rows;   /* intermediate rows the executor computes per call: the producer rows of the tiles it
                             launches (halo rows included) plus, for tiles that fuse nothing, only the rows some
                             remainder row reads -- on a graph with isolated nodes fewer than inter_rows       */
+  int intermediate_placed; /* 1 when the intermediate's rows are stored in the order they are read most (place_intermediate) */
 } tf_schedule_info;
 
 /* tf_schedule_info.march_declined */

@@ -442,6 +442,30 @@ def test_streaming_gathers_of_short_rows_change_no_bit(gpu, tf, orc):
     assert orc.rel_err(outs[0], want) <= TOL
 
 
+def test_placed_intermediate_changes_no_bit(gpu, tf, orc):
+    """place_intermediate only changes where the GEMM stores a row of the intermediate and what the lists call it: the
+    same launches in the same order give the same bits with it and without, on a power-law graph (long rows by column
+    partition, with and without the second stream) and on an Erdos-Renyi graph, and both match the oracle."""
+    say("intermediate rows placed by reads")
+    for cfg, kw in ((tf.workloads.make_config(4, 2.0 ** -5), dict(long_row_partition=1)), (tf.workloads.make_config(3, 0.05), dict())):
+        A, B, W = cfg["A"], cfg["B"], cfg["C"]
+        M, N, K = A.shape[0], cfg["N"], cfg["K"]
+        Ah = tf.CsrMatrix.from_scipy(A)
+        Bd, Wd = tf.DenseMatrix.from_numpy(B), tf.DenseMatrix.from_numpy(W)
+        outs = []
+        for place, second in ((0, False), (-1, False), (0, True)):
+            S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=N, K=K, place_intermediate=place, **kw)
+            S.validate()
+            assert S.info()["intermediate_placed"] == (1 if place == 0 else 0)
+            D = tf.DenseMatrix(M, N); D.fill(float("nan"))
+            tf.gemm_spmm(Ah, Bd, Wd, D, S, second_stream=second)
+            tf.gemm_spmm(Ah, Bd, Wd, D, S, second_stream=second)   # (a second call: regrouped values are reused)
+            outs.append(D.to_numpy())
+        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+        want, _ = orc.gemm_spmm(A, B, W, orc.unfused_schedule(M), nthreads=8)
+        assert orc.rel_err(outs[0], want) <= TOL
+
+
 def test_two_host_threads_with_their_own_schedules(gpu, tf, orc):
     """Two host threads, each with its own operands, schedules and stream, call the executors at the same time (ctypes
     releases the interpreter lock during a call): every result equals the oracle's, as if each had run alone.  What the

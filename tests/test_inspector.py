@@ -542,6 +542,42 @@ def test_short_rows_mark_their_cold_gathers_on_power_law_graphs(tf):
     assert S.info()["short_row_hot_rows"] == 0
 
 
+def test_intermediate_rows_are_placed_where_nothing_fuses(tf):
+    """place_intermediate: a GeMM-SpMM schedule in which nothing fuses and every gather goes through the schedule's own
+    lists (a power-law graph, an Erdos-Renyi graph) stores the intermediate's rows in the order they are read most;
+    the validator checks the lists against the places.  Schedules with fused tiles (a band), SpMM-SpMM schedules and
+    -1 leave the rows at their own index."""
+    cfg = tf.workloads.make_config(4, 2.0 ** -5)
+    Ah = tf.CsrMatrix.from_scipy(cfg["A"])
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1)
+    S.validate()
+    assert S.info()["intermediate_placed"] == 1 and S.info()["n_fused_rows"] == 0
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1, place_intermediate=-1)
+    S.validate()
+    assert S.info()["intermediate_placed"] == 0
+    # long rows in chunks (no column partition at this size) read A's own columns: nothing placed
+    S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128)
+    S.validate()
+    assert S.info()["n_long_chunks"] > 0 and S.info()["intermediate_placed"] == 0
+    er = tf.workloads.make_config(3, 0.05)
+    Eh = tf.CsrMatrix.from_scipy(er["A"])
+    S = tf.inspector(Eh, 1, op=tf.OP_GEMM_SPMM, N=128, K=256)
+    S.validate()
+    assert S.info()["intermediate_placed"] == 1
+    # the rows of the list read A in place (reorder_adjacency = -1): nothing to translate, nothing placed
+    S = tf.inspector(Eh, 1, op=tf.OP_GEMM_SPMM, N=128, K=256, reorder_adjacency=-1)
+    S.validate()
+    assert S.info()["intermediate_placed"] == 0
+    band = tf.workloads.banded_random(30000, 32, 12, seed=3)
+    Bh = tf.CsrMatrix.from_scipy(band)
+    S = tf.inspector(Bh, 1, op=tf.OP_GEMM_SPMM, N=128, K=128)
+    S.validate()
+    assert S.info()["n_fused_rows"] > 0 and S.info()["intermediate_placed"] == 0
+    S = tf.inspector(Ah, 1, op=tf.OP_SPMM_SPMM, N=128)
+    S.validate()
+    assert S.info()["intermediate_placed"] == 0
+
+
 # ---- two-layer tiles -------------------------------------------------------------------------------------------
 
 def _check_two_layer_tiles(A, rng6, H, N):

@@ -42,7 +42,7 @@ class InspectOpts(C.Structure):
                 ("inner_cols", C.c_int), ("strip_cols", C.c_int), ("xcd_chunk_rows", C.c_int), ("wide_strips", C.c_int), ("long_row_partition", C.c_int),
                 ("march", C.c_int), ("grid_nx", C.c_int), ("grid_ny", C.c_int), ("grid_nz", C.c_int),
                 ("march_tile_x", C.c_int), ("march_tile_y", C.c_int), ("reorder_adjacency", C.c_int), ("hot_partition_bytes", C.c_int),
-                ("short_row_hot_bytes", C.c_int), ("two_layer_tiles", C.c_int)]
+                ("short_row_hot_bytes", C.c_int), ("two_layer_tiles", C.c_int), ("place_intermediate", C.c_int)]
 
 
 class ScheduleInfo(C.Structure):
@@ -55,7 +55,7 @@ class ScheduleInfo(C.Structure):
                 ("fused_nnz", C.c_longlong), ("workspace_bytes", C.c_longlong),
                 ("marched", C.c_int), ("march_tile_x", C.c_int), ("march_tile_y", C.c_int), ("march_slots", C.c_int),
                 ("march_declined", C.c_int), ("register_weights", C.c_int), ("n_zero_rows", C.c_int), ("two_layer_tiles", C.c_int),
-                ("short_row_hot_rows", C.c_int), ("n_computed_rows", C.c_int)]
+                ("short_row_hot_rows", C.c_int), ("n_computed_rows", C.c_int), ("intermediate_placed", C.c_int)]
 
 
 class ScheduleView(C.Structure):
@@ -363,7 +363,7 @@ class FusedSchedule:
 
 def inspector(A, NumThreads=1, *, op, N, K=0, lds_budget_bytes=0, tile_rows=0, max_redundancy=0.0,
               long_row_nnz=0, compute_units=0, inner=None, strip_cols=0, xcd_chunk_rows=0, wide_strips=0, long_row_partition=0,
-              march=0, grid=None, march_tile=None, reorder_adjacency=0, hot_partition_bytes=0, short_row_hot_bytes=0, two_layer_tiles=0):
+              march=0, grid=None, march_tile=None, reorder_adjacency=0, hot_partition_bytes=0, short_row_hot_bytes=0, two_layer_tiles=0, place_intermediate=0):
     """swiftware::fusion::inspector(A, NumThreads) (README.md:25).  NumThreads is accepted
     for signature parity and unused: the schedule is sized by the GPU, not by a CPU
     thread count.  The extra keywords are the parameters the reference passes to its
@@ -374,7 +374,7 @@ def inspector(A, NumThreads=1, *, op, N, K=0, lds_budget_bytes=0, tile_rows=0, m
     o = InspectOpts(C.sizeof(InspectOpts), op, N, K, lds_budget_bytes, tile_rows, max_redundancy, long_row_nnz, compute_units,
                     inner._pp if inner is not None else None, inner._pi if inner is not None else None,
                     inner.N if inner is not None else 0, strip_cols, xcd_chunk_rows, wide_strips, long_row_partition,
-                    march, *(grid or (0, 0, 0)), *(march_tile or (0, 0)), reorder_adjacency, hot_partition_bytes, short_row_hot_bytes, two_layer_tiles)
+                    march, *(grid or (0, 0, 0)), *(march_tile or (0, 0)), reorder_adjacency, hot_partition_bytes, short_row_hot_bytes, two_layer_tiles, place_intermediate)
     h = _VP()
     _check(lib().tf_inspect(A.M, A.N, A._pp, A._pi, C.byref(o), C.byref(h)))
     return FusedSchedule(h, A, inner)

@@ -104,7 +104,7 @@ hipError_t launch_fused_gemm_spmm(const TileDesc *, int, const int *, const floa
 hipError_t launch_fused_gemm_spmm_stream(const TileDesc *, int, const int *, const int *, const int *,
                                          const float *, const float *, int, int, int, const int *,
                                          const float *, float *, float *, int, int, hipStream_t, int relu_in = 0);
-hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t);
+hipError_t launch_gemm(const float *, const float *, float *, const int *, int, int, int, int, hipStream_t, int y_by_position = 0);
 hipError_t launch_fill(float *, size_t, float, hipStream_t);
 hipError_t launch_pad(const float *, int, int, float *, int, int, hipStream_t);
 hipError_t launch_copy_cols(const float *, int, int, int, int, float *, int, int, int, int, int, hipStream_t);
@@ -777,10 +777,11 @@ static tf_status gemm_spmm_pass(const tf_csr *A, const float *Bd, const float *C
   const bool overlap = d->side && s->plain_hot > 0 && (flags & TF_SECOND_STREAM);
   if (!s->plain_rows.empty()) {  // intermediate rows of tiles that fuse nothing
     const int n_plain = (int)s->plain_rows.size();
-    const bool all = n_plain == s->M && s->plain_hot == 0;
+    const int placed = s->t_pos.empty() ? 0 : 1;  // the intermediate's rows stored in the order of the list
+    const bool all = n_plain == s->M && s->plain_hot == 0 && !placed;
     if (overlap) {
       TF_PHASE(s, "gemm_rows_kernel (hot rows)", st,
-               tf::launch_gemm(Bd, Cd, d->inter, d->plain_rows, s->plain_hot, s->opts.K, s->opts.N, s->opts.compute_units, st));
+               tf::launch_gemm(Bd, Cd, d->inter, d->plain_rows, s->plain_hot, s->opts.K, s->opts.N, s->opts.compute_units, st, placed));
       // the regrouped values (of the hot and of the cold segments) before the fork: the cold segments run on
       // this stream and are not ordered after anything the side stream does until the join
       if (tf_status rc2 = tf::ensure_segment_values(A, s, st)) return rc2;
@@ -790,11 +791,11 @@ static tf_status gemm_spmm_pass(const tf_csr *A, const float *Bd, const float *C
       TF_HIP(hipEventRecord(d->join, d->side));
       if (n_plain > s->plain_hot)
         TF_PHASE(s, "gemm_rows_kernel (other rows)", st,
-                 tf::launch_gemm(Bd, Cd, d->inter, d->plain_rows + s->plain_hot, n_plain - s->plain_hot, s->opts.K, s->opts.N,
-                                 s->opts.compute_units, st));
+                 tf::launch_gemm(Bd, Cd, d->inter + (placed ? (size_t)s->plain_hot * s->opts.N : 0), d->plain_rows + s->plain_hot,
+                                 n_plain - s->plain_hot, s->opts.K, s->opts.N, s->opts.compute_units, st, placed));
     } else {
       TF_PHASE(s, "gemm_rows_kernel", st,
-               tf::launch_gemm(Bd, Cd, d->inter, all ? nullptr : d->plain_rows, n_plain, s->opts.K, s->opts.N, s->opts.compute_units, st));
+               tf::launch_gemm(Bd, Cd, d->inter, all ? nullptr : d->plain_rows, n_plain, s->opts.K, s->opts.N, s->opts.compute_units, st, placed));
     }
   }
   return tf::run_remainder(A, D, s, acc, overlap && !s->plain_rows.empty(), st);

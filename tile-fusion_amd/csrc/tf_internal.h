@@ -140,6 +140,10 @@ struct tf_schedule {
   // go to their slots.  Every entry of an ELL row names the LDS byte offset of the row it reads; the
   // inspector assigns the slots so that a row stays until its last reader has run.
   bool march = false;
+  // GeMM-SpMM schedules in which nothing fuses and every gather goes through the schedule's own copies of the columns:
+  // t_pos[c] = where row c of the intermediate is stored (its place in plain_rows: the rows of the hot partitions
+  // first, the others by falling number of reads), -1 for rows nobody reads.  Empty: rows at their own index.
+  std::vector<int> t_pos;
   int march_declined = TF_MARCH_NOT_TRIED;  // why there are no marching runs (TF_MARCH_*), TF_MARCH_BUILT when there are
   int march_grid[3] = {0, 0, 0};     // the grid the runs were cut from (x fastest)
   int march_tile[2] = {0, 0};        // grid points per run and plane: x, y

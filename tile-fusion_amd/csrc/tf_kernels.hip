@@ -822,7 +822,9 @@ constexpr int kGemmSeg = 16;  // row blocks whose row numbers a wavefront keeps 
 // issues in order, so address arithmetic, a wait for a row number or a branch between two MFMAs leaves the
 // pipe without work from this wavefront (39,000 -> 33,500 cycles per block and wavefront for K = 128, of
 // which the block's 256 MFMAs of the two wavefronts of a SIMD take 32,800).
-template <int NB, bool LIST, int G4C>
+// YPOS (row lists only): the result of list position q goes to row q of Y instead of row rows[q] -- the rows of the
+// result stored side by side in the order of the list.
+template <int NB, bool LIST, int G4C, bool YPOS = false>
 __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__restrict__ X,
                                                                const float *__restrict__ W,
                                                                float *__restrict__ Y,
@@ -876,7 +878,7 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int x = rb * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-        if (x < n_rows) Y[(size_t)(LIST ? rows[x] : x) * N + NB * j + nb] = acc1[r];
+        if (x < n_rows) Y[(size_t)(LIST && !YPOS ? rows[x] : x) * N + NB * j + nb] = acc1[r];
       }
     }
   }
@@ -888,6 +890,8 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
     const int total_groups = (rb_end - rb0) * G4;
     // row (of X and Y) behind position x of this segment
     auto row_at = [&](int x) { return LIST ? ridx[x] : min(rb0 * 32 + x, n_rows - 1); };
+    // ... and the row of Y it is stored to
+    auto yrow_at = [&](int x) { return LIST && !YPOS ? ridx[x] : min(rb0 * 32 + x, n_rows - 1); };
     if constexpr (G4C > 0) {
       static_assert(G4C >= 4 && G4C % 4 == 0, "four operand sets in turn, a block starts with the first");
       const int nblk = rb_end - rb0;
@@ -906,7 +910,7 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
         wvec<NB> out;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) out.v[nb] = acc[nb][r];
-        *reinterpret_cast<wvec<NB> *>(Y + (size_t)row_at(b * 32 + 8 * (r / 4) + 4 * h + (r % 4)) * N + NB * j) = out;
+        *reinterpret_cast<wvec<NB> *>(Y + (size_t)yrow_at(b * 32 + 8 * (r / 4) + 4 * h + (r % 4)) * N + NB * j) = out;
       };
       for (int b = 0; b < nblk; ++b) {
         const float *pn = operand_row(b + 1);
@@ -998,7 +1002,7 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_rows_kernel(const float *__re
             wvec<NB> out;
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) out.v[nb] = acc[nb][r];
-            *reinterpret_cast<wvec<NB> *>(Y + (size_t)row_at(x) * N + NB * j) = out;
+            *reinterpret_cast<wvec<NB> *>(Y + (size_t)yrow_at(x) * N + NB * j) = out;
           }
         }
       }
@@ -2126,8 +2130,9 @@ hipError_t launch_fused_gemm_spmm_stream(const TileDesc *tiles, int n_tiles, con
 }
 
 hipError_t launch_gemm(const float *X, const float *W, float *Y, const int *rows, int n_rows, int K,
-                       int N, int compute_units, hipStream_t st) {
+                       int N, int compute_units, hipStream_t st, int y_by_position) {
   if (n_rows <= 0) return hipSuccess;
+  if (y_by_position && !rows) return hipErrorInvalidValue;
   const int NB = N / 32;
   hipError_t err = hipSuccess;
   const int w_bytes = K * N * 4;
@@ -2137,23 +2142,23 @@ hipError_t launch_gemm(const float *X, const float *W, float *Y, const int *rows
     const int nrb = (n_rows + 31) / 32;
     const int grid = std::max(1, std::min(compute_units * per_cu, (nrb + kGemmBlock / 64 - 1) / (kGemmBlock / 64)));
     const int lds = w_bytes + (rows ? (kGemmBlock / 64) * kGemmSeg * 32 * 4 : 0);  // + the wavefronts' row numbers
-#define CALL3(NB_, LIST_, G4C_)                                                                     \
-  err = allow_lds(gemm_rows_kernel<NB_, LIST_, G4C_>, lds);                                         \
+#define CALL3(NB_, LIST_, G4C_, YPOS_)                                                              \
+  err = allow_lds(gemm_rows_kernel<NB_, LIST_, G4C_, YPOS_>, lds);                                  \
   if (err == hipSuccess)                                                                            \
-    hipLaunchKernelGGL((gemm_rows_kernel<NB_, LIST_, G4C_>), dim3(grid), dim3(kGemmBlock), lds, st, X, W, Y, \
+    hipLaunchKernelGGL((gemm_rows_kernel<NB_, LIST_, G4C_, YPOS_>), dim3(grid), dim3(kGemmBlock), lds, st, X, W, Y, \
                        rows, n_rows, K)
   // K = 128 and 256 with up to 128 columns have kernels of their own (K built in)
-#define CALL2(NB_, LIST_)                        \
-  do {                                           \
-    if constexpr (NB_ <= 4) {                    \
-      if (K == 128) { CALL3(NB_, LIST_, 4); }    \
-      else if (K == 256) { CALL3(NB_, LIST_, 8); } \
-      else { CALL3(NB_, LIST_, 0); }             \
-    } else {                                     \
-      CALL3(NB_, LIST_, 0);                      \
-    }                                            \
+#define CALL2(NB_, LIST_, YPOS_)                        \
+  do {                                                  \
+    if constexpr (NB_ <= 4) {                           \
+      if (K == 128) { CALL3(NB_, LIST_, 4, YPOS_); }    \
+      else if (K == 256) { CALL3(NB_, LIST_, 8, YPOS_); } \
+      else { CALL3(NB_, LIST_, 0, YPOS_); }             \
+    } else {                                            \
+      CALL3(NB_, LIST_, 0, YPOS_);                      \
+    }                                                   \
   } while (0)
-#define CALL(NB_) do { if (rows) { CALL2(NB_, true); } else { CALL2(NB_, false); } } while (0)
+#define CALL(NB_) do { if (rows && y_by_position) { CALL2(NB_, true, true); } else if (rows) { CALL2(NB_, true, false); } else { CALL2(NB_, false, false); } } while (0)
     TF_DISPATCH_NB(NB, CALL);
 #undef CALL
 #undef CALL2
