@@ -200,7 +200,8 @@ typedef struct {
                             Default 3.0 for SpMM-SpMM, 1.5 for GeMM-SpMM.                    */
   int long_row_nnz;      /* remainder rows with more stored entries than this are worked on by a
                             whole workgroup each (in chunks of max(this, 1024) entries, partial
-                            sums added in a fixed order); default 32, max 2048                */
+                            sums added in a fixed order); default 32 -- 64 where the long rows are
+                            regrouped by column partition (long_row_partition) --, max 2048    */
   int compute_units;     /* sizing hint; default: the current device, or 256 with no device  */
   /* SpMM-SpMM only, optional: sparsity pattern of the inner matrix B (M x inner_cols, host
      arrays).  In every run of the reference B is A (fusion/example/SpMM_SpMM_Demo_Utils.h:
@@ -266,7 +267,7 @@ typedef struct {
   /* Short remainder rows kept in list order (reorder_adjacency) on a graph with hub rows: bytes of most-read
      intermediate rows that those rows' gathers may keep in an L2; gathers of all other rows are marked in the
      schedule and fetched with streaming loads, so that rows read once do not push out rows with readers.
-     0 = 8 MB when the long rows are column-partitioned (long_row_partition: a power-law graph), else off;
+     0 = 32 MB when the long rows are column-partitioned (long_row_partition: a power-law graph), else off;
      -1 = off; n > 0 = n bytes.  Only when N is a multiple of 4, and only if the set takes a quarter of the reads. */
   int short_row_hot_bytes;
   /* GeMM-SpMM schedules of a square matrix with K and N of 32, 64 or 128 also get two-layer tiles when the pattern

@@ -261,9 +261,13 @@ def test_long_rows_by_column_partition(tf):
     S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1)
     S.validate()
     info = S.info()
-    assert info["n_long_rows"] == base.info()["n_long_rows"]
     rl = np.diff(A.indptr)
-    long_nnz = int(rl[rl > 32].sum())
+    # (left to the library, the threshold is 32 entries for rows in chunks and 64 for rows regrouped by partition)
+    assert base.info()["n_long_rows"] == int((rl > 32).sum()) and info["n_long_rows"] == int((rl > 64).sum())
+    S32 = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1, long_row_nnz=32)
+    S32.validate()
+    assert S32.info()["n_long_rows"] == base.info()["n_long_rows"]
+    long_nnz = int(rl[rl > 64].sum())
     assert 0 < info["long_row_hot_cols"] <= 8 * (12 << 20) // (128 * 4)
     # at least one segment per 64 entries, and the eight hot lists are padded to whole workgroups
     assert info["n_long_chunks"] >= long_nnz // 64 and info["n_long_chunks"] % 1 == 0
@@ -530,7 +534,7 @@ def test_short_rows_mark_their_cold_gathers_on_power_law_graphs(tf):
     S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1)
     S.validate()
     info = S.info()
-    assert info["long_row_hot_cols"] > 0 and 0 < info["short_row_hot_rows"] <= (8 << 20) // 512
+    assert info["long_row_hot_cols"] > 0 and 0 < info["short_row_hot_rows"] <= (32 << 20) // 512
     S = tf.inspector(Ah, 1, op=tf.OP_GEMM_SPMM, N=128, K=128, long_row_partition=1, short_row_hot_bytes=1 << 20)
     S.validate()
     assert 0 < S.info()["short_row_hot_rows"] <= 2048

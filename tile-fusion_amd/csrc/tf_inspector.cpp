@@ -527,6 +527,30 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
       // (three times an L2's 4 MB measured best on the R-MAT graph: 2.68 ms per step with 4 MB, 2.54 with 12 or
       // 16 MB, 2.60 with 32 MB -- the reads inside a partition are skewed too, and its hottest rows are what stays)
       const int part_rows = std::max(64, (o.hot_partition_bytes > 0 ? o.hot_partition_bytes : (12 << 20)) / (o.N * 4));
+      // Regrouped rows pay for their partial sums (a row of 4N bytes written and read again per group): with the
+      // threshold left to the library, rows of up to 64 entries stay whole rows of the row kernel (measured on the
+      // 2^21-node R-MAT step, thresholds 32 / 40 / 48 / 64 / 96: 2.04 / 1.97 / 1.97 / 1.96 / 1.97 ms).
+      if (want && user->long_row_nnz <= 0 && S->long_chunks.size() < (size_t)INT_MAX) {
+        constexpr int kPartitionedFrom = 64;
+        std::vector<tf::LongRow> keep_rows;
+        std::vector<tf::LongChunk> keep_chunks;
+        for (const auto &lr : S->long_rows) {
+          if (Ap[lr.row + 1] - Ap[lr.row] <= kPartitionedFrom) { S->rem_rows.push_back(lr.row); continue; }
+          tf::LongRow nr{lr.row, (int)keep_chunks.size(), lr.count, 0};
+          for (int c = 0; c < lr.count; ++c) {
+            tf::LongChunk ch = S->long_chunks[lr.first + c];
+            ch.slot = (int)keep_chunks.size();
+            keep_chunks.push_back(ch);
+          }
+          keep_rows.push_back(nr);
+        }
+        S->long_rows.swap(keep_rows);
+        S->long_chunks.swap(keep_chunks);
+        std::sort(S->rem_rows.begin(), S->rem_rows.end());
+        S->opts.long_row_nnz = o.long_row_nnz = kPartitionedFrom;
+        long_nnz = 0;
+        for (const auto &lr : S->long_rows) long_nnz += Ap[lr.row + 1] - Ap[lr.row];
+      }
       if (want && !S->long_rows.empty() && long_nnz < INT_MAX) {
         constexpr int kParts = 8, kSegMax = 64, kPad = 256, kMinGroup = 4;
         std::vector<int> reads(M, 0);
@@ -673,10 +697,11 @@ extern "C" tf_status tf_inspect(int L, int M, const int *Ap, const int *Ai,
         // take half of their reads on the 2^21-node R-MAT graph) next to a stream of rows read once; left
         // alone, that stream leaves an L2 hit rate under a quarter.  Which XCD a row runs on cannot help here as it
         // does for the long rows' segments: a short row's few columns are spread over all partitions
-        // (measured on that step: the rows' launch 0.495 -> 0.45 ms with 8 MB of unmarked rows; 4 MB 0.52, 16 MB 0.47).
+        // (measured on that step: the rows' launch 0.495 -> 0.45 ms with 8 MB of unmarked rows; 4 MB 0.52, 16 MB 0.47 -- and, once the
+        // intermediate's rows lie in the order of their reads, 8 / 16 / 32 / 64 MB: 0.419 / 0.393 / 0.388 / 0.386 ms).
         {
           const int want = o.short_row_hot_bytes;
-          const long long bytes = want > 0 ? want : (want == 0 && S->long_part ? (8 << 20) : 0);
+          const long long bytes = want > 0 ? want : (want == 0 && S->long_part ? (32 << 20) : 0);
           const size_t keep_n = (size_t)(bytes / ((long long)o.N * 4));
           if (keep_n > 0 && o.N % 4 == 0) {
             std::vector<int> reads(M, 0), order;
